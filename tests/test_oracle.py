@@ -1,0 +1,382 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+  * storage conversions            vs torch's own casts
+  * prefill arithmetic             vs torch's conv1d (the reference's oracle,
+                                   causal-conv1d-mps/test.py:83-107) on the
+                                   reference's grid (test.py:110-116, seed 42)
+  * indices / history / state      vs a brute-force loop on tiny shapes
+  * invariants                     streaming, chunking, state-length
+                                   independence, linearity, causality,
+                                   permutation equivariance, mask special cases
+  * eager module restatement       vs golden vectors produced by the real
+                                   CanonLayer (tests/golden/)
+"""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import canon_oracle as co
+from oracle.canon_eager import EagerCanon
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    return t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+def ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in representable values of the (16-bit) storage type."""
+    def key(t):
+        i = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+        return torch.where(i >= 0x8000, 0x8000 - i, i)
+    return (key(a) - key(b)).abs()
+
+
+# --------------------------------------------------------------------------
+# conversions
+# --------------------------------------------------------------------------
+def test_conversions_match_torch():
+    L = co.lib()
+    g = torch.Generator().manual_seed(0)
+    vals = torch.cat([
+        torch.randn(4000, generator=g),
+        torch.randn(2000, generator=g) * 1e-6,
+        torch.randn(2000, generator=g) * 6e4,
+        torch.randn(500, generator=g) * 1e-41,       # fp32 subnormals
+        torch.tensor([0.0, -0.0, 1.0, -1.0, 65504.0, 65519.9, 65520.0, 1e9, -1e9,
+                      float("inf"), float("-inf"), 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                      2.0 ** -14, 2.0 ** -14 * 0.9999, 3.3895314e38, 1.0 + 2.0 ** -8,
+                      1.0 + 2.0 ** -8 + 2.0 ** -20, 1.0 + 3 * 2.0 ** -8]),
+    ])
+    want_bf = vals.bfloat16().view(torch.int16).to(torch.int32) & 0xFFFF
+    want_h = vals.half().view(torch.int16).to(torch.int32) & 0xFFFF
+    for v, wb, wh in zip(vals.tolist(), want_bf.tolist(), want_h.tolist()):
+        assert L.canon_oracle_float_to_bf16(v) == wb, v
+        assert L.canon_oracle_float_to_f16(v) == wh, v
+    assert L.canon_oracle_float_to_bf16(float("nan")) & 0x7FC0 == 0x7FC0
+    # every 16-bit pattern back to float
+    allbits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    bf = allbits.view(torch.bfloat16).float()
+    hf = allbits.view(torch.float16).float()
+    for i in range(0, 65536, 7):
+        b = int(allbits[i]) & 0xFFFF
+        x, y = L.canon_oracle_bf16_to_float(b), float(bf[i])
+        assert x == y or (x != x and y != y)
+        x, y = L.canon_oracle_f16_to_float(b), float(hf[i])
+        assert x == y or (x != x and y != y)
+
+
+# --------------------------------------------------------------------------
+# arithmetic vs torch conv1d on the reference's grid
+# --------------------------------------------------------------------------
+def torch_reference(x, weight, bias, silu):
+    """fp32 restatement of causal-conv1d-mps/test.py:83-107."""
+    itype = x.dtype
+    xq = x.float()
+    wq = weight.to(itype).float()
+    bq = bias.to(itype).float() if bias is not None else None
+    W = weight.shape[1]
+    y = F.conv1d(F.pad(xq, (W - 1, 0)), wq.unsqueeze(1), bias=bq, groups=x.shape[1])
+    return F.silu(y) if silu else y
+
+
+@pytest.mark.parametrize("itype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("has_bias", [False, True])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_fwd_matches_torch_conv1d_on_reference_grid(dim, has_bias, silu, itype):
+    for seqlen in [1, 2, 8, 16, 32, 64, 128, 256]:
+        torch.manual_seed(42)
+        x = torch.randn(2, dim, seqlen).to(itype)
+        w = torch.randn(dim, 4)
+        b = torch.randn(dim) if has_bias else None
+        got = co.conv1d_fwd(x, w, b, activation="silu" if silu else None)
+        want32 = torch_reference(x, w, b, silu)
+        if itype == torch.float32:
+            if not silu:
+                # torch evaluates the depthwise conv as the same fma chain
+                scale = want32.abs().clamp_min(1.0)
+                assert ((got - want32).abs() / scale).max().item() <= 1e-6
+                assert (got != want32).float().mean().item() <= 0.01
+            else:
+                torch.testing.assert_close(got, want32, rtol=1e-6, atol=1e-6)
+        else:
+            want = want32.to(itype)
+            d = ulp_diff(got, want)
+            assert d.max().item() <= 1, (seqlen, d.max().item())
+            assert (d > 0).float().mean().item() <= 0.002
+
+
+# --------------------------------------------------------------------------
+# brute force on tiny shapes
+# --------------------------------------------------------------------------
+def brute_fwd(x, w, bias, mask, init, S_out, silu, res_mode):
+    """float64-free, index-by-index restatement (fp32 only, python loops)."""
+    B, C, L = x.shape
+    W = w.shape[1]
+    out = np.zeros((B, C, L), np.float32)
+    fs = np.zeros((B, C, S_out), np.float32) if S_out else None
+    for b in range(B):
+        for c in range(C):
+            xm = [np.float32(x[b, c, t] * (mask[b, t] if mask is not None else np.float32(1)))
+                  for t in range(L)]
+            hist = [np.float32(0)] * (W - 1) if init is None else list(init[b, c, init.shape[2] - (W - 1):]) if W > 1 else []
+            seq = hist + xm     # seq[t + W - 1] == xm[t]
+            for t in range(L):
+                acc = np.float64(bias[c]) if bias is not None else np.float64(0)
+                acc = np.float32(acc)
+                for k in range(W):
+                    # fma: exact product in float64, one rounding of the sum
+                    acc = np.float32(np.float64(w[c, k]) * np.float64(seq[t + k]) + np.float64(acc))
+                if silu:
+                    acc = np.float32(acc / np.float32(np.float32(1) + np.exp(-acc, dtype=np.float32)))
+                if res_mode == 1:
+                    acc = np.float32(acc + xm[t])
+                elif res_mode == 2:
+                    acc = np.float32(acc + x[b, c, t])
+                out[b, c, t] = acc
+            if S_out:
+                full = ([np.float32(0)] * S_out + (list(init[b, c]) if init is not None else []) + xm)
+                fs[b, c] = full[-S_out:]
+    return out, fs
+
+
+@pytest.mark.parametrize("W", [2, 3, 4])
+@pytest.mark.parametrize("L", [1, 2, 3, 4, 5, 9])
+def test_fwd_matches_brute_force(W, L):
+    rng = np.random.default_rng(100 * W + L)
+    B, C = 2, 3
+    for has_bias, has_mask, has_init, silu, res_mode in itertools.product(
+            [False, True], [False, True], [False, True], [False, True], [0, 1, 2]):
+        x = rng.standard_normal((B, C, L)).astype(np.float32)
+        w = rng.standard_normal((C, W)).astype(np.float32)
+        bias = rng.standard_normal(C).astype(np.float32) if has_bias else None
+        mask = (rng.random((B, L)) > 0.4).astype(np.float32) if has_mask else None
+        S_in = int(rng.integers(W - 1, 6)) if W > 1 else 2
+        init = rng.standard_normal((B, C, S_in)).astype(np.float32) if has_init else None
+        S_out = int(rng.integers(1, 9))
+        want, want_fs = brute_fwd(x, w, bias, mask, init, S_out, silu, res_mode)
+        t = torch.from_numpy
+        got, got_fs = co.conv1d_fwd(
+            t(x), t(w), None if bias is None else t(bias),
+            mask=None if mask is None else t(mask),
+            initial_state=None if init is None else t(init),
+            final_state_len=S_out, activation="silu" if silu else None, residual=res_mode)
+        if silu:
+            np.testing.assert_allclose(got.numpy(), want, rtol=2e-6, atol=1e-6)
+        else:
+            np.testing.assert_array_equal(got.numpy(), want)
+        np.testing.assert_array_equal(got_fs.numpy(), want_fs)
+
+
+def test_update_matches_brute_force():
+    rng = np.random.default_rng(7)
+    B, C = 3, 5
+    for W, S, has_bias, silu, res in itertools.product([2, 3, 4], [3, 4, 8], [False, True],
+                                                       [False, True], [False, True]):
+        if S < W - 1:
+            continue
+        x = rng.standard_normal((B, C)).astype(np.float32)
+        st = rng.standard_normal((B, C, S)).astype(np.float32)
+        w = rng.standard_normal((C, W)).astype(np.float32)
+        bias = rng.standard_normal(C).astype(np.float32) if has_bias else None
+        want = np.zeros((B, C), np.float32)
+        for b in range(B):
+            for c in range(C):
+                seq = list(st[b, c, S - (W - 1):]) + [x[b, c]]
+                acc = np.float32(bias[c]) if has_bias else np.float32(0)
+                for k in range(W):
+                    acc = np.float32(np.float64(w[c, k]) * np.float64(seq[k]) + np.float64(acc))
+                if silu:
+                    acc = np.float32(acc / np.float32(np.float32(1) + np.exp(-acc, dtype=np.float32)))
+                if res:
+                    acc = np.float32(acc + x[b, c])
+                want[b, c] = acc
+        want_state = np.concatenate([st[:, :, 1:], x[:, :, None]], axis=2)
+        t = torch.from_numpy
+        st_t = t(st.copy())
+        got = co.conv1d_update(t(x), st_t, t(w), None if bias is None else t(bias),
+                               activation="silu" if silu else None, residual=res)
+        if silu:
+            np.testing.assert_allclose(got.numpy(), want, rtol=2e-6, atol=1e-6)
+        else:
+            np.testing.assert_array_equal(got.numpy(), want)
+        np.testing.assert_array_equal(st_t.numpy(), want_state)
+
+
+# --------------------------------------------------------------------------
+# invariants
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("S", [3, 4, 8])
+def test_streaming_equals_prefill(dtype, S):
+    torch.manual_seed(S)
+    B, C, L = 2, 24, 19
+    x = torch.randn(B, C, L).to(dtype)
+    w = (torch.randn(C, 4) * 0.3).to(dtype)
+    b = (torch.randn(C) * 0.1).to(dtype)
+    for act in (None, "silu"):
+        full, fs = co.conv1d_fwd(x, w, b, final_state_len=S, activation=act)
+        state = torch.zeros(B, C, S, dtype=dtype)
+        cols = [co.conv1d_update(x[:, :, t].contiguous(), state, w, b, activation=act)
+                for t in range(L)]
+        assert torch.equal(bits(torch.stack(cols, dim=-1)), bits(full))
+        assert torch.equal(bits(state), bits(fs))
+        assert torch.equal(bits(fs), bits(x[:, :, -S:]))
+
+
+def test_chunked_prefill_equals_one_shot():
+    torch.manual_seed(3)
+    B, C, L = 2, 10, 23
+    x = torch.randn(B, C, L)
+    w = torch.randn(C, 4)
+    mask = (torch.rand(B, L) > 0.3).float()
+    full, fs = co.conv1d_fwd(x, w, None, mask=mask, final_state_len=5, residual=1)
+    for cut in (1, 2, 3, 7, 20, 22):
+        a, sa = co.conv1d_fwd(x[:, :, :cut], w, None, mask=mask[:, :cut], final_state_len=3, residual=1)
+        bpart, sb = co.conv1d_fwd(x[:, :, cut:], w, None, mask=mask[:, cut:], initial_state=sa,
+                                  final_state_len=5, residual=1)
+        assert torch.equal(torch.cat([a, bpart], dim=-1), full)
+        if L - cut >= 5 or cut >= 3:
+            # enough history travelled through the 3-slot intermediate state
+            k = min(5, (L - cut) + 3)
+            assert torch.equal(sb[:, :, -k:], fs[:, :, -k:])
+
+
+def test_linearity_causality_permutation_and_masks():
+    torch.manual_seed(5)
+    B, C, L = 3, 12, 40
+    x1, x2 = torch.randn(B, C, L).double(), torch.randn(B, C, L).double()
+    # values on a coarse grid make every fp32 operation exact -> exact linearity
+    q = lambda t: (t * 8).round().div(8).float()
+    x1, x2 = q(x1), q(x2)
+    w = q(torch.randn(C, 4).double())
+    y1, y2 = co.conv1d_fwd(x1, w), co.conv1d_fwd(x2, w)
+    assert torch.equal(co.conv1d_fwd(x1 + x2, w), y1 + y2)
+    assert torch.equal(co.conv1d_fwd(x1, 2 * w), 2 * y1)
+    # causality: a change at t0 reaches t0 .. t0+3 only
+    xp = x1.clone()
+    xp[:, :, 17] += 1.0
+    d = (co.conv1d_fwd(xp, w) != y1).any(dim=0).any(dim=0)
+    assert d.nonzero().flatten().tolist() == [17, 18, 19, 20]
+    # batch / channel permutation equivariance
+    pb, pc = torch.randperm(B), torch.randperm(C)
+    assert torch.equal(co.conv1d_fwd(x1[pb][:, pc], w[pc]), y1[pb][:, pc])
+    # masks: all ones == none; all zeros -> act(bias) (+ masked residual == 0)
+    bias = torch.randn(C)
+    ones, zeros = torch.ones(B, L), torch.zeros(B, L)
+    for act in (None, "silu"):
+        assert torch.equal(co.conv1d_fwd(x1, w, bias, mask=ones, activation=act, residual=1),
+                           co.conv1d_fwd(x1, w, bias, activation=act, residual=1))
+        z = co.conv1d_fwd(x1, w, bias, mask=zeros, activation=act, residual=1)
+        want = F.silu(bias) if act else bias
+        torch.testing.assert_close(z, want[None, :, None].expand(B, C, L), rtol=1e-6, atol=1e-7)
+    # masking multiplies: -x * 0 keeps its sign bit (the captured state must be bit exact)
+    neg = -x1.abs() - 1
+    _, fs = co.conv1d_fwd(neg, w, mask=zeros, final_state_len=4)
+    assert torch.equal(bits(fs), bits(torch.full_like(fs, -0.0)))
+
+
+# --------------------------------------------------------------------------
+# eager module restatement vs the real CanonLayer's vectors
+# --------------------------------------------------------------------------
+def _load_golden():
+    with open(os.path.join(GOLDEN, "canon_layer_cases.json")) as f:
+        manifest = json.load(f)
+    arrays = np.load(os.path.join(GOLDEN, "canon_layer_cases.npz"))
+    return manifest["cases"], arrays
+
+
+def golden_tensor(arrays, key, dtype):
+    a = torch.from_numpy(arrays[key])
+    return a.view(torch.bfloat16) if dtype == torch.bfloat16 else a
+
+
+@pytest.mark.parametrize("case", _load_golden()[0], ids=lambda c: c["name"])
+def test_eager_restatement_matches_canon_layer_golden(case):
+    _, arrays = _load_golden()
+    name = case["name"]
+    dtype = getattr(torch, case["dtype"])
+    w = golden_tensor(arrays, f"{name}/weight", dtype)
+    b = golden_tensor(arrays, f"{name}/bias", dtype) if case["bias"] else None
+    layer = EagerCanon(w, b, case["activation"])
+    cache = {}
+    for i, call in enumerate(case["calls"]):
+        key = f"{name}/call{i}"
+        x = golden_tensor(arrays, f"{key}/x", dtype)
+        mask = torch.from_numpy(arrays[f"{key}/mask"]) if call["mask"] else None
+        out = layer.forward(x, mask, cache if call["cache"] else None, "k")
+        want = golden_tensor(arrays, f"{key}/out", dtype)
+        assert torch.equal(bits(out), bits(want)), (name, i)
+        if call["cache"]:
+            want_state = golden_tensor(arrays, f"{key}/state", dtype)
+            assert torch.equal(bits(cache["k"]), bits(want_state)), (name, i)
+
+
+# --------------------------------------------------------------------------
+# kernel-level oracle vs the eager module (ties the two oracles together)
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", [False, True])
+def test_eager_rounding_mode_reproduces_eager_module(dtype, act):
+    torch.manual_seed(11)
+    B, T, D = 3, 50, 32
+    x = torch.randn(B, T, D).to(dtype)
+    w = (torch.randn(D, 4) * 0.4).to(dtype)
+    bias = (torch.randn(D) * 0.1).to(dtype)
+    lens = [50, 31, 7]
+    mask = torch.zeros(B, T, dtype=torch.int64)
+    for i, n in enumerate(lens):
+        mask[i, :n] = 1
+    cache = {}
+    want = EagerCanon(w, bias, act).forward(x, mask, cache, 0)
+    got, fs = co.conv1d_fwd(x.transpose(1, 2), w, bias, mask=mask, final_state_len=8,
+                            activation="silu" if act else None, residual=1, round_mode=1)
+    got = got.transpose(1, 2)
+    assert torch.equal(bits(fs), bits(cache[0]))
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    elif not act:
+        assert torch.equal(bits(got), bits(want))
+    else:
+        d = ulp_diff(got, want)   # expf of libm vs torch's vectorised exp
+        assert d.max().item() <= 1 and (d > 0).float().mean().item() < 0.01
+    # and the single-rounding result stays within one ulp of exact arithmetic
+    if dtype != torch.float32:
+        fused = co.conv1d_fwd(x.transpose(1, 2), w, bias, mask=mask,
+                              activation="silu" if act else None, residual=1)
+        x64 = (x * mask.unsqueeze(-1)).double().transpose(1, 2)
+        y64 = F.conv1d(F.pad(x64, (3, 0)), w.double().unsqueeze(1), bias.double(), groups=D)
+        if act:
+            y64 = F.silu(y64)
+        exact = (y64 + x64).to(dtype)
+        assert ulp_diff(fused, exact).max().item() <= 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_eager_step_mode_reproduces_eager_module(dtype):
+    torch.manual_seed(13)
+    B, D, S = 4, 48, 8
+    w = (torch.randn(D, 4) * 0.4).to(dtype)
+    bias = (torch.randn(D) * 0.1).to(dtype)
+    for act in (False, True):
+        layer = EagerCanon(w, bias, act)
+        cache = {0: torch.randn(B, D, S).to(dtype)}
+        state = cache[0].clone()
+        for _ in range(6):
+            x = torch.randn(B, 1, D).to(dtype)
+            want = layer.forward(x, None, cache, 0)[:, 0]
+            got = co.conv1d_update(x[:, 0].contiguous(), state, w, bias,
+                                   activation="silu" if act else None, residual=True, round_mode=1)
+            assert torch.equal(bits(state), bits(cache[0]))
+            if dtype == torch.float32:
+                torch.testing.assert_close(got, want, rtol=2e-6, atol=2e-6)
+            else:
+                d = ulp_diff(got, want)
+                assert d.max().item() <= 1 and (d > 0).float().mean().item() < 0.02

@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the Canon causal depthwise conv1d hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one prefill launch over bf16 x[B=8, C=3456, L=1024] (bias, residual
+add fused, no activation), inputs resident in HBM.  Launches rotate over
+enough distinct (x, out) buffer pairs that the working set is several times
+the 256 MB Infinity Cache, so the rate is an HBM rate, not a cache rate.
+Launches go through the C ABI (canon_conv1d_fwd) with prebuilt argument
+structs; time is taken with HIP events on the launch stream.
+
+The one JSON line also carries: the decode update (B=256, C=3456, state 3,
+64 carried steps) in microseconds per step, the same prefill in the
+channel-contiguous layout, the roofline fraction, and a CPU baseline (the
+eager PyTorch formulation of the reference on this box's host cores).
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "viby-model_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, vendor figure
+B, C, L, W = 8, 3456, 1024, 4   # the configuration the metric is quoted on
+DEC_B, DEC_S, DEC_STEPS = 256, 3, 64
+
+
+def prefill_bytes(b, c, l, esize=2, wsize=2):
+    # one read of x, one write of out, taps and bias once
+    return 2 * b * c * l * esize + c * W * wsize + c * wsize
+
+
+def decode_bytes(b, c, s, esize=2, wsize=2):
+    # state read + written, token read, output written, taps and bias
+    return b * c * (2 * s + 2) * esize + c * W * wsize + c * wsize
+
+
+def time_region(fn, steps, warmup):
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps  # ms per step
+
+
+def bench_prefill(layout, steps, warmup, nbuf):
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(0)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    xs, outs, params = [], [], []
+    for _ in range(nbuf):
+        if layout == "bcl":
+            x = torch.randn(B, C, L, generator=g, device=dev).bfloat16()
+        else:
+            x = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        o = torch.empty_like(x)
+        xs.append(x)
+        outs.append(o)
+        params.append(cc._fill_fwd(x, o, w, bias, None, None, None, 0, 1, 0))
+    plan = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(params[0])).decode()
+    fwd = _lib.lib().canon_conv1d_fwd
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    refs = [ctypes.byref(p) for p in params]
+
+    def step(i):
+        rc = fwd(refs[i % nbuf], stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_fwd")
+
+    ms = time_region(step, steps, warmup)
+    return ms, plan
+
+
+def bench_decode(reps, warmup):
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(1)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    state = torch.randn(DEC_B, C, DEC_S, generator=g, device=dev).bfloat16()
+    toks = torch.randn(DEC_STEPS, DEC_B, C, generator=g, device=dev).bfloat16()
+    outs = torch.empty_like(toks)
+    params = [cc._fill_update(toks[i], outs[i], state, w, bias, None, 0, 0, 0) for i in range(DEC_STEPS)]
+    refs = [ctypes.byref(p) for p in params]
+    upd = _lib.lib().canon_conv1d_update
+    plan = _lib.lib().canon_conv1d_update_plan(refs[0]).decode()
+
+    def run64(stream):
+        for r in refs:
+            rc = upd(r, stream)
+            if rc:
+                _lib.check(rc, "canon_conv1d_update")
+
+    cur = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ms_eager = time_region(lambda i: run64(cur), reps, warmup) / DEC_STEPS
+
+    # the same 64 carried steps as one HIP graph (what a decode loop would replay)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run64(ctypes.c_void_p(side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        run64(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    ms_graph = time_region(lambda i: graph.replay(), reps, warmup) / DEC_STEPS
+    return ms_eager * 1e3, ms_graph * 1e3, plan
+
+
+def cpu_baseline(budget_s=12.0):
+    """The reference's eager formulation (mask-free Canon-D call: pad + grouped
+    conv1d + residual, model/model.py:604-675) on the host cores, same shape."""
+    import torch
+    from oracle.canon_eager import EagerCanon
+    cores = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, L, C, generator=g).bfloat16()
+    w = (torch.randn(C, W, generator=g) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g) * 0.01).bfloat16()
+    layer = EagerCanon(w, bias, False)
+    layer.forward(x)
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        layer.forward(x)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(prefill_bytes(B, C, L) / med / 1e9, 3), "unit": "GB/s", "cores": cores,
+        "kind": "port",
+        "sample": f"{len(times)} passes of the full bf16 [8,3456,1024] step, eager torch restatement "
+                  f"(oracle/canon_eager.py), median {med * 1e3:.1f} ms",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU by design (rows of the conv are independent; "
+                 "there is no multi-GPU path to measure). Run with --gpus 1.")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    nbuf = 6  # 6 x 113 MB = 680 MB of distinct traffic between reuses
+    ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
+    ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
+    dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
+
+    nbytes = prefill_bytes(B, C, L)
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    out = {
+        "metric": "Canon conv1d HBM GB/s (prefill B8 L1024 C3456 bf16); decode us/step B256",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 storage, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "configs[1]: prefill bf16 x[B=8,C=3456,L=1024] time-contiguous, width 4, "
+                               "bias, residual fused, no activation", "kernel": plan,
+                   "rotating_buffer_pairs": nbuf},
+        "tokens_per_s": round(B * L / (ms * 1e-3)),
+        "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
+                                 "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1)},
+        "decode": {"workload": f"configs[3]: bf16 state[{DEC_B},{C},{DEC_S}], {DEC_STEPS} carried steps",
+                   "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
+                   "us_per_step_hipgraph": round(dec_graph_us, 3),
+                   "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

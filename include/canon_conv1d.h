@@ -1,0 +1,178 @@
+/*
+ * canon_conv1d.h -- C ABI of the MI355X (gfx950) Canon causal depthwise conv1d.
+ *
+ * Two operators, the two calls Viby's CanonLayer makes into an accelerated
+ * backend (reference = JohanLi233/Viby-Model):
+ *
+ *   canon_conv1d_fwd     replaces  causal_conv1d_fn      (prefill)
+ *   canon_conv1d_update  replaces  causal_conv1d_update  (one decode token)
+ *
+ * Plain pointers, sizes and element strides only; no framework types.  Every
+ * pointer is a DEVICE pointer owned by the caller.  Kernels are enqueued on
+ * the given HIP stream and the call returns without synchronising.  Nothing
+ * here allocates device memory.
+ *
+ * Status codes are returned as int; canon_conv1d_last_error() gives the
+ * message of the last failing call made by the calling thread.
+ */
+#ifndef CANON_CONV1D_H
+#define CANON_CONV1D_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CANON_CONV1D_ABI_VERSION 1
+#define CANON_CONV1D_MIN_WIDTH 2
+#define CANON_CONV1D_MAX_WIDTH 4
+
+/* storage type of x / out / states, and (independently) of weight / bias */
+enum { CANON_DTYPE_F32 = 0, CANON_DTYPE_BF16 = 1, CANON_DTYPE_F16 = 2 };
+
+/* element type of a padding mask (any value is multiplied in, 0/1 is usual) */
+enum {
+    CANON_MASK_U8 = 0,  /* also bool */
+    CANON_MASK_I32 = 1,
+    CANON_MASK_I64 = 2,
+    CANON_MASK_F32 = 3,
+    CANON_MASK_BF16 = 4,
+    CANON_MASK_F16 = 5
+};
+
+enum { CANON_ACT_NONE = 0, CANON_ACT_SILU = 1 };
+
+/* residual term added to the activated conv output */
+enum {
+    CANON_RESIDUAL_NONE = 0,
+    CANON_RESIDUAL_MASKED = 1,   /* out += x * mask  (eager CanonLayer, model/model.py:595,675) */
+    CANON_RESIDUAL_UNMASKED = 2  /* out += x         (fused branches,  model/model.py:491)     */
+};
+
+/*
+ * CANON_ROUND_FUSED: fp32 accumulate, SiLU and residual in fp32, one rounding
+ *                    to the storage type at the store.
+ * CANON_ROUND_EAGER: additionally rounds to the storage type after the conv,
+ *                    after SiLU and after the residual add -- the rounding
+ *                    points of the reference's eager module, so 16-bit
+ *                    results equal it bit for bit.  The update call in this
+ *                    mode follows model/model.py:385-396 (each product
+ *                    rounded, then the sum, then bias, then SiLU).
+ */
+enum { CANON_ROUND_FUSED = 0, CANON_ROUND_EAGER = 1 };
+
+enum {
+    CANON_OK = 0,
+    CANON_ERR_INVALID_ARGUMENT = 1,  /* caller error: shapes, strides, null pointers */
+    CANON_ERR_UNSUPPORTED = 2,       /* valid upstream feature this build does not implement */
+    CANON_ERR_LAUNCH = 3             /* HIP reported an error at launch */
+};
+
+/*
+ * Prefill.  Replaces causal_conv1d_fn(x, weight, bias, seq_idx, initial_states,
+ * return_final_states, final_states_out, activation) as called at
+ * model/model.py:460-466, and fuses what CanonLayer does around that call:
+ * the padding-mask multiply (model/model.py:454-457), the residual add (:491)
+ * and the conv-state capture (:470-489).
+ *
+ *   xm[b,c,t]  = mask ? round(x[b,c,t] * mask[b,t]) : x[b,c,t]
+ *   y[b,c,t]   = act(bias[c] + sum_{k<W} weight[c,k] * xm[b,c,t-(W-1)+k])
+ *   out        = y (+ xm | + x)
+ * with xm == 0 for t < 0, or the last W-1 entries of initial_state when given.
+ * final_state (optional) receives the last final_len entries of
+ * initial_state ++ xm, zero filled on the left.
+ *
+ * x / out are logical [batch, channels, seqlen] with element strides; both
+ * the time-contiguous ([B,C,L]) and the channel-contiguous ([B,L,C] viewed
+ * as [B,C,L], which is what model/model.py:459 passes) layouts have a
+ * vectorised kernel, anything else takes a strided scalar kernel.
+ * out must not alias x.
+ */
+typedef struct canon_conv1d_fwd_params {
+    uint32_t struct_size;           /* sizeof(canon_conv1d_fwd_params) */
+    int32_t x_dtype;                /* CANON_DTYPE_*: x, out, initial_state, final_state */
+    int32_t w_dtype;                /* CANON_DTYPE_*: weight and bias (rounded to x_dtype on load) */
+    int32_t mask_dtype;             /* CANON_MASK_*, ignored when mask == NULL */
+    int32_t width;                  /* W, 2..4 */
+    int32_t activation;             /* CANON_ACT_* */
+    int32_t residual_mode;          /* CANON_RESIDUAL_* */
+    int32_t round_mode;             /* CANON_ROUND_* */
+    int64_t batch, channels, seqlen;
+    const void *x;
+    int64_t x_stride_b, x_stride_c, x_stride_l;          /* in elements */
+    void *out;
+    int64_t out_stride_b, out_stride_c, out_stride_l;
+    const void *weight;             /* [channels, width] */
+    int64_t w_stride_c, w_stride_k;
+    const void *bias;               /* [channels] contiguous, or NULL */
+    const void *mask;               /* [batch, seqlen], or NULL */
+    int64_t mask_stride_b, mask_stride_l;
+    const void *initial_state;      /* [batch, channels, initial_len], or NULL */
+    int64_t init_stride_b, init_stride_c, init_stride_s;
+    int32_t initial_len;            /* >= W-1 when initial_state != NULL */
+    int32_t final_len;              /* >= 1 when final_state != NULL */
+    void *final_state;              /* [batch, channels, final_len], or NULL */
+    int64_t final_stride_b, final_stride_c, final_stride_s;
+} canon_conv1d_fwd_params;
+
+/*
+ * Decode update.  Replaces causal_conv1d_update(x, conv_state, weight, bias,
+ * activation) as called at model/model.py:305-311 (eager restatement:
+ * model/model.py:372-398).
+ *
+ *   xt[b,c]  = token_mask ? round(x[b,c] * token_mask[b]) : x[b,c]     (model/model.py:277-282)
+ *   y[b,c]   = act(bias[c] + sum_{k<W-1} weight[c,k] * state[b,c,S-(W-1)+k] + weight[c,W-1] * xt[b,c])
+ *   out      = y (+ xt | + x)
+ *   state   <- state shifted left by one, xt appended      (in place, pure copies)
+ *
+ * state_len S >= W-1.  A contiguous [B,C,S] state with S in {3,4,8} and
+ * channel-contiguous x/out takes the vectorised kernel.
+ */
+typedef struct canon_conv1d_update_params {
+    uint32_t struct_size;           /* sizeof(canon_conv1d_update_params) */
+    int32_t x_dtype, w_dtype, mask_dtype;
+    int32_t width;
+    int32_t activation;
+    int32_t residual_mode;
+    int32_t round_mode;
+    int32_t state_len;
+    int32_t reserved0;
+    int64_t batch, channels;
+    const void *x;
+    int64_t x_stride_b, x_stride_c;
+    void *out;
+    int64_t out_stride_b, out_stride_c;
+    void *conv_state;               /* [batch, channels, state_len], updated in place */
+    int64_t state_stride_b, state_stride_c, state_stride_s;
+    const void *weight;
+    int64_t w_stride_c, w_stride_k;
+    const void *bias;
+    const void *token_mask;         /* [batch], or NULL */
+    int64_t mask_stride_b;
+    const int32_t *cache_seqlens;        /* upstream's circular-buffer mode: must be NULL */
+    const int32_t *conv_state_indices;   /* upstream's batch indirection:    must be NULL */
+} canon_conv1d_update_params;
+
+int canon_conv1d_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *canon_conv1d_last_error(void);
+
+/* Enqueue on `stream` (a hipStream_t; NULL = the default stream). */
+int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream);
+int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
+
+/*
+ * Name of the kernel family the call above would launch for these arguments
+ * ("bcl_vec", "blc_vec", "generic", "update_vec", "update_generic"), or NULL
+ * if the arguments are rejected.  Launches nothing.  Lets a caller or a test
+ * assert that a layout takes the fast path.
+ */
+const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p);
+const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CANON_CONV1D_H */

@@ -1,0 +1,41 @@
+"""Shared helpers of the parity tests."""
+import torch
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    """Raw storage bits (so that -0.0 != 0.0 and NaNs compare by pattern)."""
+    t = t.detach().cpu().contiguous()
+    return t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+def ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in representable values of a 16-bit float type (bf16 / fp16)."""
+    def key(t):
+        i = t.detach().cpu().contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+        return torch.where(i >= 0x8000, 0x8000 - i, i)
+    return (key(a) - key(b)).abs()
+
+
+def assert_parity(got: torch.Tensor, want: torch.Tensor, exact: bool, what: str = "") -> None:
+    """The bar of this repository.
+
+    16-bit storage: at most 1 ulp from the fp32-accumulate oracle (bit exact
+    when `exact`).  fp32: bit exact when `exact`, else 1e-5 relative.
+    """
+    got, want = got.detach().cpu(), want.detach().cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype, (what, got.shape, want.shape)
+    if exact:
+        assert torch.equal(bits(got), bits(want)), f"{what}: not bit exact"
+    elif got.dtype == torch.float32:
+        err = (got - want).abs() / want.abs().clamp_min(1e-3)
+        assert err.max().item() <= 1e-5, f"{what}: rel err {err.max().item():.3e} > 1e-5"
+    else:
+        d = ulp_diff(got, want)
+        assert d.max().item() <= 1, f"{what}: {d.max().item()} ulp > 1"
+
+
+def right_padded_mask(lens, L, dtype=torch.int64):
+    m = torch.zeros(len(lens), L, dtype=dtype)
+    for b, n in enumerate(lens):
+        m[b, :n] = 1
+    return m

@@ -1,0 +1,337 @@
+"""HIP kernels (through the C ABI, via the drop-in package) vs the CPU oracle.
+
+Bar: conv_state bit exact; outputs bit exact without SiLU (same fma chain on
+both sides), with SiLU within 1 bf16/fp16 ulp resp. 1e-5 relative for fp32
+(the GPU uses v_exp_f32 / v_rcp_f32, the oracle libm).
+"""
+import itertools
+
+import pytest
+import torch
+
+from helpers import assert_parity, bits, right_padded_mask
+from oracle import canon_oracle as co
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def cc():
+    import causal_conv1d
+    return causal_conv1d
+
+
+def layouts(x_bcl_cpu):
+    """The same logical [B,C,L] tensor on the GPU in both dense layouts."""
+    xg = x_bcl_cpu.to(DEV)
+    yield "bcl", xg
+    yield "blc", xg.transpose(1, 2).contiguous().transpose(1, 2)
+
+
+def run_fwd(cc, x, w, b, act=None, mask=None, residual=False, init=None, S_out=None, rounding="fused"):
+    fs = None
+    if S_out is not None:
+        fs = torch.full((x.shape[0], x.shape[1], S_out), float("nan"), dtype=x.dtype, device=DEV)
+    r = cc.causal_conv1d_fn(x, w.to(DEV), None if b is None else b.to(DEV), activation=act,
+                            attention_mask=None if mask is None else mask.to(DEV), residual=residual,
+                            initial_states=None if init is None else init.to(DEV),
+                            final_states_out=fs, rounding=rounding)
+    torch.cuda.synchronize()
+    return r
+
+
+# ---- BASELINE config 1 ------------------------------------------------------
+def test_config1_fp32_canon_a(cc):
+    torch.manual_seed(0)
+    x = torch.randn(1, 640, 1024)
+    w = torch.randn(640, 4) * 0.02
+    b = torch.zeros(640)
+    want = co.conv1d_fwd(x, w, b, residual=1)
+    for name, xg in layouts(x):
+        assert cc.kernel_plan_fwd(xg, w.to(DEV)) == f"{name}_vec"
+        got = run_fwd(cc, xg, w, b, residual=True)
+        assert got.stride() == xg.stride()
+        assert_parity(got, want, exact=True, what=f"config1/{name}")
+
+
+# ---- BASELINE config 2 ------------------------------------------------------
+@pytest.mark.parametrize("C", [640, 960, 3456])
+@pytest.mark.parametrize("act", [None, "silu"])
+def test_config2_bf16_prefill(cc, C, act):
+    g = torch.Generator().manual_seed(C)
+    x = torch.randn(8, C, 1024, generator=g).bfloat16()
+    w = (torch.randn(C, 4, generator=g) * 0.02).bfloat16()
+    b = (torch.randn(C, generator=g) * 0.01).bfloat16()
+    want = co.conv1d_fwd(x, w, b, activation=act)
+    for name, xg in layouts(x):
+        assert cc.kernel_plan_fwd(xg, w.to(DEV)) == f"{name}_vec"
+        got = run_fwd(cc, xg, w, b, act=act)
+        assert_parity(got, want, exact=act is None, what=f"config2/C{C}/{act}/{name}")
+
+
+# ---- BASELINE config 3 ------------------------------------------------------
+@pytest.mark.parametrize("residual", ["masked", "unmasked"])
+def test_config3_ragged_padded_prefill(cc, residual):
+    g = torch.Generator().manual_seed(3)
+    B, C, L = 32, 3456, 1024
+    x = torch.randn(B, C, L, generator=g).bfloat16()
+    w = (torch.randn(C, 4, generator=g) * 0.02).bfloat16()
+    b = (torch.randn(C, generator=g) * 0.01).bfloat16()
+    lens = torch.randint(128, 1025, (B,), generator=g).tolist()
+    mask = right_padded_mask(lens, L)
+    want, want_fs = co.conv1d_fwd(x, w, b, mask=mask, residual=residual, final_state_len=4)
+    for name, xg in layouts(x):
+        got, fs = run_fwd(cc, xg, w, b, mask=mask, residual=residual, S_out=4)
+        assert_parity(got, want, exact=True, what=f"config3/{name}")
+        assert torch.equal(bits(fs), bits(want_fs)), f"config3/{name}: state"
+        del got, fs, xg
+    # size-independent properties at full size: all-ones mask == no mask
+    xg = x.to(DEV)
+    ones = torch.ones(B, L, dtype=torch.bool)
+    a = run_fwd(cc, xg, w, b, mask=ones, residual=residual)
+    c = run_fwd(cc, xg, w, b, residual=residual)
+    assert torch.equal(bits(a), bits(c))
+
+
+# ---- BASELINE config 4 ------------------------------------------------------
+@pytest.mark.parametrize("S", [3, 4, 8])
+def test_config4_decode_64_steps(cc, S):
+    g = torch.Generator().manual_seed(4)
+    B, C, steps = 256, 3456, 64
+    state0 = torch.randn(B, C, S, generator=g).bfloat16()
+    xs = torch.randn(steps, B, C, generator=g).bfloat16()
+    w = (torch.randn(C, 4, generator=g) * 0.02).bfloat16()
+    b = (torch.randn(C, generator=g) * 0.01).bfloat16()
+    st_ref = state0.clone()
+    st_gpu = state0.to(DEV)
+    ptr = st_gpu.data_ptr()
+    wg, bg, xg = w.to(DEV), b.to(DEV), xs.to(DEV)
+    assert cc.kernel_plan_update(xg[0], st_gpu, wg, bg) == "update_vec"
+    for i in range(steps):
+        want = co.conv1d_update(xs[i], st_ref, w, b)
+        got = cc.causal_conv1d_update(xg[i], st_gpu, wg, bg)
+        assert_parity(got, want, exact=True, what=f"config4/S{S}/step{i}")
+    assert st_gpu.data_ptr() == ptr
+    assert torch.equal(bits(st_gpu), bits(st_ref))
+    # closed form: the state is the last S tokens (S <= steps)
+    assert torch.equal(bits(st_gpu), bits(xs[-S:].permute(1, 2, 0)))
+
+
+# ---- the reference's own grid (causal-conv1d-mps/test.py:110-146) -----------
+@pytest.mark.parametrize("itype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("has_bias", [False, True])
+def test_reference_grid(cc, itype, silu, has_bias):
+    for dim, seqlen in itertools.product([64, 128, 256], [1, 2, 8, 16, 32, 64, 128, 256]):
+        torch.manual_seed(42)
+        x = torch.randn(2, dim, seqlen).to(itype)
+        w = torch.randn(dim, 4)                      # fp32 weights, cast by the callee
+        b = torch.randn(dim) if has_bias else None
+        act = "silu" if silu else None
+        want = co.conv1d_fwd(x, w, b, activation=act)
+        for name, xg in layouts(x):
+            got = run_fwd(cc, xg, w, b, act=act)
+            assert_parity(got, want, exact=not silu, what=f"grid/{dim}/{seqlen}/{name}")
+        # the reference's own tolerance, for the record (test.py:121-126)
+        rtol, atol = {torch.float32: (3e-4, 1e-3), torch.bfloat16: (5e-3, 2e-2), torch.float16: (3e-3, 5e-3)}[itype]
+        torch.testing.assert_close(got.cpu(), want, rtol=rtol, atol=atol)
+
+
+# ---- fused mask + residual, the reference's fused test (test.py:149-197) ----
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("has_bias", [False, True])
+def test_short_conv_fused_reference_case(cc, silu, has_bias):
+    for dim, seqlen in itertools.product([64, 128], [8, 16, 32, 64]):
+        torch.manual_seed(42)
+        x = torch.randn(2, seqlen, dim)
+        w = torch.randn(dim, 4)
+        b = torch.randn(dim) if has_bias else None
+        mask = torch.ones(2, seqlen)
+        for i in range(2):
+            mask[i, int(torch.randint(seqlen // 2, seqlen, (1,))):] = 0
+        got = cc.short_conv_fused(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), mask.to(DEV),
+                                  activation=silu, residual=True)
+        want = co.conv1d_fwd(x.transpose(1, 2), w, b, mask=mask, activation="silu" if silu else None,
+                             residual="unmasked").transpose(1, 2)
+        assert_parity(got, want, exact=not silu, what=f"fused/{dim}/{seqlen}")
+
+
+# ---- edge shapes, odd strides, every kernel family --------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_edge_shapes_and_strides(cc, dtype):
+    g = torch.Generator().manual_seed(9)
+    cases = [(1, 1, 1), (2, 3, 5), (1, 8, 3), (3, 7, 129), (2, 16, 128), (2, 24, 136), (1, 40, 1000),
+             (2, 8, 2048 + 8), (1, 2, 8192), (5, 1000, 9)]
+    for (B, C, L), W in itertools.product(cases, [2, 3, 4]):
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = torch.randn(C, W, generator=g).to(dtype)
+        b = torch.randn(C, generator=g).to(dtype)
+        lens = torch.randint(1, L + 1, (B,), generator=g).tolist()
+        mask = right_padded_mask(lens, L, torch.int32)
+        want, wfs = co.conv1d_fwd(x, w, b, mask=mask, residual=1, final_state_len=W)
+        for name, xg in layouts(x):
+            got, fs = run_fwd(cc, xg, w, b, mask=mask, residual=True, S_out=W)
+            assert_parity(got, want, exact=True, what=f"edge/{B}x{C}x{L}/W{W}/{name}")
+            assert torch.equal(bits(fs), bits(wfs))
+    # views that are neither dense layout: slices in every dimension, misaligned base
+    big = torch.randn(3, 37, 301, generator=g).to(dtype)
+    w = torch.randn(20, 4, generator=g).to(dtype)
+    xg = big.to(DEV)[1:3, 5:25, 3:280:2]
+    want = co.conv1d_fwd(big[1:3, 5:25, 3:280:2], w, None, activation="silu")
+    got = run_fwd(cc, xg, w, None, act="silu")
+    assert_parity(got, want, exact=False, what="edge/strided view")
+    # dense but misaligned (base pointer off by one element) -> scalar kernel, same answer
+    flat = torch.randn(2 * 16 * 256 + 1, generator=g).to(dtype)
+    xv = flat[1:].view(2, 16, 256)
+    w = torch.randn(16, 4, generator=g).to(dtype)
+    xg = flat.to(DEV)[1:].view(2, 16, 256)
+    assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "generic"
+    assert_parity(run_fwd(cc, xg, w, None), co.conv1d_fwd(xv, w), exact=True, what="edge/misaligned")
+
+
+def test_empty_inputs(cc):
+    w = torch.randn(8, 4, device=DEV)
+    for shape in [(0, 8, 16), (2, 8, 0)]:
+        out = cc.causal_conv1d_fn(torch.empty(shape, device=DEV), w)
+        assert out.shape == shape
+    st = torch.zeros(0, 8, 4, device=DEV)
+    assert cc.causal_conv1d_update(torch.empty(0, 8, device=DEV), st, w).shape == (0, 8)
+
+
+# ---- initial / final states, chunking, streaming ----------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chunked_prefill_and_streaming_equivalence(cc, dtype):
+    g = torch.Generator().manual_seed(21)
+    B, C, L = 2, 64, 512
+    x = torch.randn(B, C, L, generator=g).to(dtype)
+    w = (torch.randn(C, 4, generator=g) * 0.3).to(dtype)
+    b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+    for name, xg in layouts(x):
+        full, fs_full = run_fwd(cc, xg, w, b, S_out=8)
+        # prefill in two pieces joined through a 3-slot state
+        for cut in (8, 128, 264):
+            first = xg[:, :, :cut]
+            second = xg[:, :, cut:]
+            if name == "bcl":
+                first, second = first.contiguous(), second.contiguous()
+            a, sa = run_fwd(cc, first, w, b, S_out=3)
+            c, sc = run_fwd(cc, second, w, b, init=sa, S_out=8)
+            assert torch.equal(bits(torch.cat([a, c], dim=-1)), bits(full)), (name, cut)
+            assert torch.equal(bits(sc), bits(fs_full))
+        # prefill then single-token updates == one prefill
+        head = xg[:, :, :500].contiguous() if name == "bcl" else xg[:, :, :500]
+        out_h, state = run_fwd(cc, head, w, b, S_out=4)
+        cols = []
+        for t in range(500, L):
+            cols.append(cc.causal_conv1d_update(xg[:, :, t], state, w.to(DEV), b.to(DEV)))
+        got = torch.cat([out_h, torch.stack(cols, dim=-1)], dim=-1)
+        assert torch.equal(bits(got), bits(full)), name
+        assert torch.equal(bits(state), bits(fs_full[:, :, -4:]))
+
+
+def test_update_variants_vs_oracle(cc):
+    g = torch.Generator().manual_seed(33)
+    for dtype, W, S, (B, C), act, res in itertools.product(
+            [torch.float32, torch.bfloat16, torch.float16], [2, 3, 4], [3, 4, 5, 8],
+            [(1, 8), (3, 20), (5, 256), (2, 1000)], [None, "silu"], [False, "masked", "unmasked"]):
+        x = torch.randn(B, C, generator=g).to(dtype)
+        st = torch.randn(B, C, S, generator=g).to(dtype)
+        w = torch.randn(C, W, generator=g)
+        b = torch.randn(C, generator=g)
+        tm = (torch.rand(B, generator=g) > 0.3).to(torch.int64)
+        # oracle: masked token in, residual adds masked or raw token
+        xt = (x * tm[:, None]).to(dtype)
+        st_ref = st.clone()
+        want = co.conv1d_update(xt, st_ref, w, b, activation=act, residual=(res == "masked"))
+        if res == "unmasked":
+            want = want.float() + x.float()      # rounded before this add: loose comparison below
+        st_gpu = st.to(DEV)
+        got = cc.causal_conv1d_update(x.to(DEV), st_gpu, w.to(DEV), b.to(DEV), activation=act,
+                                      token_mask=tm.to(DEV), residual=res)
+        assert torch.equal(bits(st_gpu), bits(st_ref)), (dtype, W, S, B, C)
+        if res == "unmasked":
+            torch.testing.assert_close(got.cpu().float(), want, rtol=2e-2, atol=2e-2)
+        else:
+            assert_parity(got, want, exact=act is None, what=f"update/{dtype}/W{W}/S{S}/{B}x{C}/{res}")
+
+
+def test_update_residual_exact(cc):
+    g = torch.Generator().manual_seed(34)
+    for dtype, S in itertools.product([torch.float32, torch.bfloat16], [3, 4, 8, 6]):
+        B, C = 4, 264
+        x = torch.randn(B, C, generator=g).to(dtype)
+        st = torch.randn(B, C, S, generator=g).to(dtype)
+        w = torch.randn(C, 4, generator=g).to(dtype)
+        st_ref = st.clone()
+        want = co.conv1d_update(x, st_ref, w, None, residual=True)
+        st_gpu = st.to(DEV)
+        got = cc.short_conv_update(x.to(DEV), st_gpu, w.to(DEV), None, activation=False, residual=True)
+        assert_parity(got, want, exact=True, what=f"update residual S{S}")
+        assert torch.equal(bits(st_gpu), bits(st_ref))
+
+
+def test_noncontiguous_state_takes_strided_kernel_and_stays_in_place(cc):
+    g = torch.Generator().manual_seed(35)
+    B, C, S = 3, 64, 4
+    big = torch.randn(B, C, 2 * S, generator=g).bfloat16()
+    x = torch.randn(B, C, generator=g).bfloat16()
+    w = torch.randn(C, 4, generator=g).bfloat16()
+    big_g = big.to(DEV)
+    view = big_g[:, :, ::2]
+    assert cc.kernel_plan_update(x.to(DEV), view, w.to(DEV)) == "update_generic"
+    st_ref = big[:, :, ::2].contiguous()
+    want = co.conv1d_update(x, st_ref, w)
+    got = cc.causal_conv1d_update(x.to(DEV), view, w.to(DEV))
+    assert_parity(got, want, exact=True)
+    assert torch.equal(bits(big_g[:, :, ::2]), bits(st_ref))
+    assert torch.equal(bits(big_g[:, :, 1::2]), bits(big[:, :, 1::2]))   # untouched neighbours
+
+
+# ---- eager rounding mode: bit parity with the eager module ------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("act", [False, True])
+def test_eager_rounding_matches_eager_module(cc, dtype, act):
+    from oracle.canon_eager import EagerCanon
+    torch.manual_seed(77)
+    B, T, D = 4, 200, 96
+    x = torch.randn(B, T, D).to(dtype)
+    w = (torch.randn(D, 4) * 0.4).to(dtype)
+    bias = (torch.randn(D) * 0.1).to(dtype)
+    mask = right_padded_mask([200, 150, 64, 3], T)
+    cache = {}
+    want = EagerCanon(w, bias, act).forward(x, mask, cache, 0)
+    fs = torch.empty(B, D, 8, dtype=dtype, device=DEV)
+    got, fs = cc.causal_conv1d_fn(x.to(DEV).transpose(1, 2), w.to(DEV), bias.to(DEV),
+                                  activation="silu" if act else None, attention_mask=mask.to(DEV),
+                                  residual="masked", rounding="eager", final_states_out=fs)
+    got = got.transpose(1, 2)
+    assert torch.equal(bits(fs), bits(cache[0]))
+    assert_parity(got, want, exact=(not act and dtype != torch.float32), what="eager mode")
+    # decode steps in eager mode
+    state = fs
+    layer = EagerCanon(w, bias, act)
+    for _ in range(4):
+        xt = torch.randn(B, 1, D).to(dtype)
+        want = layer.forward(xt, None, cache, 0)[:, 0]
+        got = cc.causal_conv1d_update(xt[:, 0].to(DEV), state, w.to(DEV), bias.to(DEV),
+                                      activation="silu" if act else None, residual="unmasked",
+                                      rounding="eager")
+        assert torch.equal(bits(state), bits(cache[0]))
+        assert_parity(got, want, exact=False, what="eager step")
+
+
+def test_errors_surface(cc):
+    x = torch.randn(2, 8, 16, device=DEV)
+    w = torch.randn(8, 4, device=DEV)
+    with pytest.raises(ValueError, match="does not match"):
+        cc.causal_conv1d_fn(x, torch.randn(5, 4, device=DEV))
+    with pytest.raises(NotImplementedError, match="width"):
+        cc.causal_conv1d_fn(x, torch.randn(8, 5, device=DEV))
+    with pytest.raises(NotImplementedError):
+        cc.causal_conv1d_fn(x, w, seq_idx=torch.zeros(2, 16, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError, match="shorter than width-1"):
+        cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 2, device=DEV), w)
+    with pytest.raises(NotImplementedError, match="backward"):
+        cc.causal_conv1d_fn(x.requires_grad_(), w)

@@ -1,0 +1,418 @@
+"""MI355X (gfx950) causal depthwise conv1d, importable as ``causal_conv1d``.
+
+This is the package name Viby's ``model/model.py:21-25`` imports, so with this
+directory's parent on ``sys.path`` the Canon layers take this implementation
+on ROCm devices without any change to the model code::
+
+    from causal_conv1d import causal_conv1d_fn, causal_conv1d_update
+
+``causal_conv1d_fn`` / ``causal_conv1d_update`` keep the upstream call
+signatures used at ``model/model.py:460-466`` and ``:305-311`` (keyword set as
+mirrored in ``causal-conv1d-mps/causal_conv1d_mps/autograd.py:501-510``).
+Keyword-only extras fuse what CanonLayer does around those calls
+(``attention_mask``, ``residual``), modelled on the reference's own fused API
+``short_conv_fused`` / ``short_conv_update``
+(``causal_conv1d_mps/__init__.py:154-161`` and ``:304-312``), which is also
+exported here with the same argument meaning.
+
+Everything runs in hand-written HIP kernels behind a C ABI
+(``include/canon_conv1d.h``); there is no PyTorch fallback: a missing library
+or a rejected call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple, Union
+
+import torch
+
+from . import _lib
+from ._lib import FwdParams, UpdateParams
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "causal_conv1d_fn",
+    "causal_conv1d_update",
+    "short_conv_fused",
+    "short_conv_update",
+    "kernel_plan_fwd",
+    "kernel_plan_update",
+]
+
+MIN_WIDTH, MAX_WIDTH = 2, 4   # CANON_CONV1D_MIN_WIDTH / _MAX_WIDTH
+
+_RESIDUAL = {False: 0, None: 0, 0: 0, True: 1, 1: 1, "masked": 1, 2: 2, "unmasked": 2}
+
+
+def _activation_flag(activation) -> int:
+    if activation not in (None, "silu", "swish"):
+        raise NotImplementedError("activation must be None, silu, or swish")
+    return 0 if activation is None else 1
+
+
+def _residual_mode(residual) -> int:
+    try:
+        return _RESIDUAL[residual]
+    except (KeyError, TypeError):
+        raise ValueError(f"residual must be False, True/'masked' or 'unmasked', got {residual!r}") from None
+
+
+def _round_mode(rounding: str) -> int:
+    try:
+        return _lib.ROUND_CODE[rounding]
+    except KeyError:
+        raise ValueError(f"rounding must be 'fused' or 'eager', got {rounding!r}") from None
+
+
+def _require_gpu(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cuda":
+        raise ValueError(f"{what} must be on a ROCm GPU device (device type 'cuda'), got {t.device}")
+
+
+def _no_grad_needed(*tensors) -> None:
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise NotImplementedError(
+            "causal_conv1d (gfx950): backward is not implemented; call under torch.no_grad() "
+            "or detach the inputs")
+
+
+def _check_shapes(x_dim: int, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
+    """Shape / dtype errors first (they do not depend on where the tensors live)."""
+    if weight.dim() != 2:
+        raise ValueError(f"Expected 2D weight tensor (dim, width), got {weight.dim()}D")
+    if x_dim != weight.shape[0]:
+        raise ValueError(f"Input dim {x_dim} does not match weight dim {weight.shape[0]}")
+    if not MIN_WIDTH <= weight.shape[1] <= MAX_WIDTH:
+        raise NotImplementedError(f"width {weight.shape[1]} not supported (only widths 2..4)")
+    if weight.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"Unsupported weight dtype {weight.dtype}")
+    if bias is not None:
+        if bias.dim() != 1:
+            raise ValueError(f"Expected 1D bias tensor, got {bias.dim()}D")
+        if bias.shape[0] != x_dim:
+            raise ValueError(f"Bias dim {bias.shape[0]} does not match input dim {x_dim}")
+
+
+def _check_devices(weight: torch.Tensor, bias: Optional[torch.Tensor], dev) -> None:
+    _require_gpu(weight, "Weight tensor")
+    if bias is not None:
+        _require_gpu(bias, "Bias tensor")
+    if weight.device != dev or (bias is not None and bias.device != dev):
+        raise ValueError("weight and bias must be on the same device as x")
+
+
+def _prep_bias(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    # the kernels read weight and bias with one element type
+    if bias is None:
+        return None
+    if bias.dtype != weight.dtype or not bias.is_contiguous():
+        bias = bias.to(weight.dtype).contiguous()
+    return bias
+
+
+def _stream(dev: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd) -> FwdParams:
+    p = FwdParams()
+    p.struct_size = ctypes.sizeof(FwdParams)
+    p.x_dtype = _lib.DTYPE_CODE[x.dtype]
+    p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
+    p.width = weight.shape[1]
+    p.activation, p.residual_mode, p.round_mode = act, res, rnd
+    p.batch, p.channels, p.seqlen = x.shape
+    p.x = x.data_ptr()
+    p.x_stride_b, p.x_stride_c, p.x_stride_l = x.stride()
+    p.out = out.data_ptr()
+    p.out_stride_b, p.out_stride_c, p.out_stride_l = out.stride()
+    p.weight = weight.data_ptr()
+    p.w_stride_c, p.w_stride_k = weight.stride()
+    p.bias = bias.data_ptr() if bias is not None else None
+    if mask is not None:
+        p.mask = mask.data_ptr()
+        p.mask_dtype = _lib.MASK_CODE[mask.dtype]
+        p.mask_stride_b, p.mask_stride_l = mask.stride()
+    if initial_states is not None:
+        p.initial_state = initial_states.data_ptr()
+        p.init_stride_b, p.init_stride_c, p.init_stride_s = initial_states.stride()
+        p.initial_len = initial_states.shape[2]
+    if final_states is not None:
+        p.final_state = final_states.data_ptr()
+        p.final_stride_b, p.final_stride_c, p.final_stride_s = final_states.stride()
+        p.final_len = final_states.shape[2]
+    return p
+
+
+def causal_conv1d_fn(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    seq_idx: Optional[torch.Tensor] = None,
+    initial_states: Optional[torch.Tensor] = None,
+    return_final_states: bool = False,
+    final_states_out: Optional[torch.Tensor] = None,
+    activation: Optional[str] = None,
+    *,
+    attention_mask: Optional[torch.Tensor] = None,
+    residual: Union[bool, str] = False,
+    rounding: str = "fused",
+) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """Causal depthwise conv over ``x`` of shape (batch, dim, seqlen).
+
+    ``out[b,c,t] = act(bias[c] + sum_k weight[c,k] * x[b,c,t-(W-1)+k])`` with
+    fp32 accumulation and one rounding to ``x.dtype``.  ``x`` may be time
+    contiguous or channel contiguous (a transposed (batch, seqlen, dim) tensor,
+    which is what ``model/model.py:459`` passes); the output has x's strides.
+
+    initial_states   (batch, dim, >= W-1): history before t = 0 instead of zeros.
+    return_final_states / final_states_out (batch, dim, S): receives the last S
+                     inputs (S = W-1 when allocated here; any S >= 1 when
+                     given, e.g. the 4- or 8-slot conv_state of CanonLayer,
+                     ``model/model.py:470-489``); the result is then
+                     ``(out, final_states)``.
+    attention_mask   (batch, seqlen) 0/1 of any dtype: inputs are multiplied by
+                     it before the conv (``model/model.py:454-457``) and the
+                     captured state holds the masked inputs.
+    residual         False | True ('masked': ``out += x*mask``, the eager
+                     CanonLayer, ``model/model.py:595,675``) | 'unmasked'
+                     (``out += x``, ``model/model.py:491``).
+    rounding         'fused' (one rounding) | 'eager' (also rounds after the
+                     conv, after SiLU and after the residual add, which
+                     reproduces the eager bf16/fp16 module bit for bit).
+    """
+    act = _activation_flag(activation)
+    res = _residual_mode(residual)
+    rnd = _round_mode(rounding)
+    if seq_idx is not None:
+        raise NotImplementedError("seq_idx (packed variable-length batches) is not supported")
+    if x.dim() != 3:
+        raise ValueError(f"Expected 3D input tensor (batch, dim, seqlen), got {x.dim()}D")
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"Unsupported input dtype {x.dtype}; expected float32, bfloat16 or float16")
+    batch, dim, seqlen = x.shape
+    _check_shapes(dim, weight, bias)
+    _require_gpu(x, "Input tensor")
+    _check_devices(weight, bias, x.device)
+    _no_grad_needed(x, weight, bias, initial_states)
+    bias = _prep_bias(weight, bias)
+
+    if attention_mask is not None:
+        if attention_mask.dim() != 2:
+            raise ValueError(f"Expected 2D attention mask, got {attention_mask.dim()}D")
+        if tuple(attention_mask.shape) != (batch, seqlen):
+            raise ValueError(
+                f"Attention mask shape {tuple(attention_mask.shape)} does not match input shape ({batch}, {seqlen})")
+        if attention_mask.dtype not in _lib.MASK_CODE:
+            raise ValueError(f"Unsupported attention mask dtype {attention_mask.dtype}")
+        if attention_mask.device != x.device:
+            raise ValueError("Attention mask must be on the same device as x")
+    width = weight.shape[1]
+    if initial_states is not None:
+        if initial_states.dim() != 3 or tuple(initial_states.shape[:2]) != (batch, dim):
+            raise ValueError(f"initial_states shape {tuple(initial_states.shape)} does not match (batch, dim, >=width-1)")
+        if initial_states.dtype != x.dtype or initial_states.device != x.device:
+            raise ValueError("initial_states must have the dtype and device of x")
+    final_states = None
+    if return_final_states or final_states_out is not None:
+        if final_states_out is not None:
+            if final_states_out.dim() != 3 or tuple(final_states_out.shape[:2]) != (batch, dim):
+                raise ValueError(
+                    f"final_states_out shape {tuple(final_states_out.shape)} does not match (batch, dim, state_len)")
+            if final_states_out.dtype != x.dtype or final_states_out.device != x.device:
+                raise ValueError("final_states_out must have the dtype and device of x")
+            final_states = final_states_out
+        else:
+            final_states = torch.empty(batch, dim, width - 1, dtype=x.dtype, device=x.device)
+
+    if x.stride(2) != 1 and x.stride(1) != 1:
+        x = x.contiguous()
+    out = torch.empty_like(x)
+    if x.numel() == 0:
+        if final_states is not None and final_states.numel():
+            raise ValueError("cannot produce final states from an empty input")
+        return out if final_states is None else (out, final_states)
+
+    p = _fill_fwd(x, out, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().canon_conv1d_fwd(ctypes.byref(p), _stream(x.device))
+    _lib.check(rc, "causal_conv1d_fn")
+    return out if final_states is None else (out, final_states)
+
+
+def _fill_update(x2, out2, conv_state, weight, bias, token_mask, act, res, rnd) -> UpdateParams:
+    p = UpdateParams()
+    p.struct_size = ctypes.sizeof(UpdateParams)
+    p.x_dtype = _lib.DTYPE_CODE[x2.dtype]
+    p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
+    p.width = weight.shape[1]
+    p.activation, p.residual_mode, p.round_mode = act, res, rnd
+    p.state_len = conv_state.shape[2]
+    p.batch, p.channels = x2.shape
+    p.x = x2.data_ptr()
+    p.x_stride_b, p.x_stride_c = x2.stride()
+    p.out = out2.data_ptr()
+    p.out_stride_b, p.out_stride_c = out2.stride()
+    p.conv_state = conv_state.data_ptr()
+    p.state_stride_b, p.state_stride_c, p.state_stride_s = conv_state.stride()
+    p.weight = weight.data_ptr()
+    p.w_stride_c, p.w_stride_k = weight.stride()
+    p.bias = bias.data_ptr() if bias is not None else None
+    if token_mask is not None:
+        p.token_mask = token_mask.data_ptr()
+        p.mask_dtype = _lib.MASK_CODE[token_mask.dtype]
+        p.mask_stride_b = token_mask.stride(0)
+    return p
+
+
+def causal_conv1d_update(
+    x: torch.Tensor,
+    conv_state: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    activation: Optional[str] = None,
+    cache_seqlens: Optional[torch.Tensor] = None,
+    conv_state_indices: Optional[torch.Tensor] = None,
+    *,
+    token_mask: Optional[torch.Tensor] = None,
+    residual: Union[bool, str] = False,
+    rounding: str = "fused",
+) -> torch.Tensor:
+    """One decode step: ``x`` (batch, dim) or (batch, dim, 1); ``conv_state``
+    (batch, dim, state_len >= W-1) is updated IN PLACE (shifted left by one,
+    the token appended), so the caller's tensor object keeps holding the state
+    (``model/model.py:305-313`` relies on that).
+
+    ``out = act(bias + sum_{k<W-1} w[k]*state[S-(W-1)+k] + w[W-1]*x)``.
+
+    token_mask  (batch,) multiplies the token before everything else
+                (``model/model.py:277-282``).
+    residual    False | True ('masked': adds the masked token,
+                ``model/model.py:313``) | 'unmasked' (``model/model.py:370``).
+    rounding    'fused' | 'eager' (the rounding points of
+                ``model/model.py:385-396``).
+    """
+    act = _activation_flag(activation)
+    res = _residual_mode(residual)
+    rnd = _round_mode(rounding)
+    if cache_seqlens is not None:
+        raise NotImplementedError("cache_seqlens (circular conv_state) is not supported")
+    if conv_state_indices is not None:
+        raise NotImplementedError("conv_state_indices is not supported")
+    squeeze_back = False
+    if x.dim() == 3:
+        if x.shape[2] != 1:
+            raise NotImplementedError("causal_conv1d_update handles one token per call (seqlen 1)")
+        x2 = x[:, :, 0]
+        squeeze_back = True
+    elif x.dim() == 2:
+        x2 = x
+    else:
+        raise ValueError(f"Expected 2D input tensor (batch, dim), got {x.dim()}D")
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"Unsupported input dtype {x.dtype}; expected float32, bfloat16 or float16")
+    if conv_state.dim() != 3:
+        raise ValueError(f"Expected 3D conv_state tensor (batch, dim, state_len), got {conv_state.dim()}D")
+    batch, dim = x2.shape
+    if tuple(conv_state.shape[:2]) != (batch, dim):
+        raise ValueError(
+            f"Input shape {tuple(x2.shape)} doesn't match conv_state batch/dim {tuple(conv_state.shape[:2])}")
+    if conv_state.dtype != x.dtype or conv_state.device != x.device:
+        raise ValueError("conv_state must have the dtype and device of x")
+    _check_shapes(dim, weight, bias)
+    _require_gpu(x, "Input tensor")
+    _check_devices(weight, bias, x.device)
+    if conv_state.shape[2] < weight.shape[1] - 1:
+        raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
+    _no_grad_needed(x, weight, bias, conv_state)
+    bias = _prep_bias(weight, bias)
+    if token_mask is not None:
+        if token_mask.dim() != 1 or token_mask.shape[0] != batch:
+            raise ValueError(f"token_mask shape {tuple(token_mask.shape)} does not match (batch,) = ({batch},)")
+        if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x.device:
+            raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
+
+    out = torch.empty((batch, dim), dtype=x.dtype, device=x.device)
+    if out.numel():
+        p = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().canon_conv1d_update(ctypes.byref(p), _stream(x.device))
+        _lib.check(rc, "causal_conv1d_update")
+    return out.unsqueeze(-1) if squeeze_back else out
+
+
+# ---------------------------------------------------------------------------
+# The reference's fused (batch, seqlen, dim) API, same argument meaning.
+# ---------------------------------------------------------------------------
+def short_conv_fused(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+    activation: bool = True,
+    residual: bool = True,
+) -> torch.Tensor:
+    """``x`` (batch, seqlen, dim) -> ``(x if residual) + act(conv(x * mask) + bias)``.
+
+    Same contract as ``causal_conv1d_mps.short_conv_fused``
+    (``causal_conv1d_mps/__init__.py:154-301``, kernel
+    ``causal_conv1d.metal:530-580``): the mask multiplies the conv inputs, the
+    residual term is the unmasked ``x``.
+    """
+    if x.dim() != 3:
+        raise ValueError(f"Expected 3D input tensor (batch, seqlen, dim), got {x.dim()}D")
+    y = causal_conv1d_fn(
+        x.transpose(1, 2), weight, bias, activation="silu" if activation else None,
+        attention_mask=attention_mask, residual="unmasked" if residual else False)
+    return y.transpose(1, 2)
+
+
+def short_conv_update(
+    x: torch.Tensor,
+    conv_state: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    cache_seqlens: Optional[torch.Tensor] = None,
+    activation: bool = True,
+    residual: bool = True,
+) -> torch.Tensor:
+    """Single-token step with the argument order of
+    ``causal_conv1d_mps.short_conv_update`` (``causal_conv1d_mps/__init__.py:304-419``).
+
+    The state is a shift register (newest token last), the layout the prefill
+    path and the eager step (``model/model.py:385-386``) use; the reference's
+    Metal kernel instead indexes it as a ring through ``cache_seqlens``
+    (``causal_conv1d.metal:755-775``), which is not reproduced: passing
+    ``cache_seqlens`` raises.
+    """
+    if cache_seqlens is not None:
+        raise NotImplementedError("cache_seqlens (ring-buffer conv_state) is not supported; the state is a shift register")
+    return causal_conv1d_update(x, conv_state, weight, bias, activation="silu" if activation else None,
+                                residual="masked" if residual else False)
+
+
+# ---------------------------------------------------------------------------
+# introspection (lets callers and tests assert that a layout takes a fast path)
+# ---------------------------------------------------------------------------
+def kernel_plan_fwd(x, weight, bias=None, activation=None, attention_mask=None, residual=False,
+                    rounding="fused", initial_states=None, final_states_out=None) -> str:
+    """Kernel family ``causal_conv1d_fn`` would launch: 'bcl_vec', 'blc_vec' or 'generic'."""
+    out = torch.empty_like(x)
+    p = _fill_fwd(x, out, weight, _prep_bias(weight, bias), attention_mask, initial_states, final_states_out,
+                  _activation_flag(activation), _residual_mode(residual), _round_mode(rounding))
+    name = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(p))
+    if name is None:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_fwd")
+    return name.decode()
+
+
+def kernel_plan_update(x, conv_state, weight, bias=None, activation=None, residual=False, rounding="fused") -> str:
+    """Kernel family ``causal_conv1d_update`` would launch: 'update_vec' or 'update_generic'."""
+    out = torch.empty_like(x)
+    p = _fill_update(x, out, conv_state, weight, _prep_bias(weight, bias), None,
+                     _activation_flag(activation), _residual_mode(residual), _round_mode(rounding))
+    name = _lib.lib().canon_conv1d_update_plan(ctypes.byref(p))
+    if name is None:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_update")
+    return name.decode()

@@ -1,0 +1,1076 @@
+// Canon causal depthwise conv1d for MI355X (gfx950, wave64): prefill and
+// single-token decode update, behind the C ABI of include/canon_conv1d.h.
+//
+// The op is a width-<=4 FIR per (batch, channel) row: ~2 flop per byte moved,
+// so every kernel here is organised around HBM traffic, not arithmetic:
+//   * one 16-byte load and one 16-byte store per lane per vector, each element
+//     of x read from HBM once and each element of out written once;
+//   * the (W-1)-element history a vector needs comes from the neighbouring
+//     lane (DPP wave shift) or from the previous vector of the same wave held
+//     in registers; only the first lane of a row segment touches memory for it;
+//   * taps and bias live in registers; bias, SiLU, mask multiply, residual and
+//     the conv-state capture are fused into the same pass.
+//
+// Arithmetic contract (shared with the CPU oracle used by the tests):
+//     acc = bias;  for k in 0..W-1: acc = fmaf(w[k], xm[t-(W-1)+k], acc)
+// taps/bias rounded to the storage type of x first; one rounding at the store.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "canon_conv1d.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// storage types
+// ---------------------------------------------------------------------------
+template <int DT> struct Elem;
+template <> struct Elem<CANON_DTYPE_F32> { static constexpr int bytes = 4; static constexpr int per_vec = 4; };
+template <> struct Elem<CANON_DTYPE_BF16> { static constexpr int bytes = 2; static constexpr int per_vec = 8; };
+template <> struct Elem<CANON_DTYPE_F16> { static constexpr int bytes = 2; static constexpr int per_vec = 8; };
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f_bits(float f) { return __float_as_uint(f); }
+
+// two packed 16-bit values -> two floats
+template <int DT> __device__ __forceinline__ void unpack2(uint32_t u, float &lo, float &hi)
+{
+    if constexpr (DT == CANON_DTYPE_BF16) {
+        lo = bits_f(u << 16);
+        hi = bits_f(u & 0xFFFF0000u);
+    } else {
+        f16x2_t h = __builtin_bit_cast(f16x2_t, u);
+        lo = (float)h.x;
+        hi = (float)h.y;
+    }
+}
+
+// two floats -> two packed 16-bit values, round to nearest even
+template <int DT> __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+    float2_t v = {lo, hi};
+    if constexpr (DT == CANON_DTYPE_BF16) {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    } else {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    }
+}
+
+// value -> storage type -> value
+template <int DT> __device__ __forceinline__ float round_through(float v)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        return v;
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        return (float)(__bf16)v;
+    } else {
+        return (float)(_Float16)v;
+    }
+}
+
+template <int DT> __device__ __forceinline__ void unpack_vec(const uint4 &v, float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        f[0] = bits_f(v.x); f[1] = bits_f(v.y); f[2] = bits_f(v.z); f[3] = bits_f(v.w);
+    } else {
+        unpack2<DT>(v.x, f[0], f[1]);
+        unpack2<DT>(v.y, f[2], f[3]);
+        unpack2<DT>(v.z, f[4], f[5]);
+        unpack2<DT>(v.w, f[6], f[7]);
+    }
+}
+
+template <int DT> __device__ __forceinline__ uint4 pack_vec(const float *f)
+{
+    uint4 v;
+    if constexpr (DT == CANON_DTYPE_F32) {
+        v.x = f_bits(f[0]); v.y = f_bits(f[1]); v.z = f_bits(f[2]); v.w = f_bits(f[3]);
+    } else {
+        v.x = pack2<DT>(f[0], f[1]);
+        v.y = pack2<DT>(f[2], f[3]);
+        v.z = pack2<DT>(f[4], f[5]);
+        v.w = pack2<DT>(f[6], f[7]);
+    }
+    return v;
+}
+
+template <int DT> __device__ __forceinline__ float load1(const void *p, int64_t i)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        return ((const float *)p)[i];
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        return bits_f((uint32_t)((const uint16_t *)p)[i] << 16);
+    } else {
+        return (float)((const _Float16 *)p)[i];
+    }
+}
+
+template <int DT> __device__ __forceinline__ void store1(void *p, int64_t i, float v)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        ((float *)p)[i] = v;
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        ((__bf16 *)p)[i] = (__bf16)v;
+    } else {
+        ((_Float16 *)p)[i] = (_Float16)v;
+    }
+}
+
+// weight / bias element of run-time type
+__device__ __forceinline__ float load_w(const void *p, int64_t i, int dt)
+{
+    if (dt == CANON_DTYPE_F32) return load1<CANON_DTYPE_F32>(p, i);
+    if (dt == CANON_DTYPE_BF16) return load1<CANON_DTYPE_BF16>(p, i);
+    return load1<CANON_DTYPE_F16>(p, i);
+}
+
+__device__ __forceinline__ float load_mask(const void *p, int64_t i, int dt)
+{
+    switch (dt) {
+    case CANON_MASK_U8: return (float)((const uint8_t *)p)[i];
+    case CANON_MASK_I32: return (float)((const int32_t *)p)[i];
+    case CANON_MASK_I64: return (float)((const int64_t *)p)[i];
+    case CANON_MASK_F32: return ((const float *)p)[i];
+    case CANON_MASK_BF16: return load1<CANON_DTYPE_BF16>(p, i);
+    default: return load1<CANON_DTYPE_F16>(p, i);
+    }
+}
+
+__device__ __forceinline__ float silu_fast(float v)
+{
+    // v / (1 + e^-v); v_exp_f32 and v_rcp_f32 are each good to 1 ulp
+    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+}
+
+__device__ __forceinline__ float silu_precise(float v) { return v / (1.0f + expf(-v)); }
+
+// lane i <- lane i-1 across the whole wave; lane 0 <- `first`
+__device__ __forceinline__ float wave_shift_up(float v, float first)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_update_dpp((int)f_bits(first), (int)f_bits(v),
+                                                        0x138 /* wave_shr:1 */, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float read_lane63(float v)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), 63));
+}
+
+// ---------------------------------------------------------------------------
+// kernel argument blocks (device copies of the validated ABI structs)
+// ---------------------------------------------------------------------------
+struct FwdArgs {
+    const char *x;
+    char *out;
+    const void *weight;
+    const void *bias;
+    const void *mask;
+    const void *init;
+    void *fin;
+    int64_t x_sb, x_sc, x_sl;
+    int64_t o_sb, o_sc, o_sl;
+    int64_t w_sc, w_sk;
+    int64_t m_sb, m_sl;
+    int64_t i_sb, i_sc, i_ss;
+    int64_t f_sb, f_sc, f_ss;
+    uint32_t B, C, L;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec;
+    // launch geometry
+    uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
+    uint32_t nseg;      // bcl: segments per row       blc: time chunks per sequence
+    uint32_t chunk;     // blc/generic: time steps per chunk
+    uint32_t ntasks;    // bcl: wave tasks             blc/generic: threads
+    uint32_t nblocks;   // logical blocks (grid may be padded to a multiple of 8)
+};
+
+struct UpdArgs {
+    const char *x;
+    char *out;
+    char *state;
+    const void *weight;
+    const void *bias;
+    const void *tmask;
+    int64_t x_sb, x_sc, o_sb, o_sc;
+    int64_t s_sb, s_sc, s_ss;
+    int64_t w_sc, w_sk;
+    int64_t m_sb;
+    uint32_t B, C;
+    int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec;
+    uint32_t nvec;      // channel vectors per batch row
+    uint32_t bgroups;   // batch groups (each thread walks NB batch rows)
+    uint32_t nthreads;
+};
+
+// Blocks are dealt round-robin to the 8 XCDs, each with its own L2.  Give XCD k
+// the k-th contiguous eighth of the logical blocks, so blocks that are
+// neighbours in memory (and share halo rows) share an L2.
+__device__ __forceinline__ uint32_t xcd_block(uint32_t nblocks)
+{
+    const uint32_t per = (nblocks + 7u) >> 3;
+    return (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+}
+
+// The activated, residual-added output of one element (fused rounding mode).
+__device__ __forceinline__ float finish(float acc, int act, int res_mode, float xm, float xr)
+{
+    if (act) acc = silu_fast(acc);
+    if (res_mode == CANON_RESIDUAL_MASKED) acc += xm;
+    else if (res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
+    return acc;
+}
+
+// Write final_state[b, c, :] for one row from global memory (the row was just
+// streamed by this wave, so these are cache hits).  One lane per slot.
+template <int DT>
+__device__ __forceinline__ void capture_row_state(const FwdArgs &a, uint32_t b, uint32_t c, int slot)
+{
+    if (slot >= a.S_out) return;
+    const int64_t t = (int64_t)a.L - a.S_out + slot;
+    float v = 0.0f;
+    if (t >= 0) {
+        v = load1<DT>(a.x, b * a.x_sb + c * a.x_sc + t * a.x_sl);
+        if (a.mask) v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+    } else if (a.init && a.S_in + t >= 0) {
+        v = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+    }
+    store1<DT>(a.fin, b * a.f_sb + c * a.f_sc + slot * a.f_ss, v);
+}
+
+// ---------------------------------------------------------------------------
+// prefill, time-contiguous rows ([B, C, L], x_stride_l == 1)
+//
+// One wave owns one segment of one (b, c) row: U vectors per lane, lane l of
+// step u holding elements [(seg*U + u)*64 + l] * E .. +E.  All U loads are
+// issued before any arithmetic.  The three elements before a vector come from
+// lane l-1 (wave shift), for lane 0 from lane 63 of the previous step, and for
+// the very first vector of the segment from memory / the initial state / zero.
+// ---------------------------------------------------------------------------
+template <int DT, int W, int U>
+__global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t task = blockIdx.x * 4u + wave;
+    if (task >= a.ntasks) return;
+    const uint32_t row = task / a.nseg;
+    const uint32_t seg = task - row * a.nseg;
+    const uint32_t b = row / a.C;
+    const uint32_t c = row - b * a.C;
+
+    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
+    char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
+    const uint32_t v0 = seg * (64u * U) + lane;
+
+    uint4 X[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        X[u] = make_uint4(0, 0, 0, 0);
+        if (v < a.nvec) X[u] = *(const uint4 *)(xrow + (int64_t)v * 16);
+    }
+
+    float w[W];
+#pragma unroll
+    for (int k = 0; k < W; ++k)
+        w[k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
+    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+
+    // history of the segment's first vector (only lane 0's copy is consumed)
+    float carry[3] = {0.0f, 0.0f, 0.0f};
+    if (lane == 0) {
+        if (seg > 0) {
+            const int64_t t0 = (int64_t)v0 * E;
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float v = load1<DT>(xrow, t0 - 3 + j);
+                if (a.mask)
+                    v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + (t0 - 3 + j) * a.m_sl, a.mask_dtype));
+                carry[j] = v;
+            }
+        } else if (a.init) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                if (j >= 3 - (W - 1))
+                    carry[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+        }
+    }
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        float xr[E], xm[E];
+        unpack_vec<DT>(X[u], xr);
+        if (a.mask && v < a.nvec) {
+            const int64_t mbase = b * a.m_sb + (int64_t)v * E * a.m_sl;
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+                xm[j] = round_through<DT>(xr[j] * load_mask(a.mask, mbase + j * a.m_sl, a.mask_dtype));
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j) xm[j] = xr[j];
+        }
+        // seq[0..2] = the three masked inputs before this vector
+        float seq[E + 3];
+        seq[0] = wave_shift_up(xm[E - 3], carry[0]);
+        seq[1] = wave_shift_up(xm[E - 2], carry[1]);
+        seq[2] = wave_shift_up(xm[E - 1], carry[2]);
+        if (u + 1 < U) {
+            carry[0] = read_lane63(xm[E - 3]);
+            carry[1] = read_lane63(xm[E - 2]);
+            carry[2] = read_lane63(xm[E - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) seq[3 + j] = xm[j];
+
+        float o[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float acc = bv;
+#pragma unroll
+            for (int k = 0; k < W; ++k) acc = fmaf(w[k], seq[j + (4 - W) + k], acc);
+            o[j] = finish(acc, a.act, a.res_mode, xm[j], xr[j]);
+        }
+        if (v < a.nvec) *(uint4 *)(orow + (int64_t)v * 16) = pack_vec<DT>(o);
+    }
+
+    if (a.fin && seg == a.nseg - 1) capture_row_state<DT>(a, b, c, lane);
+}
+
+// ---------------------------------------------------------------------------
+// prefill, channel-contiguous rows ([B, L, C] memory, x_stride_c == 1): the
+// layout CanonLayer hands over (a transposed view of [B, T, D]).
+//
+// One lane owns E adjacent channels and walks `chunk` time steps, keeping the
+// three previous (masked) rows in registers; a wave's loads are contiguous
+// 1 KB row pieces.  Rows are fetched R at a time so R loads are in flight.
+// ---------------------------------------------------------------------------
+// Taps and bias of E adjacent channels, rounded to the storage type of x.
+// `vec` (decided on the host): weight is a contiguous, 16-byte aligned [C, 4].
+template <int DT, int W>
+__device__ __forceinline__ void load_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
+                                          int w_dtype, bool vec, uint32_t c0, float (*w)[W], float *bv)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    if (W == 4 && vec) {
+        if (w_dtype == CANON_DTYPE_F32) {
+            const uint4 *p = (const uint4 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const uint4 q = p[e];
+                w[e][0] = round_through<DT>(bits_f(q.x));
+                w[e][1] = round_through<DT>(bits_f(q.y));
+                w[e][W - 2] = round_through<DT>(bits_f(q.z));
+                w[e][W - 1] = round_through<DT>(bits_f(q.w));
+            }
+        } else {
+            const uint2 *p = (const uint2 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const uint2 q = p[e];
+                float t0, t1, t2, t3;
+                if (w_dtype == CANON_DTYPE_BF16) {
+                    unpack2<CANON_DTYPE_BF16>(q.x, t0, t1);
+                    unpack2<CANON_DTYPE_BF16>(q.y, t2, t3);
+                } else {
+                    unpack2<CANON_DTYPE_F16>(q.x, t0, t1);
+                    unpack2<CANON_DTYPE_F16>(q.y, t2, t3);
+                }
+                w[e][0] = round_through<DT>(t0);
+                w[e][1] = round_through<DT>(t1);
+                w[e][W - 2] = round_through<DT>(t2);
+                w[e][W - 1] = round_through<DT>(t3);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+#pragma unroll
+            for (int k = 0; k < W; ++k)
+                w[e][k] = round_through<DT>(load_w(weight, (int64_t)(c0 + e) * w_sc + k * w_sk, w_dtype));
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) bv[e] = bias ? round_through<DT>(load_w(bias, c0 + e, w_dtype)) : 0.0f;
+}
+
+template <int DT, int W, int R>
+__global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    const uint32_t blk = xcd_block(a.nblocks);
+    if (blk >= a.nblocks) return;
+    const uint32_t tid = blk * 256u + threadIdx.x;
+    if (tid >= a.ntasks) return;
+    const uint32_t cv = tid % a.nvec;
+    const uint32_t bc = tid / a.nvec;
+    const uint32_t ch = bc % a.nseg;
+    const uint32_t b = bc / a.nseg;
+    const uint32_t c0 = cv * E;
+
+    float w[E][W], bias[E];
+    load_taps<DT, W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, w, bias);
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * Elem<DT>::bytes;
+    char *ob = a.out + ((int64_t)b * a.o_sb + c0) * Elem<DT>::bytes;
+    const int64_t xs = a.x_sl * Elem<DT>::bytes, os = a.o_sl * Elem<DT>::bytes;
+    const int64_t t_begin = (int64_t)ch * a.chunk;
+    const int64_t t_stop = t_begin + (int64_t)a.chunk;
+    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+
+    // hist[j] = masked row t_begin - 3 + j
+    float hist[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int64_t t = t_begin - 3 + j;
+#pragma unroll
+        for (int e = 0; e < E; ++e) hist[j][e] = 0.0f;
+        if (j < 3 - (W - 1)) continue;
+        if (t >= 0) {
+            const uint4 v = *(const uint4 *)(xb + t * xs);
+            unpack_vec<DT>(v, hist[j]);
+            if (a.mask) {
+                const float m = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+#pragma unroll
+                for (int e = 0; e < E; ++e) hist[j][e] = round_through<DT>(hist[j][e] * m);
+            }
+        } else if (a.init && a.S_in + t >= 0) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
+        }
+    }
+
+    for (int64_t t = t_begin; t < t_end; t += R) {
+        uint4 X[R];
+        float m[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            X[r] = make_uint4(0, 0, 0, 0);
+            m[r] = 1.0f;
+            if (t + r < t_end) {
+                X[r] = *(const uint4 *)(xb + (t + r) * xs);
+                if (a.mask) m[r] = load_mask(a.mask, b * a.m_sb + (t + r) * a.m_sl, a.mask_dtype);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (t + r < t_end) {
+                float xr[E], xm[E], o[E];
+                unpack_vec<DT>(X[r], xr);
+#pragma unroll
+                for (int e = 0; e < E; ++e) xm[e] = a.mask ? round_through<DT>(xr[e] * m[r]) : xr[e];
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    float acc = bias[e];
+                    if constexpr (W == 4) acc = fmaf(w[e][0], hist[0][e], acc);
+                    if constexpr (W >= 3) acc = fmaf(w[e][W - 3], hist[1][e], acc);
+                    acc = fmaf(w[e][W - 2], hist[2][e], acc);
+                    acc = fmaf(w[e][W - 1], xm[e], acc);
+                    o[e] = finish(acc, a.act, a.res_mode, xm[e], xr[e]);
+                    hist[0][e] = hist[1][e];
+                    hist[1][e] = hist[2][e];
+                    hist[2][e] = xm[e];
+                }
+                *(uint4 *)(ob + (t + r) * os) = pack_vec<DT>(o);
+            }
+        }
+    }
+
+    if (a.fin && ch == a.nseg - 1) {
+        for (int slot = 0; slot < a.S_out; ++slot) {
+            const int64_t t = (int64_t)a.L - a.S_out + slot;
+            float v[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = 0.0f;
+            if (t >= 0) {
+                unpack_vec<DT>(*(const uint4 *)(xb + t * xs), v);
+                if (a.mask) {
+                    const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[e] = round_through<DT>(v[e] * mm);
+                }
+            } else if (a.init && a.S_in + t >= 0) {
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    v[e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                store1<DT>(a.fin, b * a.f_sb + (int64_t)(c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// prefill, any strides / any length / either rounding mode: one thread per
+// (b, c, chunk of time steps), scalar accesses.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.ntasks) return;
+    // fastest-varying index follows the contiguous dimension of x
+    uint32_t b, c, ch;
+    if (a.x_sc == 1 && a.x_sl != 1) {
+        c = tid % a.C;
+        const uint32_t r = tid / a.C;
+        ch = r % a.nseg;
+        b = r / a.nseg;
+    } else {
+        ch = tid % a.nseg;
+        const uint32_t r = tid / a.nseg;
+        c = r % a.C;
+        b = r / a.C;
+    }
+    const int W = a.W;
+    float w[4] = {0, 0, 0, 0};
+    for (int k = 0; k < W; ++k)
+        w[4 - W + k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
+    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+
+    const int64_t xo = (int64_t)b * a.x_sb + (int64_t)c * a.x_sc;
+    const int64_t oo = (int64_t)b * a.o_sb + (int64_t)c * a.o_sc;
+    const int64_t t_begin = (int64_t)ch * a.chunk;
+    const int64_t t_stop = t_begin + (int64_t)a.chunk;
+    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+
+    float h[3] = {0, 0, 0};
+    for (int j = 4 - W; j < 3; ++j) {
+        const int64_t t = t_begin - 3 + j;
+        if (t >= 0) {
+            float v = load1<DT>(a.x, xo + t * a.x_sl);
+            if (a.mask) v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            h[j] = v;
+        } else if (a.init && a.S_in + t >= 0) {
+            h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+        }
+    }
+    for (int64_t t = t_begin; t < t_end; ++t) {
+        const float xr = load1<DT>(a.x, xo + t * a.x_sl);
+        float xm = xr;
+        if (a.mask) xm = round_through<DT>(xr * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+        float acc = bv;
+        if (W == 4) acc = fmaf(w[0], h[0], acc);
+        if (W >= 3) acc = fmaf(w[1], h[1], acc);
+        acc = fmaf(w[2], h[2], acc);
+        acc = fmaf(w[3], xm, acc);
+        if (a.eager) {
+            acc = round_through<DT>(acc);
+            if (a.act) acc = round_through<DT>(silu_precise(acc));
+            if (a.res_mode == CANON_RESIDUAL_MASKED) acc += xm;
+            else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
+        } else {
+            acc = finish(acc, a.act, a.res_mode, xm, xr);
+        }
+        store1<DT>(a.out, oo + t * a.o_sl, acc);
+        h[0] = h[1];
+        h[1] = h[2];
+        h[2] = xm;
+    }
+    if (a.fin && ch == a.nseg - 1)
+        for (int slot = 0; slot < a.S_out; ++slot) capture_row_state<DT>(a, b, c, slot);
+}
+
+// ---------------------------------------------------------------------------
+// decode update, vectorised: contiguous [B, C, S] state, channel-contiguous
+// x / out.  One lane owns E adjacent channels: it reads the E*S state
+// elements as S 16-byte vectors (they are one contiguous 16*S-byte run),
+// computes E outputs, and writes the run back shifted by one element per
+// channel with the new token in the last slot -- one fused gather / shift /
+// write, no second pass.  Each lane walks NB batch rows so the taps are
+// fetched once per NB tokens.
+// ---------------------------------------------------------------------------
+template <int DT> struct StateRun {
+    // element i of a run of uint4 vectors, as raw bits of the storage type
+    static __device__ __forceinline__ uint32_t get(const uint4 *v, int i)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) {
+            const uint4 &q = v[i >> 2];
+            const int d = i & 3;
+            return d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+        } else {
+            const uint4 &q = v[i >> 3];
+            const int d = (i >> 1) & 3;
+            const uint32_t u = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
+            return (i & 1) ? (u >> 16) : (u & 0xFFFFu);
+        }
+    }
+    static __device__ __forceinline__ float as_float(uint32_t raw)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return bits_f(raw);
+        else if constexpr (DT == CANON_DTYPE_BF16) return bits_f(raw << 16);
+        else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+    }
+    static __device__ __forceinline__ uint32_t raw_of(float f)   // exact for values already representable
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return f_bits(f);
+        else if constexpr (DT == CANON_DTYPE_BF16) return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+        else return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+};
+
+template <int DT, int W, int S, int NB>
+__global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    constexpr int BY = Elem<DT>::bytes;
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.nthreads) return;
+    const uint32_t cv = tid % a.nvec;
+    const uint32_t bg = tid / a.nvec;
+    const uint32_t c0 = cv * E;
+
+    float w[E][W], bias[E];
+    load_taps<DT, W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, w, bias);
+
+    uint4 X[NB];
+    uint4 ST[NB][S];
+    float tm[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) {
+        const uint32_t b = bg * NB + n;
+        tm[n] = 1.0f;
+        if (b < a.B) {
+            X[n] = *(const uint4 *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
+            const uint4 *sp = (const uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
+#pragma unroll
+            for (int k = 0; k < S; ++k) ST[n][k] = sp[k];
+            if (a.tmask) tm[n] = load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype);
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < NB; ++n) {
+        const uint32_t b = bg * NB + n;
+        if (b >= a.B) continue;
+        float xr[E], xt[E], o[E];
+        unpack_vec<DT>(X[n], xr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) xt[e] = a.tmask ? round_through<DT>(xr[e] * tm[n]) : xr[e];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float acc = bias[e];
+#pragma unroll
+            for (int k = 0; k < W - 1; ++k)
+                acc = fmaf(w[e][k], StateRun<DT>::as_float(StateRun<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
+            acc = fmaf(w[e][W - 1], xt[e], acc);
+            o[e] = finish(acc, a.act, a.res_mode, xt[e], xr[e]);
+        }
+        *(uint4 *)(a.out + ((int64_t)b * a.o_sb + c0) * BY) = pack_vec<DT>(o);
+
+        // new run: element (e, k) <- old (e, k+1); (e, S-1) <- token
+        uint32_t raw[E * S];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < S - 1; ++k) raw[e * S + k] = StateRun<DT>::get(ST[n], e * S + k + 1);
+            raw[e * S + S - 1] = a.tmask ? StateRun<DT>::raw_of(xt[e]) : StateRun<DT>::get(&X[n], e);
+        }
+        uint4 *dp = (uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
+#pragma unroll
+        for (int k = 0; k < S; ++k) {
+            uint4 q;
+            if constexpr (DT == CANON_DTYPE_F32) {
+                q.x = raw[4 * k]; q.y = raw[4 * k + 1]; q.z = raw[4 * k + 2]; q.w = raw[4 * k + 3];
+            } else {
+                q.x = raw[8 * k] | (raw[8 * k + 1] << 16);
+                q.y = raw[8 * k + 2] | (raw[8 * k + 3] << 16);
+                q.z = raw[8 * k + 4] | (raw[8 * k + 5] << 16);
+                q.w = raw[8 * k + 6] | (raw[8 * k + 7] << 16);
+            }
+            dp[k] = q;
+        }
+    }
+}
+
+// decode update, any strides / state length / rounding mode: one thread per (b, c)
+template <int DT>
+__global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs a)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.nthreads) return;
+    const uint32_t c = tid % a.C;
+    const uint32_t b = tid / a.C;
+    const int W = a.W, S = a.S;
+    float w[4] = {0, 0, 0, 0}, win[4] = {0, 0, 0, 0};
+    for (int k = 0; k < W; ++k)
+        w[4 - W + k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
+    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+    const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
+    const float xr = load1<DT>(a.x, (int64_t)b * a.x_sb + (int64_t)c * a.x_sc);
+    float xt = xr;
+    if (a.tmask) xt = round_through<DT>(xr * load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype));
+    for (int k = 0; k < W - 1; ++k) win[4 - W + k] = load1<DT>(a.state, so + (int64_t)(S - (W - 1) + k) * a.s_ss);
+    win[3] = xt;
+    float acc;
+    if (!a.eager) {
+        acc = bv;
+        if (W == 4) acc = fmaf(w[0], win[0], acc);
+        if (W >= 3) acc = fmaf(w[1], win[1], acc);
+        acc = fmaf(w[2], win[2], acc);
+        acc = fmaf(w[3], win[3], acc);
+        acc = finish(acc, a.act, a.res_mode, xt, xr);
+    } else {
+        float s = 0.0f;
+        for (int k = 4 - W; k < 4; ++k) s = __fadd_rn(s, round_through<DT>(__fmul_rn(win[k], w[k])));
+        s = round_through<DT>(s);
+        acc = round_through<DT>(__fadd_rn(bv, s));
+        if (a.act) acc = round_through<DT>(silu_precise(acc));
+        if (a.res_mode == CANON_RESIDUAL_MASKED) acc = __fadd_rn(acc, xt);
+        else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc = __fadd_rn(acc, xr);
+    }
+    store1<DT>(a.out, (int64_t)b * a.o_sb + (int64_t)c * a.o_sc, acc);
+    // shift left by one (ascending order: each slot is read before it is overwritten)
+    for (int k = 0; k < S - 1; ++k) {
+        if constexpr (DT == CANON_DTYPE_F32)
+            ((uint32_t *)a.state)[so + k * a.s_ss] = ((const uint32_t *)a.state)[so + (k + 1) * a.s_ss];
+        else
+            ((uint16_t *)a.state)[so + k * a.s_ss] = ((const uint16_t *)a.state)[so + (k + 1) * a.s_ss];
+    }
+    store1<DT>(a.state, so + (int64_t)(S - 1) * a.s_ss, xt);
+}
+
+// ---------------------------------------------------------------------------
+// host side: validation, planning, launch
+// ---------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool valid_dtype(int d) { return d == CANON_DTYPE_F32 || d == CANON_DTYPE_BF16 || d == CANON_DTYPE_F16; }
+bool valid_mask_dtype(int d) { return d >= CANON_MASK_U8 && d <= CANON_MASK_F16; }
+int elem_bytes(int d) { return d == CANON_DTYPE_F32 ? 4 : 2; }
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
+enum UpdKind { UPD_VEC, UPD_GENERIC };
+
+constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
+constexpr int kBlcRows = 8;             // rows in flight per lane in the channel-contiguous kernel
+constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update
+
+struct FwdPlan {
+    FwdKind kind;
+    int U;
+    FwdArgs args;
+    uint32_t grid;
+};
+
+int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_fwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_fwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_fwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->round_mode != CANON_ROUND_FUSED && p->round_mode != CANON_ROUND_EAGER)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
+    if (p->batch < 0 || p->channels < 0 || p->seqlen < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld, seqlen %lld)",
+                    (long long)p->batch, (long long)p->channels, (long long)p->seqlen);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->seqlen >= (1ll << 31) ||
+        p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
+    if (!empty) {
+        if (!p->x || !p->out || !p->weight) return fail(CANON_ERR_INVALID_ARGUMENT, "x, out and weight must not be NULL");
+        if (p->x == p->out) return fail(CANON_ERR_INVALID_ARGUMENT, "out must not alias x");
+    }
+    if (p->mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    if (p->initial_state && p->initial_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "initial_len %d is shorter than width-1 = %d", p->initial_len, p->width - 1);
+    if (p->final_state && p->final_len < 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "final_len %d must be at least 1", p->final_len);
+    if (p->final_state && p->final_len > 64)
+        return fail(CANON_ERR_UNSUPPORTED, "final_len %d above 64 is not supported", p->final_len);
+
+    FwdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.out = (char *)p->out;
+    a.weight = p->weight; a.bias = p->bias; a.mask = p->mask;
+    a.init = p->initial_state; a.fin = p->final_state;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.x_sl = p->x_stride_l;
+    a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c; a.o_sl = p->out_stride_l;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
+    a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
+    a.i_sb = p->init_stride_b; a.i_sc = p->init_stride_c; a.i_ss = p->init_stride_s;
+    a.f_sb = p->final_stride_b; a.f_sc = p->final_stride_c; a.f_ss = p->final_stride_s;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
+    a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
+    a.S_in = p->initial_state ? p->initial_len : 0;
+    a.S_out = p->final_state ? p->final_len : 0;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    plan->U = 1;
+    plan->grid = 0;
+    plan->kind = FWD_GENERIC;
+    if (empty) return CANON_OK;
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const uint64_t rows = (uint64_t)a.B * a.C;
+    const bool fused = p->round_mode == CANON_ROUND_FUSED;
+    const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
+    const bool bcl_ok = fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
+                        a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0 &&
+                        a.L / E >= 16;
+    const bool blc_ok = fused && ptr_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 &&
+                        a.x_sb % E == 0 && a.x_sl % E == 0 && a.o_sb % E == 0 && a.o_sl % E == 0 &&
+                        a.x_sl != 1;
+
+    if (bcl_ok) {
+        const uint32_t nvec = a.L / E;
+        // vectors per lane: as many as keep >= 2048 waves in flight, at most 4
+        int U = 1;
+        for (int cand = 2; cand <= 4; cand *= 2) {
+            const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
+            if (nvec >= 64u * cand && rows * nseg >= 2048) U = cand;
+        }
+        const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
+        const uint64_t ntasks = rows * nseg;
+        if (ntasks < (1ull << 31)) {
+            plan->kind = FWD_BCL;
+            plan->U = U;
+            a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
+            a.nblocks = (uint32_t)((ntasks + 3) / 4);
+            plan->grid = a.nblocks;
+            return CANON_OK;
+        }
+    }
+    if (blc_ok) {
+        const uint32_t nvec = a.C / E;
+        // time steps per lane: a multiple of the rows-in-flight count, sized so
+        // that the launch has about 8 waves per CU
+        const uint64_t lanes_per_step = (uint64_t)a.B * nvec;
+        uint64_t want_chunks = (256ull * 8 * 64 + lanes_per_step - 1) / lanes_per_step;
+        if (want_chunks < 1) want_chunks = 1;
+        uint32_t chunk = (uint32_t)((a.L + want_chunks - 1) / want_chunks);
+        chunk = ((chunk + kBlcRows - 1) / kBlcRows) * kBlcRows;
+        if (chunk < 2 * kBlcRows) chunk = 2 * kBlcRows;
+        const uint32_t nseg = (a.L + chunk - 1) / chunk;
+        const uint64_t nthreads = lanes_per_step * nseg;
+        if (nthreads < (1ull << 31)) {
+            plan->kind = FWD_BLC;
+            a.nvec = nvec; a.nseg = nseg; a.chunk = chunk; a.ntasks = (uint32_t)nthreads;
+            a.nblocks = (uint32_t)((nthreads + 255) / 256);
+            plan->grid = ((a.nblocks + 7) / 8) * 8;
+            return CANON_OK;
+        }
+    }
+    {
+        const uint32_t nseg = (a.L + kGenericChunk - 1) / kGenericChunk;
+        const uint64_t nthreads = rows * nseg;
+        if (nthreads >= (1ull << 32))
+            return fail(CANON_ERR_UNSUPPORTED, "problem too large for the strided kernel (%llu threads)",
+                        (unsigned long long)nthreads);
+        plan->kind = FWD_GENERIC;
+        a.nseg = nseg; a.chunk = kGenericChunk; a.ntasks = (uint32_t)nthreads;
+        a.nblocks = (uint32_t)((nthreads + 255) / 256);
+        plan->grid = a.nblocks;
+    }
+    return CANON_OK;
+}
+
+template <int DT, int W> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+{
+    const dim3 g(pl.grid), b(256);
+    switch (pl.U) {
+    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4>), g, b, 0, s, pl.args); break;
+    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1>), g, b, 0, s, pl.args); break;
+    }
+}
+
+template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == FWD_BCL) launch_bcl<DT, W>(pl, s);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+}
+
+template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == FWD_GENERIC) {
+        hipLaunchKernelGGL((canon_fwd_generic_kernel<DT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        return;
+    }
+    switch (pl.args.W) {
+    case 2: launch_fwd_w<DT, 2>(pl, s); break;
+    case 3: launch_fwd_w<DT, 3>(pl, s); break;
+    default: launch_fwd_w<DT, 4>(pl, s); break;
+    }
+}
+
+struct UpdPlan {
+    UpdKind kind;
+    UpdArgs args;
+    uint32_t grid;
+};
+
+int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_update_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_update_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_update_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->round_mode != CANON_ROUND_FUSED && p->round_mode != CANON_ROUND_EAGER)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
+    if (p->cache_seqlens) return fail(CANON_ERR_UNSUPPORTED, "cache_seqlens (circular conv_state) is not supported");
+    if (p->conv_state_indices) return fail(CANON_ERR_UNSUPPORTED, "conv_state_indices is not supported");
+    if (p->batch < 0 || p->channels < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld)", (long long)p->batch, (long long)p->channels);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels must be below 2^31");
+    if (p->state_len < 1 || p->state_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_len %d is shorter than width-1 = %d", p->state_len, p->width - 1);
+    const bool empty = p->batch == 0 || p->channels == 0;
+    if (!empty && (!p->x || !p->out || !p->conv_state || !p->weight))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "x, out, conv_state and weight must not be NULL");
+    if (p->token_mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+
+    UpdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.out = (char *)p->out; a.state = (char *)p->conv_state;
+    a.weight = p->weight; a.bias = p->bias; a.tmask = p->token_mask;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c;
+    a.s_sb = p->state_stride_b; a.s_sc = p->state_stride_c; a.s_ss = p->state_stride_s;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k; a.m_sb = p->mask_stride_b;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels;
+    a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    plan->kind = UPD_GENERIC;
+    plan->grid = 0;
+    if (empty) return CANON_OK;
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const int S = p->state_len;
+    const bool vec_ok = p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
+                        aligned16(p->x) && aligned16(p->out) && aligned16(p->conv_state) &&
+                        a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb % E == 0 && a.o_sb % E == 0 &&
+                        a.s_ss == 1 && a.s_sc == S && a.s_sb % E == 0;
+    if (vec_ok) {
+        plan->kind = UPD_VEC;
+        a.nvec = a.C / E;
+        a.bgroups = (a.B + kUpdNB - 1) / kUpdNB;
+        a.nthreads = a.nvec * a.bgroups;
+        plan->grid = (a.nthreads + 255) / 256;
+    } else {
+        a.nthreads = a.B * a.C;
+        plan->grid = (a.nthreads + 255) / 256;
+    }
+    return CANON_OK;
+}
+
+template <int DT, int W> void launch_update_vec_w(const UpdPlan &pl, hipStream_t s)
+{
+    const dim3 g(pl.grid), b(256);
+    switch (pl.args.S) {
+    case 3: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 3, kUpdNB>), g, b, 0, s, pl.args); break;
+    case 4: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 4, kUpdNB>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 8, kUpdNB>), g, b, 0, s, pl.args); break;
+    }
+}
+
+template <int DT> void launch_update(const UpdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == UPD_GENERIC) {
+        hipLaunchKernelGGL((canon_update_generic_kernel<DT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        return;
+    }
+    switch (pl.args.W) {
+    case 2: launch_update_vec_w<DT, 2>(pl, s); break;
+    case 3: launch_update_vec_w<DT, 3>(pl, s); break;
+    default: launch_update_vec_w<DT, 4>(pl, s); break;
+    }
+}
+
+int check_launch(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return CANON_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int canon_conv1d_abi_version(void) { return CANON_CONV1D_ABI_VERSION; }
+
+const char *canon_conv1d_last_error(void) { return g_err; }
+
+int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream)
+{
+    FwdPlan pl;
+    const int rc = plan_fwd(p, &pl);
+    if (rc != CANON_OK) return rc;
+    if (pl.grid == 0) return CANON_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (p->x_dtype) {
+    case CANON_DTYPE_F32: launch_fwd<CANON_DTYPE_F32>(pl, s); break;
+    case CANON_DTYPE_BF16: launch_fwd<CANON_DTYPE_BF16>(pl, s); break;
+    default: launch_fwd<CANON_DTYPE_F16>(pl, s); break;
+    }
+    return check_launch("canon_conv1d_fwd");
+}
+
+int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream)
+{
+    UpdPlan pl;
+    const int rc = plan_update(p, &pl);
+    if (rc != CANON_OK) return rc;
+    if (pl.grid == 0) return CANON_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (p->x_dtype) {
+    case CANON_DTYPE_F32: launch_update<CANON_DTYPE_F32>(pl, s); break;
+    case CANON_DTYPE_BF16: launch_update<CANON_DTYPE_BF16>(pl, s); break;
+    default: launch_update<CANON_DTYPE_F16>(pl, s); break;
+    }
+    return check_launch("canon_conv1d_update");
+}
+
+const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)
+{
+    FwdPlan pl;
+    if (plan_fwd(p, &pl) != CANON_OK) return nullptr;
+    return pl.kind == FWD_BCL ? "bcl_vec" : pl.kind == FWD_BLC ? "blc_vec" : "generic";
+}
+
+const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p)
+{
+    UpdPlan pl;
+    if (plan_update(p, &pl) != CANON_OK) return nullptr;
+    return pl.kind == UPD_VEC ? "update_vec" : "update_generic";
+}
+
+}  // extern "C"

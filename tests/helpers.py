@@ -16,18 +16,21 @@ def ulp_diff(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return (key(a) - key(b)).abs()
 
 
-def assert_parity(got: torch.Tensor, want: torch.Tensor, exact: bool, what: str = "") -> None:
+def assert_parity(got: torch.Tensor, want: torch.Tensor, exact: bool, what: str = "", res=None) -> None:
     """The bar of this repository.
 
     16-bit storage: at most 1 ulp from the fp32-accumulate oracle (bit exact
-    when `exact`).  fp32: bit exact when `exact`, else 1e-5 relative.
+    when `exact`).  fp32: bit exact when `exact`, else 1e-5 relative; when a
+    residual term `res` was added, relative to the larger of the result and
+    that term (the sum can cancel, which no fp32 evaluation order survives).
     """
     got, want = got.detach().cpu(), want.detach().cpu()
     assert got.shape == want.shape and got.dtype == want.dtype, (what, got.shape, want.shape)
     if exact:
         assert torch.equal(bits(got), bits(want)), f"{what}: not bit exact"
     elif got.dtype == torch.float32:
-        err = (got - want).abs() / want.abs().clamp_min(1e-3)
+        scale = want.abs() if res is None else torch.maximum(want.abs(), res.detach().cpu().float().abs())
+        err = (got - want).abs() / scale.clamp_min(1e-3)
         assert err.max().item() <= 1e-5, f"{what}: rel err {err.max().item():.3e} > 1e-5"
     else:
         d = ulp_diff(got, want)

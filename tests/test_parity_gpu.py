@@ -155,7 +155,7 @@ def test_short_conv_fused_reference_case(cc, silu, has_bias):
                                   activation=silu, residual=True)
         want = co.conv1d_fwd(x.transpose(1, 2), w, b, mask=mask, activation="silu" if silu else None,
                              residual="unmasked").transpose(1, 2)
-        assert_parity(got, want, exact=not silu, what=f"fused/{dim}/{seqlen}")
+        assert_parity(got, want, exact=not silu, what=f"fused/{dim}/{seqlen}", res=x)
 
 
 # ---- edge shapes, odd strides, every kernel family --------------------------
@@ -254,7 +254,8 @@ def test_update_variants_vs_oracle(cc):
         if res == "unmasked":
             torch.testing.assert_close(got.cpu().float(), want, rtol=2e-2, atol=2e-2)
         else:
-            assert_parity(got, want, exact=act is None, what=f"update/{dtype}/W{W}/S{S}/{B}x{C}/{res}")
+            assert_parity(got, want, exact=act is None, what=f"update/{dtype}/W{W}/S{S}/{B}x{C}/{res}",
+                          res=xt if res else None)
 
 
 def test_update_residual_exact(cc):
@@ -308,7 +309,7 @@ def test_eager_rounding_matches_eager_module(cc, dtype, act):
                                   residual="masked", rounding="eager", final_states_out=fs)
     got = got.transpose(1, 2)
     assert torch.equal(bits(fs), bits(cache[0]))
-    assert_parity(got, want, exact=(not act and dtype != torch.float32), what="eager mode")
+    assert_parity(got, want, exact=(not act and dtype != torch.float32), what="eager mode", res=x)
     # decode steps in eager mode
     state = fs
     layer = EagerCanon(w, bias, act)
@@ -319,7 +320,7 @@ def test_eager_rounding_matches_eager_module(cc, dtype, act):
                                       activation="silu" if act else None, residual="unmasked",
                                       rounding="eager")
         assert torch.equal(bits(state), bits(cache[0]))
-        assert_parity(got, want, exact=False, what="eager step")
+        assert_parity(got, want, exact=False, what="eager step", res=xt[:, 0])
 
 
 def test_errors_surface(cc):

@@ -75,6 +75,17 @@ template <int DT> __device__ __forceinline__ float round_through(float v)
     }
 }
 
+// x * m rounded to the storage type.  For fp16 the product is hidden from the
+// instruction selector: it would otherwise fuse multiply and conversion into
+// v_fma_mixlo_f16 with a +0 addend, which turns a -0 product into +0, and the
+// captured conv state must carry the bits of x * mask exactly.
+template <int DT> __device__ __forceinline__ float mul_round(float x, float m)
+{
+    float p = x * m;
+    if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(p));
+    return round_through<DT>(p);
+}
+
 template <int DT> __device__ __forceinline__ void unpack_vec(const uint4 &v, float *f)
 {
     if constexpr (DT == CANON_DTYPE_F32) {
@@ -143,6 +154,57 @@ __device__ __forceinline__ float load_mask(const void *p, int64_t i, int dt)
     }
 }
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16-byte access; NT marks streaming data that will not be touched again soon
+template <bool NT> __device__ __forceinline__ uint4 load_vec(const void *p)
+{
+    const u32x4_t *q = (const u32x4_t *)p;
+    u32x4_t v;
+    if constexpr (NT) v = __builtin_nontemporal_load(q);
+    else v = *q;
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint4 &v)
+{
+    const u32x4_t q = {v.x, v.y, v.z, v.w};
+    if constexpr (NT) __builtin_nontemporal_store(q, (u32x4_t *)p);
+    else *(u32x4_t *)p = q;
+}
+
+// N consecutive mask entries; the element-type switch sits outside the loop
+template <int N>
+__device__ __forceinline__ void load_mask_vec(const void *p, int64_t base, int64_t stride, int dt, float *m)
+{
+    switch (dt) {
+    case CANON_MASK_U8:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[base + j * stride];
+        break;
+    case CANON_MASK_I32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[base + j * stride];
+        break;
+    case CANON_MASK_I64:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int64_t *)p)[base + j * stride];
+        break;
+    case CANON_MASK_F32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[base + j * stride];
+        break;
+    case CANON_MASK_BF16:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, base + j * stride);
+        break;
+    default:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, base + j * stride);
+        break;
+    }
+}
+
 __device__ __forceinline__ float silu_fast(float v)
 {
     // v / (1 + e^-v); v_exp_f32 and v_rcp_f32 are each good to 1 ulp
@@ -163,6 +225,17 @@ __device__ __forceinline__ float read_lane63(float v)
     return bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), 63));
 }
 
+// Division by a run-time constant as multiply-high and shifts (set up on the host).
+struct FastDiv {
+    uint32_t d, m, s1, s2;
+};
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
+{
+    const uint32_t t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 // ---------------------------------------------------------------------------
 // kernel argument blocks (device copies of the validated ABI structs)
 // ---------------------------------------------------------------------------
@@ -181,13 +254,14 @@ struct FwdArgs {
     int64_t i_sb, i_sc, i_ss;
     int64_t f_sb, f_sc, f_ss;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_pair, nt;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
     uint32_t nseg;      // bcl: segments per row       blc: time chunks per sequence
     uint32_t chunk;     // blc/generic: time steps per chunk
     uint32_t ntasks;    // bcl: wave tasks             blc/generic: threads
     uint32_t nblocks;   // logical blocks (grid may be padded to a multiple of 8)
+    FastDiv div_nseg, div_C, div_nvec;
 };
 
 struct UpdArgs {
@@ -206,6 +280,7 @@ struct UpdArgs {
     uint32_t nvec;      // channel vectors per batch row
     uint32_t bgroups;   // batch groups (each thread walks NB batch rows)
     uint32_t nthreads;
+    FastDiv div_nvec;
 };
 
 // Blocks are dealt round-robin to the 8 XCDs, each with its own L2.  Give XCD k
@@ -236,11 +311,127 @@ __device__ __forceinline__ void capture_row_state(const FwdArgs &a, uint32_t b, 
     float v = 0.0f;
     if (t >= 0) {
         v = load1<DT>(a.x, b * a.x_sb + c * a.x_sc + t * a.x_sl);
-        if (a.mask) v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+        if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
     } else if (a.init && a.S_in + t >= 0) {
         v = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
     }
     store1<DT>(a.fin, b * a.f_sb + c * a.f_sc + slot * a.f_ss, v);
+}
+
+// Taps and bias of NC adjacent channels, in two phases so that the loads can
+// be issued early and nothing waits on them until the values are needed:
+// fetch_taps() only loads raw bits, decode_taps() converts them (rounded to
+// the storage type of x).  `vec` (decided on the host): weight is a
+// contiguous, 16-byte aligned [C, 4].
+template <int NC> struct RawTaps {
+    uint32_t w[NC][4];   // fp32: one tap per word; 16-bit + vec: two taps per word in w[.][0..1];
+                         // 16-bit scalar path: one tap per word, low half
+    uint32_t b[NC];
+};
+
+template <int W, int NC>
+__device__ __forceinline__ void fetch_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
+                                           int w_dtype, bool vec, uint32_t c0, RawTaps<NC> &r)
+{
+    const bool wide = w_dtype == CANON_DTYPE_F32;
+    if (W == 4 && vec) {
+        if (wide) {
+            const uint4 *p = (const uint4 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < NC; ++e) {
+                const uint4 q = p[e];
+                r.w[e][0] = q.x; r.w[e][1] = q.y; r.w[e][2] = q.z; r.w[e][3] = q.w;
+            }
+        } else {
+            const uint2 *p = (const uint2 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < NC; ++e) {
+                const uint2 q = p[e];
+                r.w[e][0] = q.x; r.w[e][1] = q.y;
+            }
+        }
+    } else if (wide) {
+#pragma unroll
+        for (int e = 0; e < NC; ++e)
+#pragma unroll
+            for (int k = 0; k < W; ++k) r.w[e][k] = ((const uint32_t *)weight)[(int64_t)(c0 + e) * w_sc + k * w_sk];
+    } else {
+#pragma unroll
+        for (int e = 0; e < NC; ++e)
+#pragma unroll
+            for (int k = 0; k < W; ++k) r.w[e][k] = ((const uint16_t *)weight)[(int64_t)(c0 + e) * w_sc + k * w_sk];
+    }
+    if (bias) {
+        if (wide) {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
+        }
+    }
+}
+
+// One channel's taps for a whole wave (c is wave-uniform): shaped so that the
+// common cases become scalar-memory loads.  `pair`: bias may be read as the
+// aligned 32-bit word that contains element c.
+template <int W>
+__device__ __forceinline__ void fetch_taps_uniform(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
+                                                   int w_dtype, bool vec, bool pair, uint32_t c, RawTaps<1> &r)
+{
+    const bool wide = w_dtype == CANON_DTYPE_F32;
+    if (bias && pair) {
+        if (wide) {
+            r.b[0] = ((const uint32_t *)bias)[c];
+        } else {
+            const uint32_t d = ((const uint32_t *)bias)[c >> 1];
+            r.b[0] = (c & 1u) ? (d >> 16) : (d & 0xFFFFu);
+        }
+        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, c, r);
+    } else {
+        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, c, r);
+    }
+}
+
+template <int WDT> __device__ __forceinline__ float half_bits_f(uint32_t raw)
+{
+    if constexpr (WDT == CANON_DTYPE_BF16) return bits_f(raw << 16);
+    else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+}
+
+template <int DT, int WDT, int W, int NC>
+__device__ __forceinline__ void decode_taps_typed(const RawTaps<NC> &r, bool vec, bool has_bias, float (*w)[W], float *bv)
+{
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        if constexpr (WDT == CANON_DTYPE_F32) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) w[e][k] = round_through<DT>(bits_f(r.w[e][k]));
+            bv[e] = has_bias ? round_through<DT>(bits_f(r.b[e])) : 0.0f;
+        } else {
+            if (W == 4 && vec) {
+                float t0, t1, t2, t3;
+                unpack2<WDT>(r.w[e][0], t0, t1);
+                unpack2<WDT>(r.w[e][1], t2, t3);
+                w[e][0] = round_through<DT>(t0);
+                w[e][1] = round_through<DT>(t1);
+                w[e][W - 2] = round_through<DT>(t2);
+                w[e][W - 1] = round_through<DT>(t3);
+            } else {
+#pragma unroll
+                for (int k = 0; k < W; ++k) w[e][k] = round_through<DT>(half_bits_f<WDT>(r.w[e][k]));
+            }
+            bv[e] = has_bias ? round_through<DT>(half_bits_f<WDT>(r.b[e])) : 0.0f;
+        }
+    }
+}
+
+template <int DT, int W, int NC>
+__device__ __forceinline__ void decode_taps(const RawTaps<NC> &r, int w_dtype, bool vec, bool has_bias, float (*w)[W], float *bv)
+{
+    if (w_dtype == CANON_DTYPE_F32) decode_taps_typed<DT, CANON_DTYPE_F32, W, NC>(r, vec, has_bias, w, bv);
+    else if (w_dtype == CANON_DTYPE_BF16) decode_taps_typed<DT, CANON_DTYPE_BF16, W, NC>(r, vec, has_bias, w, bv);
+    else decode_taps_typed<DT, CANON_DTYPE_F16, W, NC>(r, vec, has_bias, w, bv);
 }
 
 // ---------------------------------------------------------------------------
@@ -251,37 +442,45 @@ __device__ __forceinline__ void capture_row_state(const FwdArgs &a, uint32_t b, 
 // issued before any arithmetic.  The three elements before a vector come from
 // lane l-1 (wave shift), for lane 0 from lane 63 of the previous step, and for
 // the very first vector of the segment from memory / the initial state / zero.
+// Everything that does not change per element (activation, residual, mask
+// element type) is branched on once per vector, never per element, so the
+// unmasked path is ~130 VALU instructions per 2 KB row and hides under the
+// memory time.
 // ---------------------------------------------------------------------------
-template <int DT, int W, int U>
+template <int DT, int W, int U, bool MASK, bool NT>
 __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
     const int lane = threadIdx.x & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t task = blockIdx.x * 4u + wave;
+    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
     if (task >= a.ntasks) return;
-    const uint32_t row = task / a.nseg;
-    const uint32_t seg = task - row * a.nseg;
-    const uint32_t b = row / a.C;
+    uint32_t row = task, seg = 0;
+    if (a.nseg > 1) {
+        row = fdiv(task, a.div_nseg);
+        seg = task - row * a.nseg;
+    }
+    const uint32_t b = fdiv(row, a.div_C);
     const uint32_t c = row - b * a.C;
 
     const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
     char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
     const uint32_t v0 = seg * (64u * U) + lane;
 
+    // row data first (the long latency), then the taps (scalar-cache hits)
     uint4 X[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t v = v0 + u * 64u;
         X[u] = make_uint4(0, 0, 0, 0);
-        if (v < a.nvec) X[u] = *(const uint4 *)(xrow + (int64_t)v * 16);
+        if (v < a.nvec) X[u] = load_vec<NT>(xrow + (int64_t)v * 16);
     }
 
-    float w[W];
-#pragma unroll
-    for (int k = 0; k < W; ++k)
-        w[k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
-    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+    RawTaps<1> raw;
+    fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
+
+    float w[1][W], bvv[1];
+    decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
+    const float bv = bvv[0];
 
     // history of the segment's first vector (only lane 0's copy is consumed)
     float carry[3] = {0.0f, 0.0f, 0.0f};
@@ -291,8 +490,8 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
                 float v = load1<DT>(xrow, t0 - 3 + j);
-                if (a.mask)
-                    v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + (t0 - 3 + j) * a.m_sl, a.mask_dtype));
+                if constexpr (MASK)
+                    v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + (t0 - 3 + j) * a.m_sl, a.mask_dtype));
                 carry[j] = v;
             }
         } else if (a.init) {
@@ -306,16 +505,16 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint32_t v = v0 + u * 64u;
-        float xr[E], xm[E];
+        float xr[E], xm_store[MASK ? E : 1];
+        float *xm = MASK ? xm_store : xr;
         unpack_vec<DT>(X[u], xr);
-        if (a.mask && v < a.nvec) {
-            const int64_t mbase = b * a.m_sb + (int64_t)v * E * a.m_sl;
+        if constexpr (MASK) {
+            float m[E];
 #pragma unroll
-            for (int j = 0; j < E; ++j)
-                xm[j] = round_through<DT>(xr[j] * load_mask(a.mask, mbase + j * a.m_sl, a.mask_dtype));
-        } else {
+            for (int j = 0; j < E; ++j) m[j] = 0.0f;
+            if (v < a.nvec) load_mask_vec<E>(a.mask, b * a.m_sb + (int64_t)v * E * a.m_sl, a.m_sl, a.mask_dtype, m);
 #pragma unroll
-            for (int j = 0; j < E; ++j) xm[j] = xr[j];
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], m[j]);
         }
         // seq[0..2] = the three masked inputs before this vector
         float seq[E + 3];
@@ -335,10 +534,21 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
         for (int j = 0; j < E; ++j) {
             float acc = bv;
 #pragma unroll
-            for (int k = 0; k < W; ++k) acc = fmaf(w[k], seq[j + (4 - W) + k], acc);
-            o[j] = finish(acc, a.act, a.res_mode, xm[j], xr[j]);
+            for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
+            o[j] = acc;
         }
-        if (v < a.nvec) *(uint4 *)(orow + (int64_t)v * 16) = pack_vec<DT>(o);
+        if (a.act) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] = silu_fast(o[j]);
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += xr[j];
+        } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += xm[j];
+        }
+        if (v < a.nvec) store_vec<NT>(orow + (int64_t)v * 16, pack_vec<DT>(o));
     }
 
     if (a.fin && seg == a.nseg - 1) capture_row_state<DT>(a, b, c, lane);
@@ -352,55 +562,45 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 // three previous (masked) rows in registers; a wave's loads are contiguous
 // 1 KB row pieces.  Rows are fetched R at a time so R loads are in flight.
 // ---------------------------------------------------------------------------
-// Taps and bias of E adjacent channels, rounded to the storage type of x.
-// `vec` (decided on the host): weight is a contiguous, 16-byte aligned [C, 4].
-template <int DT, int W>
-__device__ __forceinline__ void load_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
-                                          int w_dtype, bool vec, uint32_t c0, float (*w)[W], float *bv)
+template <int DT, int W, bool MASK, bool NT>
+__device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias, float (*hist)[Elem<DT>::per_vec],
+                                        const uint4 &X, float m, char *optr)
 {
     constexpr int E = Elem<DT>::per_vec;
-    if (W == 4 && vec) {
-        if (w_dtype == CANON_DTYPE_F32) {
-            const uint4 *p = (const uint4 *)weight + c0;
+    float xr[E], xm_store[MASK ? E : 1], o[E];
+    float *xm = MASK ? xm_store : xr;
+    unpack_vec<DT>(X, xr);
+    if constexpr (MASK) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) {
-                const uint4 q = p[e];
-                w[e][0] = round_through<DT>(bits_f(q.x));
-                w[e][1] = round_through<DT>(bits_f(q.y));
-                w[e][W - 2] = round_through<DT>(bits_f(q.z));
-                w[e][W - 1] = round_through<DT>(bits_f(q.w));
-            }
-        } else {
-            const uint2 *p = (const uint2 *)weight + c0;
-#pragma unroll
-            for (int e = 0; e < E; ++e) {
-                const uint2 q = p[e];
-                float t0, t1, t2, t3;
-                if (w_dtype == CANON_DTYPE_BF16) {
-                    unpack2<CANON_DTYPE_BF16>(q.x, t0, t1);
-                    unpack2<CANON_DTYPE_BF16>(q.y, t2, t3);
-                } else {
-                    unpack2<CANON_DTYPE_F16>(q.x, t0, t1);
-                    unpack2<CANON_DTYPE_F16>(q.y, t2, t3);
-                }
-                w[e][0] = round_through<DT>(t0);
-                w[e][1] = round_through<DT>(t1);
-                w[e][W - 2] = round_through<DT>(t2);
-                w[e][W - 1] = round_through<DT>(t3);
-            }
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < E; ++e)
-#pragma unroll
-            for (int k = 0; k < W; ++k)
-                w[e][k] = round_through<DT>(load_w(weight, (int64_t)(c0 + e) * w_sc + k * w_sk, w_dtype));
+        for (int e = 0; e < E; ++e) xm[e] = mul_round<DT>(xr[e], m);
     }
 #pragma unroll
-    for (int e = 0; e < E; ++e) bv[e] = bias ? round_through<DT>(load_w(bias, c0 + e, w_dtype)) : 0.0f;
+    for (int e = 0; e < E; ++e) {
+        float acc = bias[e];
+        if constexpr (W == 4) acc = fmaf(w[e][0], hist[0][e], acc);
+        if constexpr (W >= 3) acc = fmaf(w[e][W - 3], hist[1][e], acc);
+        acc = fmaf(w[e][W - 2], hist[2][e], acc);
+        acc = fmaf(w[e][W - 1], xm[e], acc);
+        o[e] = acc;
+        hist[0][e] = hist[1][e];
+        hist[1][e] = hist[2][e];
+        hist[2][e] = xm[e];
+    }
+    if (a.act) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
+    }
+    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] += xr[e];
+    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] += xm[e];
+    }
+    store_vec<NT>(optr, pack_vec<DT>(o));
 }
 
-template <int DT, int W, int R>
+template <int DT, int W, int R, bool MASK, bool NT>
 __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
@@ -408,14 +608,11 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
     if (blk >= a.nblocks) return;
     const uint32_t tid = blk * 256u + threadIdx.x;
     if (tid >= a.ntasks) return;
-    const uint32_t cv = tid % a.nvec;
-    const uint32_t bc = tid / a.nvec;
-    const uint32_t ch = bc % a.nseg;
-    const uint32_t b = bc / a.nseg;
+    const uint32_t bc = fdiv(tid, a.div_nvec);
+    const uint32_t cv = tid - bc * a.nvec;
+    const uint32_t b = fdiv(bc, a.div_nseg);
+    const uint32_t ch = bc - b * a.nseg;
     const uint32_t c0 = cv * E;
-
-    float w[E][W], bias[E];
-    load_taps<DT, W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, w, bias);
 
     const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * Elem<DT>::bytes;
     char *ob = a.out + ((int64_t)b * a.o_sb + c0) * Elem<DT>::bytes;
@@ -423,6 +620,18 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
     const int64_t t_begin = (int64_t)ch * a.chunk;
     const int64_t t_stop = t_begin + (int64_t)a.chunk;
     const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+
+    // the first batch of rows is requested before the history rows and the taps
+    uint4 X[R];
+    float m[R];
+    if (t_begin + R <= t_end) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            X[r] = load_vec<NT>(xb + (t_begin + r) * xs);
+            m[r] = 0.0f;
+            if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + (t_begin + r) * a.m_sl, a.mask_dtype);
+        }
+    }
 
     // hist[j] = masked row t_begin - 3 + j
     float hist[3][E];
@@ -433,12 +642,11 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         for (int e = 0; e < E; ++e) hist[j][e] = 0.0f;
         if (j < 3 - (W - 1)) continue;
         if (t >= 0) {
-            const uint4 v = *(const uint4 *)(xb + t * xs);
-            unpack_vec<DT>(v, hist[j]);
-            if (a.mask) {
-                const float m = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+            unpack_vec<DT>(load_vec<false>(xb + t * xs), hist[j]);
+            if constexpr (MASK) {
+                const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
 #pragma unroll
-                for (int e = 0; e < E; ++e) hist[j][e] = round_through<DT>(hist[j][e] * m);
+                for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mm);
             }
         } else if (a.init && a.S_in + t >= 0) {
 #pragma unroll
@@ -447,40 +655,38 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         }
     }
 
-    for (int64_t t = t_begin; t < t_end; t += R) {
-        uint4 X[R];
-        float m[R];
+    RawTaps<E> raw;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
+    float w[E][W], bias[E];
+    decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+
+    int64_t t = t_begin;
+    for (; t + R <= t_end; t += R) {
+        // request the next full batch before working on this one
+        uint4 Xn[R];
+        float mn[R];
+        const int64_t tn = t + R;
+        if (tn + R <= t_end) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            X[r] = make_uint4(0, 0, 0, 0);
-            m[r] = 1.0f;
-            if (t + r < t_end) {
-                X[r] = *(const uint4 *)(xb + (t + r) * xs);
-                if (a.mask) m[r] = load_mask(a.mask, b * a.m_sb + (t + r) * a.m_sl, a.mask_dtype);
+            for (int r = 0; r < R; ++r) {
+                Xn[r] = load_vec<NT>(xb + (tn + r) * xs);
+                mn[r] = 0.0f;
+                if constexpr (MASK) mn[r] = load_mask(a.mask, b * a.m_sb + (tn + r) * a.m_sl, a.mask_dtype);
             }
         }
 #pragma unroll
+        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t + r) * os);
+#pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (t + r < t_end) {
-                float xr[E], xm[E], o[E];
-                unpack_vec<DT>(X[r], xr);
-#pragma unroll
-                for (int e = 0; e < E; ++e) xm[e] = a.mask ? round_through<DT>(xr[e] * m[r]) : xr[e];
-#pragma unroll
-                for (int e = 0; e < E; ++e) {
-                    float acc = bias[e];
-                    if constexpr (W == 4) acc = fmaf(w[e][0], hist[0][e], acc);
-                    if constexpr (W >= 3) acc = fmaf(w[e][W - 3], hist[1][e], acc);
-                    acc = fmaf(w[e][W - 2], hist[2][e], acc);
-                    acc = fmaf(w[e][W - 1], xm[e], acc);
-                    o[e] = finish(acc, a.act, a.res_mode, xm[e], xr[e]);
-                    hist[0][e] = hist[1][e];
-                    hist[1][e] = hist[2][e];
-                    hist[2][e] = xm[e];
-                }
-                *(uint4 *)(ob + (t + r) * os) = pack_vec<DT>(o);
-            }
+            X[r] = Xn[r];
+            m[r] = mn[r];
         }
+    }
+    for (; t < t_end; ++t) {   // fewer than R rows left
+        const uint4 xv = load_vec<NT>(xb + t * xs);
+        float mv = 0.0f;
+        if constexpr (MASK) mv = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+        blc_row<DT, W, MASK, NT>(a, w, bias, hist, xv, mv, ob + t * os);
     }
 
     if (a.fin && ch == a.nseg - 1) {
@@ -490,11 +696,11 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
 #pragma unroll
             for (int e = 0; e < E; ++e) v[e] = 0.0f;
             if (t >= 0) {
-                unpack_vec<DT>(*(const uint4 *)(xb + t * xs), v);
-                if (a.mask) {
+                unpack_vec<DT>(load_vec<false>(xb + t * xs), v);
+                if constexpr (MASK) {
                     const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
 #pragma unroll
-                    for (int e = 0; e < E; ++e) v[e] = round_through<DT>(v[e] * mm);
+                    for (int e = 0; e < E; ++e) v[e] = mul_round<DT>(v[e], mm);
                 }
             } else if (a.init && a.S_in + t >= 0) {
 #pragma unroll
@@ -547,7 +753,7 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
         const int64_t t = t_begin - 3 + j;
         if (t >= 0) {
             float v = load1<DT>(a.x, xo + t * a.x_sl);
-            if (a.mask) v = round_through<DT>(v * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
             h[j] = v;
         } else if (a.init && a.S_in + t >= 0) {
             h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
@@ -556,7 +762,7 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
     for (int64_t t = t_begin; t < t_end; ++t) {
         const float xr = load1<DT>(a.x, xo + t * a.x_sl);
         float xm = xr;
-        if (a.mask) xm = round_through<DT>(xr * load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+        if (a.mask) xm = mul_round<DT>(xr, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
         float acc = bv;
         if (W == 4) acc = fmaf(w[0], h[0], acc);
         if (W >= 3) acc = fmaf(w[1], h[1], acc);
@@ -624,12 +830,9 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
     constexpr int BY = Elem<DT>::bytes;
     const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
     if (tid >= a.nthreads) return;
-    const uint32_t cv = tid % a.nvec;
-    const uint32_t bg = tid / a.nvec;
+    const uint32_t bg = fdiv(tid, a.div_nvec);
+    const uint32_t cv = tid - bg * a.nvec;
     const uint32_t c0 = cv * E;
-
-    float w[E][W], bias[E];
-    load_taps<DT, W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, w, bias);
 
     uint4 X[NB];
     uint4 ST[NB][S];
@@ -646,22 +849,42 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
             if (a.tmask) tm[n] = load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype);
         }
     }
+    RawTaps<E> raw;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
+    float w[E][W], bias[E];
+    decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
         const uint32_t b = bg * NB + n;
         if (b >= a.B) continue;
         float xr[E], xt[E], o[E];
         unpack_vec<DT>(X[n], xr);
+        if (a.tmask) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) xt[e] = a.tmask ? round_through<DT>(xr[e] * tm[n]) : xr[e];
+            for (int e = 0; e < E; ++e) xt[e] = mul_round<DT>(xr[e], tm[n]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) xt[e] = xr[e];
+        }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             float acc = bias[e];
 #pragma unroll
             for (int k = 0; k < W - 1; ++k)
                 acc = fmaf(w[e][k], StateRun<DT>::as_float(StateRun<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
-            acc = fmaf(w[e][W - 1], xt[e], acc);
-            o[e] = finish(acc, a.act, a.res_mode, xt[e], xr[e]);
+            o[e] = fmaf(w[e][W - 1], xt[e], acc);
+        }
+        if (a.act) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
+        }
+        if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += xt[e];
+        } else if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += xr[e];
         }
         *(uint4 *)(a.out + ((int64_t)b * a.o_sb + c0) * BY) = pack_vec<DT>(o);
 
@@ -671,7 +894,11 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
         for (int e = 0; e < E; ++e) {
 #pragma unroll
             for (int k = 0; k < S - 1; ++k) raw[e * S + k] = StateRun<DT>::get(ST[n], e * S + k + 1);
-            raw[e * S + S - 1] = a.tmask ? StateRun<DT>::raw_of(xt[e]) : StateRun<DT>::get(&X[n], e);
+            raw[e * S + S - 1] = StateRun<DT>::get(&X[n], e);   // the token's own bits
+        }
+        if (a.tmask) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) raw[e * S + S - 1] = StateRun<DT>::raw_of(xt[e]);
         }
         uint4 *dp = (uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
 #pragma unroll
@@ -706,7 +933,7 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
     const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
     const float xr = load1<DT>(a.x, (int64_t)b * a.x_sb + (int64_t)c * a.x_sc);
     float xt = xr;
-    if (a.tmask) xt = round_through<DT>(xr * load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype));
+    if (a.tmask) xt = mul_round<DT>(xr, load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype));
     for (int k = 0; k < W - 1; ++k) win[4 - W + k] = load1<DT>(a.state, so + (int64_t)(S - (W - 1) + k) * a.s_ss);
     win[3] = xt;
     float acc;
@@ -719,7 +946,7 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
         acc = finish(acc, a.act, a.res_mode, xt, xr);
     } else {
         float s = 0.0f;
-        for (int k = 4 - W; k < 4; ++k) s = __fadd_rn(s, round_through<DT>(__fmul_rn(win[k], w[k])));
+        for (int k = 4 - W; k < 4; ++k) s = __fadd_rn(s, mul_round<DT>(win[k], w[k]));
         s = round_through<DT>(s);
         acc = round_through<DT>(__fadd_rn(bv, s));
         if (a.act) acc = round_through<DT>(silu_precise(acc));
@@ -756,11 +983,25 @@ bool valid_mask_dtype(int d) { return d >= CANON_MASK_U8 && d <= CANON_MASK_F16;
 int elem_bytes(int d) { return d == CANON_DTYPE_F32 ? 4 : 2; }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+FastDiv make_fastdiv(uint32_t d)
+{
+    // floor(n / d) for 0 <= n < 2^32 (Granlund-Montgomery round-up method)
+    FastDiv f;
+    f.d = d ? d : 1;
+    uint32_t l = 0;
+    while ((1ull << l) < f.d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - f.d)) / f.d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 0 ? l - 1 : 0;
+    return f;
+}
+
 enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
-constexpr int kBlcRows = 8;             // rows in flight per lane in the channel-contiguous kernel
+constexpr int kBlcRows = 4;             // rows per batch (two batches in flight) in the channel-contiguous kernel
+constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update
 
 struct FwdPlan {
@@ -823,6 +1064,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.S_in = p->initial_state ? p->initial_len : 0;
     a.S_out = p->final_state ? p->final_len : 0;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
     plan->grid = 0;
     plan->kind = FWD_GENERIC;
@@ -830,6 +1072,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
 
     const int E = 16 / elem_bytes(p->x_dtype);
     const uint64_t rows = (uint64_t)a.B * a.C;
+    a.nt = 2 * rows * a.L * elem_bytes(p->x_dtype) >= kStreamBytes;
     const bool fused = p->round_mode == CANON_ROUND_FUSED;
     const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
     const bool bcl_ok = fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
@@ -853,6 +1096,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
             plan->kind = FWD_BCL;
             plan->U = U;
             a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
+            a.div_nseg = make_fastdiv(a.nseg); a.div_C = make_fastdiv(a.C);
             a.nblocks = (uint32_t)((ntasks + 3) / 4);
             plan->grid = a.nblocks;
             return CANON_OK;
@@ -873,6 +1117,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
         if (nthreads < (1ull << 31)) {
             plan->kind = FWD_BLC;
             a.nvec = nvec; a.nseg = nseg; a.chunk = chunk; a.ntasks = (uint32_t)nthreads;
+            a.div_nvec = make_fastdiv(nvec); a.div_nseg = make_fastdiv(nseg);
             a.nblocks = (uint32_t)((nthreads + 255) / 256);
             plan->grid = ((a.nblocks + 7) / 8) * 8;
             return CANON_OK;
@@ -892,20 +1137,33 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     return CANON_OK;
 }
 
-template <int DT, int W> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
     switch (pl.U) {
-    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4>), g, b, 0, s, pl.args); break;
-    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1>), g, b, 0, s, pl.args); break;
+    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, NT>), g, b, 0, s, pl.args); break;
+    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, NT>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, NT>), g, b, 0, s, pl.args); break;
     }
+}
+
+template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
 }
 
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 {
-    if (pl.kind == FWD_BCL) launch_bcl<DT, W>(pl, s);
-    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+    const bool mask = pl.args.mask != nullptr;
+    // the streaming (non-temporal) variants exist for width 4 only
+    if (W == 4 && pl.args.nt) {
+        if (mask) launch_fwd_vec<DT, W, true, W == 4>(pl, s);
+        else launch_fwd_vec<DT, W, false, W == 4>(pl, s);
+    } else {
+        if (mask) launch_fwd_vec<DT, W, true, false>(pl, s);
+        else launch_fwd_vec<DT, W, false, false>(pl, s);
+    }
 }
 
 template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
@@ -983,6 +1241,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
         a.nvec = a.C / E;
         a.bgroups = (a.B + kUpdNB - 1) / kUpdNB;
         a.nthreads = a.nvec * a.bgroups;
+        a.div_nvec = make_fastdiv(a.nvec);
         plan->grid = (a.nthreads + 255) / 256;
     } else {
         a.nthreads = a.B * a.C;

@@ -28,6 +28,9 @@ for p in (ROOT, os.path.join(ROOT, "viby-model_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, vendor figure
+# HBM bytes per launch of the headline kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
+# plain copy of known size (profiles/prefill_time_contiguous_bf16_B8_C3456_L1024.txt)
+MEASURED_TRAFFIC_BYTES = 113.54e6
 B, C, L, W = 8, 3456, 1024, 4   # the configuration the metric is quoted on
 DEC_B, DEC_S, DEC_STEPS = 256, 3, 64
 
@@ -161,6 +164,9 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="also run this many plain device-to-device copies of one x-sized buffer "
+                         "(a kernel of known traffic to scale profiler byte counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU by design (rows of the conv are independent; "
@@ -168,6 +174,14 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    if args.calibration_copies:
+        src = torch.empty(B * C * L, dtype=torch.bfloat16, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(args.calibration_copies):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     nbuf = 6  # 6 x 113 MB = 680 MB of distinct traffic between reuses
     ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
@@ -192,7 +206,7 @@ def main():
                    "us_per_step_hipgraph": round(dec_graph_us, 3),
                    "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

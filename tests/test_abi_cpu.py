@@ -1,0 +1,247 @@
+"""CPU-side checks of the C ABI and of the host logic (no kernel is launched).
+
+  * the shared library loads and exports every function the header declares
+  * the ctypes mirrors of the parameter structs match the C layout (checked
+    against gcc's sizeof/offsetof of the real header)
+  * argument validation and kernel-family planning (pure host code)
+  * the Python wrappers raise the reference's error types / messages
+    (causal-conv1d-mps/test.py:220-236) before touching a device
+  * there is no fallback: a missing library is an ImportError
+"""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "canon_conv1d.h")
+
+import causal_conv1d as cc                      # noqa: E402
+from causal_conv1d import _lib                  # noqa: E402
+from causal_conv1d._lib import FwdParams, UpdateParams  # noqa: E402
+
+
+def test_library_exports_every_declared_function():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(canon_conv1d_[a-z_]+)\s*\(", text))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    L = _lib.lib()
+    for name in declared:
+        assert getattr(L, name) is not None
+    assert L.canon_conv1d_abi_version() == _lib.ABI_VERSION
+    assert L.canon_conv1d_last_error() is not None
+
+
+def test_ctypes_structs_match_the_header(tmp_path):
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){']
+    for cname, cls in (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams)):
+        lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')
+        for fname, _ in cls._fields_:
+            lines.append(f'printf("{cname} {fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines.append('return 0;}')
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-o", str(exe), str(src)])
+    out = subprocess.check_output([str(exe)], text=True).split("\n")
+    got = {tuple(l.split()[:2]): int(l.split()[2]) for l in out if l}
+    for cname, cls in (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams)):
+        assert got[(cname, "size")] == ctypes.sizeof(cls)
+        for fname, _ in cls._fields_:
+            assert got[(cname, fname)] == getattr(cls, fname).offset, (cname, fname)
+
+
+# ---------------------------------------------------------------------------
+# planning / validation: fake (never dereferenced) device addresses
+# ---------------------------------------------------------------------------
+FAKE_X, FAKE_OUT, FAKE_W, FAKE_STATE = 0x10000000, 0x20000000, 0x30000000, 0x40000000
+
+
+def fwd_params(B=8, C=3456, L=1024, layout="bcl", dtype=1, **over):
+    p = FwdParams()
+    p.struct_size = ctypes.sizeof(FwdParams)
+    p.x_dtype = p.w_dtype = dtype
+    p.width = 4
+    p.batch, p.channels, p.seqlen = B, C, L
+    p.x, p.out, p.weight = FAKE_X, FAKE_OUT, FAKE_W
+    if layout == "bcl":
+        strides = (C * L, L, 1)
+    else:
+        strides = (C * L, 1, C)
+    p.x_stride_b, p.x_stride_c, p.x_stride_l = strides
+    p.out_stride_b, p.out_stride_c, p.out_stride_l = strides
+    p.w_stride_c, p.w_stride_k = 4, 1
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def plan(p):
+    r = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(p))
+    return r.decode() if r is not None else None
+
+
+def last_error():
+    return _lib.lib().canon_conv1d_last_error().decode()
+
+
+def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
+    for C in (640, 960, 3456):
+        assert plan(fwd_params(C=C, layout="bcl")) == "bcl_vec"
+        assert plan(fwd_params(C=C, layout="blc")) == "blc_vec"
+    assert plan(fwd_params(B=1, C=640, L=1024, dtype=0)) == "bcl_vec"     # BASELINE config 1
+    # ragged sizes, misalignment, eager rounding -> strided kernel
+    assert plan(fwd_params(L=1023)) == "generic"
+    assert plan(fwd_params(C=3457, layout="blc")) == "generic"
+    assert plan(fwd_params(x=FAKE_X + 2)) == "generic"
+    assert plan(fwd_params(round_mode=1)) == "generic"
+    assert plan(fwd_params(L=64)) == "generic"                             # rows too short for a wave
+    # strided but aligned rows (a channel slice of a bigger tensor) stay vectorised
+    assert plan(fwd_params(C=128, x_stride_b=4096 * 1024, x_stride_c=1024)) == "bcl_vec"
+
+
+def test_fwd_validation_messages():
+    cases = [
+        (dict(struct_size=8), "struct_size"),
+        (dict(width=5), "width 5"),
+        (dict(width=1), "width 1"),
+        (dict(x_dtype=7), "x_dtype"),
+        (dict(activation=3), "activation"),
+        (dict(residual_mode=9), "residual_mode"),
+        (dict(round_mode=2), "round_mode"),
+        (dict(batch=-1), "negative"),
+        (dict(out=FAKE_X), "alias"),
+        (dict(x=0), "NULL"),
+        (dict(mask=FAKE_STATE, mask_dtype=17), "mask_dtype"),
+        (dict(initial_state=FAKE_STATE, initial_len=2), "initial_len"),
+        (dict(final_state=FAKE_STATE, final_len=0), "final_len"),
+        (dict(batch=1 << 20, channels=1 << 12), "2^31"),
+    ]
+    for over, needle in cases:
+        assert plan(fwd_params(**over)) is None, over
+        assert needle in last_error(), (over, last_error())
+    assert _lib.lib().canon_conv1d_fwd_plan(None) is None
+    # empty problems are accepted (and launch nothing)
+    assert plan(fwd_params(B=0)) is not None
+    assert plan(fwd_params(L=0, x=0, out=0)) is not None
+
+
+def update_params(B=256, C=3456, S=3, dtype=1, **over):
+    p = UpdateParams()
+    p.struct_size = ctypes.sizeof(UpdateParams)
+    p.x_dtype = p.w_dtype = dtype
+    p.width, p.state_len = 4, S
+    p.batch, p.channels = B, C
+    p.x, p.out, p.conv_state, p.weight = FAKE_X, FAKE_OUT, FAKE_STATE, FAKE_W
+    p.x_stride_b, p.x_stride_c = C, 1
+    p.out_stride_b, p.out_stride_c = C, 1
+    p.state_stride_b, p.state_stride_c, p.state_stride_s = C * S, S, 1
+    p.w_stride_c, p.w_stride_k = 4, 1
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def uplan(p):
+    r = _lib.lib().canon_conv1d_update_plan(ctypes.byref(p))
+    return r.decode() if r is not None else None
+
+
+def test_update_plan_and_validation():
+    for S in (3, 4, 8):
+        assert uplan(update_params(S=S)) == "update_vec"
+    assert uplan(update_params(S=5)) == "update_generic"
+    assert uplan(update_params(C=3457)) == "update_generic"
+    assert uplan(update_params(state_stride_s=2, state_stride_c=6, state_stride_b=3456 * 6)) == "update_generic"
+    assert uplan(update_params(round_mode=1)) == "update_generic"
+    for over, needle in [(dict(S=2), "state_len"), (dict(width=7), "width"),
+                         (dict(cache_seqlens=FAKE_STATE), "cache_seqlens"),
+                         (dict(conv_state_indices=FAKE_STATE), "conv_state_indices"),
+                         (dict(conv_state=0), "NULL"), (dict(struct_size=4), "struct_size")]:
+        if "S" in over:
+            p = update_params(S=over["S"])
+        else:
+            p = update_params(**over)
+        assert uplan(p) is None, over
+        assert needle in last_error(), (over, last_error())
+
+
+# ---------------------------------------------------------------------------
+# Python wrappers: the reference's error conventions, raised on the host
+# ---------------------------------------------------------------------------
+def test_wrapper_errors_match_reference_conventions():
+    x = torch.randn(2, 4, 8)
+    with pytest.raises(ValueError, match="does not match"):
+        cc.causal_conv1d_fn(x, torch.randn(5, 4))
+    with pytest.raises(ValueError, match="Expected 3D input tensor"):
+        cc.causal_conv1d_fn(torch.randn(4, 8), torch.randn(4, 4))
+    with pytest.raises(ValueError, match="Expected 2D weight tensor"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 1, 4))
+    with pytest.raises(ValueError, match="Expected 1D bias tensor"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), torch.randn(4, 1))
+    with pytest.raises(ValueError, match="Bias dim 3 does not match"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), torch.randn(3))
+    with pytest.raises(NotImplementedError, match="activation must be None, silu, or swish"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), activation="relu")
+    with pytest.raises(NotImplementedError, match="seq_idx"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), seq_idx=torch.zeros(2, 8, dtype=torch.int32))
+    with pytest.raises(NotImplementedError, match="width 5"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 5))
+    with pytest.raises(ValueError, match="Unsupported input dtype"):
+        cc.causal_conv1d_fn(x.double(), torch.randn(4, 4))
+    # a CPU tensor is an error, never a silent slow path
+    with pytest.raises(ValueError, match="must be on a ROCm GPU device"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4))
+    with pytest.raises(ValueError, match="Expected 2D input tensor"):
+        cc.causal_conv1d_update(torch.randn(4), torch.zeros(2, 4, 4), torch.randn(4, 4))
+    with pytest.raises(ValueError, match="Expected 3D conv_state"):
+        cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4), torch.randn(4, 4))
+    with pytest.raises(ValueError, match="doesn't match conv_state"):
+        cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(3, 4, 4), torch.randn(4, 4))
+    with pytest.raises(NotImplementedError, match="cache_seqlens"):
+        cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4, 4), torch.randn(4, 4),
+                                cache_seqlens=torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="must be on a ROCm GPU device"):
+        cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4, 4), torch.randn(4, 4))
+    with pytest.raises(ValueError, match="Expected 3D input tensor"):
+        cc.short_conv_fused(torch.randn(4, 8), torch.randn(8, 4))
+
+
+def test_missing_library_is_an_import_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", os.path.join(ROOT, "does", "not", "exist.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.lib()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "viby-model_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"oracle", text, flags=re.I), os.path.join(dirpath, f)
+
+
+def test_canon_layer_module_mirrors_the_reference_class():
+    """Same constructor, parameter names/shapes and cache attribute as model/model.py:201-241."""
+    import types
+    from causal_conv1d.canon import CanonLayer
+    cfg = types.SimpleNamespace(canon_kernel=4, canon_bias=True, canon_activation=False)
+    layer = CanonLayer(640, cfg, "b")
+    sd = layer.state_dict()
+    assert set(sd) == {"weight", "bias_param"}
+    assert tuple(sd["weight"].shape) == (640, 1, 4) and tuple(sd["bias_param"].shape) == (640,)
+    layer.reset_parameters()
+    assert float(layer.weight.abs().max()) <= 0.5 + 1e-6          # kaiming-uniform(a=sqrt 5), fan_in 4
+    nobias = CanonLayer(8, types.SimpleNamespace(canon_kernel=3, canon_bias=False, canon_activation=True), "a")
+    assert nobias.bias_param is None and set(nobias.state_dict()) == {"weight"}
+    cache = types.SimpleNamespace(_max_layers=18)
+    assert nobias._slot(cache) is cache.canon_cache_a and len(cache.canon_cache_a) == 18
+    with pytest.raises(ValueError, match="must be on a ROCm GPU device"):
+        layer(torch.randn(1, 4, 640))

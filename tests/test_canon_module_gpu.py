@@ -1,0 +1,98 @@
+"""The drop-in CanonLayer (HIP kernels) against vectors of the reference's own
+CanonLayer (tests/golden/, produced from model/model.py's eager branch) and
+against the eager restatement at larger sizes."""
+import json
+import os
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_parity, bits, right_padded_mask
+from oracle.canon_eager import EagerCanon
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _cases():
+    with open(os.path.join(GOLDEN, "canon_layer_cases.json")) as f:
+        return json.load(f)["cases"]
+
+
+def _tensor(arrays, key, dtype):
+    a = torch.from_numpy(arrays[key])
+    return a.view(torch.bfloat16) if dtype == torch.bfloat16 else a
+
+
+def make_layer(D, W, w, b, act, dtype, rounding):
+    from causal_conv1d.canon import CanonLayer
+    cfg = types.SimpleNamespace(canon_kernel=W, canon_bias=b is not None, canon_activation=act)
+    layer = CanonLayer(D, cfg, "a", rounding=rounding).to(device=DEV, dtype=dtype)
+    with torch.no_grad():
+        layer.weight.copy_(w.view(D, 1, W))
+        if b is not None:
+            layer.bias_param.copy_(b)
+    return layer
+
+
+@pytest.mark.parametrize("rounding", ["eager", "fused"])
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: c["name"])
+def test_canon_layer_golden_vectors(case, rounding):
+    arrays = np.load(os.path.join(GOLDEN, "canon_layer_cases.npz"))
+    name, dtype = case["name"], getattr(torch, case["dtype"])
+    w = _tensor(arrays, f"{name}/weight", dtype)
+    b = _tensor(arrays, f"{name}/bias", dtype) if case["bias"] else None
+    layer = make_layer(case["D"], case["W"], w, b, case["activation"], dtype, rounding)
+    cache = types.SimpleNamespace()
+    with torch.no_grad():
+        for i, call in enumerate(case["calls"]):
+            key = f"{name}/call{i}"
+            x = _tensor(arrays, f"{key}/x", dtype)
+            mask = torch.from_numpy(arrays[f"{key}/mask"]).to(DEV) if call["mask"] else None
+            out = layer(x.to(DEV), attention_mask=mask, cache=cache if call["cache"] else None,
+                        layer_idx=0 if call["cache"] else None)
+            want = _tensor(arrays, f"{key}/out", dtype)
+            if call["cache"]:
+                want_state = _tensor(arrays, f"{key}/state", dtype)
+                assert torch.equal(bits(cache.canon_cache_a[0]), bits(want_state)), (name, i, "state")
+            if rounding == "eager" and dtype != torch.float32:
+                # same rounding points as the reference: bit exact (1 ulp where SiLU's exp differs)
+                assert_parity(out, want, exact=not case["activation"], what=f"{name}/call{i}")
+            elif dtype == torch.float32:
+                assert_parity(out, want, exact=False, what=f"{name}/call{i}", res=x)
+            else:
+                # single rounding vs the reference's three: within the reference's own bf16 tolerance
+                torch.testing.assert_close(out.cpu().float(), want.float(), rtol=5e-3, atol=2e-2)
+
+
+@pytest.mark.parametrize("site,C", [("a", 640), ("b", 960), ("d", 3456)])
+def test_canon_layer_prefill_then_decode_at_model_shapes(site, C):
+    """BASELINE shapes of the four call sites: prefill with a padding mask, then 8 decode steps."""
+    torch.manual_seed(5)
+    B, T = 4, 256
+    dtype = torch.bfloat16
+    w = (torch.randn(C, 4) * 0.3).to(dtype)
+    x = torch.randn(B, T, C).to(dtype)
+    mask = right_padded_mask([256, 200, 131, 17], T)
+    ref = EagerCanon(w, None, False)
+    ref_cache = {}
+    want = ref.forward(x, mask, ref_cache, 0)
+    layer = make_layer(C, 4, w, None, False, dtype, "eager")
+    cache = types.SimpleNamespace()
+    with torch.no_grad():
+        got = layer(x.to(DEV), attention_mask=mask.to(DEV), cache=cache, layer_idx=3)
+        assert_parity(got, want, exact=True, what=f"site {site} prefill")
+        state = cache.canon_cache_a[3]
+        assert torch.equal(bits(state), bits(ref_cache[0]))
+        full_mask = mask
+        for step in range(8):
+            tok = torch.randn(B, 1, C).to(dtype)
+            full_mask = torch.cat([full_mask, torch.tensor([[1], [1], [0], [1]])], dim=1)
+            want = ref.forward(tok, full_mask, ref_cache, 0)
+            got = layer(tok.to(DEV), attention_mask=full_mask.to(DEV), cache=cache, layer_idx=3)
+            assert cache.canon_cache_a[3] is state            # updated in place, same object
+            assert torch.equal(bits(state), bits(ref_cache[0])), step
+            assert_parity(got, want, exact=False, what=f"site {site} step {step}")

@@ -191,6 +191,41 @@ def test_edge_shapes_and_strides(cc, dtype):
     assert_parity(run_fwd(cc, xg, w, None), co.conv1d_fwd(xv, w), exact=True, what="edge/misaligned")
 
 
+@pytest.mark.parametrize("xdtype", [torch.bfloat16, torch.float32])
+def test_every_mask_dtype_and_alignment(cc, xdtype):
+    g = torch.Generator().manual_seed(55)
+    B, C, L = 3, 16, 640
+    x = torch.randn(B, C, L, generator=g).to(xdtype)
+    w = torch.randn(C, 4, generator=g).to(xdtype)
+    keep = torch.rand(B, L, generator=g) > 0.3
+    want, wfs = co.conv1d_fwd(x, w, None, mask=keep, residual=1, final_state_len=4)
+    for mdtype in [torch.bool, torch.uint8, torch.int32, torch.int64, torch.float32, torch.bfloat16, torch.float16]:
+        m = keep.to(mdtype)
+        # contiguous (wide loads), a strided view and a misaligned view (narrow loads)
+        wide = torch.zeros(B, 2 * L + 1, dtype=mdtype)
+        wide[:, 1::2] = m
+        shifted = torch.zeros(B * L + 1, dtype=mdtype)
+        shifted[1:] = m.flatten()
+        variants = {"contig": m.to(DEV), "strided": wide.to(DEV)[:, 1::2], "misaligned": shifted.to(DEV)[1:].view(B, L)}
+        for vname, mg in variants.items():
+            for name, xg in layouts(x):
+                fs = torch.empty(B, C, 4, dtype=xdtype, device=DEV)
+                got, fs = cc.causal_conv1d_fn(xg, w.to(DEV), attention_mask=mg, residual=True, final_states_out=fs)
+                assert_parity(got, want, exact=True, what=f"mask {mdtype} {vname} {name}")
+                assert torch.equal(bits(fs), bits(wfs))
+    # non-0/1 values multiply in (and round to the storage type first)
+    scale = (torch.rand(B, L, generator=g) * 3).to(torch.float32)
+    want = co.conv1d_fwd(x, w, None, mask=scale, residual="unmasked")
+    for name, xg in layouts(x):
+        got = cc.causal_conv1d_fn(xg, w.to(DEV), attention_mask=scale.to(DEV), residual="unmasked")
+        assert_parity(got, want, exact=True, what=f"scaled mask {name}")
+    big = torch.tensor([[2 ** 40, -2 ** 33, 1, 0] * (L // 4)] * B, dtype=torch.int64)
+    want = co.conv1d_fwd(x, w, None, mask=big)
+    for name, xg in layouts(x):
+        got = cc.causal_conv1d_fn(xg, w.to(DEV), attention_mask=big.to(DEV))
+        assert_parity(got, want, exact=True, what=f"int64 mask beyond 32 bits {name}")
+
+
 def test_empty_inputs(cc):
     w = torch.randn(8, 4, device=DEV)
     for shape in [(0, 8, 16), (2, 8, 0)]:

@@ -1,0 +1,118 @@
+"""``CanonLayer`` on the fused HIP kernels: one launch per call.
+
+Same constructor, parameters and ``forward`` signature as the reference's
+``CanonLayer`` (``model/model.py:201-225`` and ``:400-406``), so it can replace
+that class inside ``VibyBlock`` / ``Attention`` / ``FeedForward``
+(``model/model.py:765-794, 961-971, 1021-1027, 1049-1055``):
+
+* parameters ``weight [C, 1, K]`` and ``bias_param [C] | None`` with the same
+  names and initialisation (``model/model.py:212-225``), so checkpoints load;
+* per-layer conv states live on the cache object as the list attribute
+  ``canon_cache_<name>`` (``model/model.py:227-241``).
+
+What one call does, and which reference branch defines it.  The reference has
+three branches whose residual/state conventions differ; this module follows
+the plain-PyTorch branch, which is the one that runs wherever no accelerated
+package is installed and the one the parity vectors come from:
+
+* block of T tokens (``model/model.py:587-675``): ``xm = x * mask``;
+  ``out = xm + act(conv(xm) + bias)``; with a cache, the last
+  ``state_len = max(8, K)`` masked inputs are captured right-aligned (history,
+  if a state already exists, is taken from it: chunked continuation);
+* single token with a cache (``model/model.py:262-289, 367-398``): the token is
+  multiplied by the last mask column, the state is shifted left and the token
+  appended, ``out = x + act(conv + bias)`` (residual on the unmasked token).
+
+``rounding='eager'`` reproduces that branch's intermediate bf16/fp16 roundings
+bit for bit; the default ``'fused'`` rounds once.
+
+Forward only: with gradients enabled and parameters that require them the
+underlying calls raise (use ``torch.no_grad()`` / ``torch.inference_mode()``).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import causal_conv1d_fn, causal_conv1d_update
+
+STATE_LEN_MIN = 8  # model/model.py:286, :626
+
+
+class CanonLayer(nn.Module):
+    def __init__(self, hidden_size: int, config, name: str, rounding: str = "fused"):
+        super().__init__()
+        self.name = name
+        self.hidden_size = hidden_size
+        self.kernel_size = config.canon_kernel
+        self.bias = config.canon_bias
+        self.activation = config.canon_activation
+        self.rounding = rounding
+        self.weight = nn.Parameter(torch.randn(hidden_size, 1, self.kernel_size))
+        if self.bias:
+            self.bias_param = nn.Parameter(torch.zeros(hidden_size))
+        else:
+            self.register_parameter("bias_param", None)
+
+    def reset_parameters(self) -> None:
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        if self.bias_param is not None:
+            fan_in = self.weight.size(1) * self.weight.size(2)
+            bound = 1.0 / math.sqrt(fan_in) if fan_in > 0 else 0.0
+            nn.init.uniform_(self.bias_param, -bound, bound)
+
+    # -- cache plumbing: a list per site hung on the cache object --------------
+    def _slot(self, cache):
+        attr = f"canon_cache_{self.name}"
+        if not hasattr(cache, attr):
+            setattr(cache, attr, [None] * getattr(cache, "_max_layers", 256))
+        return getattr(cache, attr)
+
+    def _state_len(self) -> int:
+        return max(STATE_LEN_MIN, self.kernel_size)
+
+    def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                cache=None, layer_idx: Optional[int] = None) -> torch.Tensor:
+        B, T, D = x.shape
+        use_cache = cache is not None and layer_idx is not None
+        state = self._slot(cache)[layer_idx] if use_cache else None
+        taps = self.weight.squeeze(1)
+        act = "silu" if self.activation else None
+
+        if use_cache and T == 1:
+            token_mask = None
+            if attention_mask is not None and attention_mask.dim() == 2 and attention_mask.shape[0] == B:
+                token_mask = attention_mask[:, -1]
+            if state is None:
+                state = torch.zeros(B, D, self._state_len(), dtype=x.dtype, device=x.device)
+            y = causal_conv1d_update(x[:, 0], state, taps, self.bias_param, activation=act,
+                                     token_mask=token_mask, residual="unmasked", rounding=self.rounding)
+            self._slot(cache)[layer_idx] = state
+            return y.unsqueeze(1)
+
+        mask = None
+        if attention_mask is not None and attention_mask.dim() == 2:
+            if tuple(attention_mask.shape) == (B, T):
+                mask = attention_mask
+            elif attention_mask.size(0) == B and attention_mask.size(1) >= T:
+                mask = attention_mask[:, -T:]
+
+        new_state = None
+        if use_cache:
+            new_state = torch.empty(B, D, state.size(-1) if state is not None else self._state_len(),
+                                    dtype=x.dtype, device=x.device)
+        history = state if (state is not None and self.kernel_size > 1) else None
+        out = causal_conv1d_fn(x.transpose(1, 2), taps, self.bias_param, activation=act,
+                               initial_states=history, final_states_out=new_state,
+                               attention_mask=mask, residual="masked", rounding=self.rounding)
+        if use_cache:
+            out, new_state = out
+            if state is not None:
+                state.copy_(new_state)   # the cached tensor object stays the same
+            else:
+                state = new_state
+            self._slot(cache)[layer_idx] = state
+        return out.transpose(1, 2)

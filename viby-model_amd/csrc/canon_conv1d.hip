@@ -11,16 +11,25 @@
 //   * taps and bias live in registers; bias, SiLU, mask multiply, residual and
 //     the conv-state capture are fused into the same pass.
 //
-// Arithmetic contract (shared with the CPU oracle used by the tests):
+// Arithmetic contract (the tests hold a CPU restatement of exactly this):
 //     acc = bias;  for k in 0..W-1: acc = fmaf(w[k], xm[t-(W-1)+k], acc)
 // taps/bias rounded to the storage type of x first; one rounding at the store.
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
 
 #include "canon_conv1d.h"
+
+// build-time tuning knobs of the channel-contiguous prefill kernel
+#ifndef CANON_BLC_ROWS
+#define CANON_BLC_ROWS 4
+#endif
+#ifndef CANON_BLC_PREFETCH
+#define CANON_BLC_PREFETCH 1
+#endif
 
 namespace {
 
@@ -173,10 +182,75 @@ template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint
     else *(u32x4_t *)p = q;
 }
 
-// N consecutive mask entries; the element-type switch sits outside the loop
-template <int N>
-__device__ __forceinline__ void load_mask_vec(const void *p, int64_t base, int64_t stride, int dt, float *m)
+// (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
+// the value almost always fits 32 bits and one conversion instruction does it
+__device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
 {
+    if ((int32_t)hi == ((int32_t)lo >> 31)) return (float)(int32_t)lo;
+    return (float)(int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// N (4 or 8) consecutive mask entries starting at element `base`.  The
+// element-type switch sits outside the loops; `vec` (decided on the host)
+// says the entries are contiguous and the run is aligned to its own size, so
+// it is fetched with a few wide loads instead of N narrow ones.
+template <int N>
+__device__ __forceinline__ void load_mask_vec(const void *p, int64_t base, int64_t stride, int dt, bool vec, float *m)
+{
+    if (vec) {
+        switch (dt) {
+        case CANON_MASK_U8: {
+            uint32_t q[N / 4];
+#pragma unroll
+            for (int i = 0; i < N / 4; ++i) q[i] = ((const uint32_t *)((const uint8_t *)p + base))[i];
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[j] = (float)((q[j / 4] >> (8 * (j % 4))) & 0xFFu);
+            return;
+        }
+        case CANON_MASK_I32: {
+#pragma unroll
+            for (int i = 0; i < N / 4; ++i) {
+                const uint4 q = ((const uint4 *)((const int32_t *)p + base))[i];
+                m[4 * i] = (float)(int32_t)q.x; m[4 * i + 1] = (float)(int32_t)q.y;
+                m[4 * i + 2] = (float)(int32_t)q.z; m[4 * i + 3] = (float)(int32_t)q.w;
+            }
+            return;
+        }
+        case CANON_MASK_I64: {
+#pragma unroll
+            for (int i = 0; i < N / 2; ++i) {
+                const uint4 q = ((const uint4 *)((const int64_t *)p + base))[i];
+                m[2 * i] = i64_words_to_float(q.x, q.y);
+                m[2 * i + 1] = i64_words_to_float(q.z, q.w);
+            }
+            return;
+        }
+        case CANON_MASK_F32: {
+#pragma unroll
+            for (int i = 0; i < N / 4; ++i) {
+                const uint4 q = ((const uint4 *)((const float *)p + base))[i];
+                m[4 * i] = bits_f(q.x); m[4 * i + 1] = bits_f(q.y); m[4 * i + 2] = bits_f(q.z); m[4 * i + 3] = bits_f(q.w);
+            }
+            return;
+        }
+        default: {   // bf16 / fp16
+            uint32_t q[N / 2];
+            if constexpr (N == 8) {
+                const uint4 v = *(const uint4 *)((const uint16_t *)p + base);
+                q[0] = v.x; q[1] = v.y; q[2 % (N / 2)] = v.z; q[3 % (N / 2)] = v.w;
+            } else {
+                const uint2 v = *(const uint2 *)((const uint16_t *)p + base);
+                q[0] = v.x; q[1] = v.y;
+            }
+#pragma unroll
+            for (int i = 0; i < N / 2; ++i) {
+                if (dt == CANON_MASK_BF16) unpack2<CANON_DTYPE_BF16>(q[i], m[2 * i], m[2 * i + 1]);
+                else unpack2<CANON_DTYPE_F16>(q[i], m[2 * i], m[2 * i + 1]);
+            }
+            return;
+        }
+        }
+    }
     switch (dt) {
     case CANON_MASK_U8:
 #pragma unroll
@@ -254,7 +328,7 @@ struct FwdArgs {
     int64_t i_sb, i_sc, i_ss;
     int64_t f_sb, f_sc, f_ss;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_pair, nt;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
     uint32_t nseg;      // bcl: segments per row       blc: time chunks per sequence
@@ -276,7 +350,7 @@ struct UpdArgs {
     int64_t w_sc, w_sk;
     int64_t m_sb;
     uint32_t B, C;
-    int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec;
+    int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec, b_vec;
     uint32_t nvec;      // channel vectors per batch row
     uint32_t bgroups;   // batch groups (each thread walks NB batch rows)
     uint32_t nthreads;
@@ -331,7 +405,7 @@ template <int NC> struct RawTaps {
 
 template <int W, int NC>
 __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
-                                           int w_dtype, bool vec, uint32_t c0, RawTaps<NC> &r)
+                                           int w_dtype, bool vec, bool bvec, uint32_t c0, RawTaps<NC> &r)
 {
     const bool wide = w_dtype == CANON_DTYPE_F32;
     if (W == 4 && vec) {
@@ -341,6 +415,14 @@ __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias,
             for (int e = 0; e < NC; ++e) {
                 const uint4 q = p[e];
                 r.w[e][0] = q.x; r.w[e][1] = q.y; r.w[e][2] = q.z; r.w[e][3] = q.w;
+            }
+        } else if constexpr (NC % 2 == 0) {
+            const uint4 *p = (const uint4 *)((const uint2 *)weight + c0);   // c0 is a multiple of NC
+#pragma unroll
+            for (int e = 0; e < NC; e += 2) {
+                const uint4 q = p[e / 2];
+                r.w[e][0] = q.x; r.w[e][1] = q.y;
+                r.w[e + 1][0] = q.z; r.w[e + 1][1] = q.w;
             }
         } else {
             const uint2 *p = (const uint2 *)weight + c0;
@@ -365,6 +447,13 @@ __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias,
         if (wide) {
 #pragma unroll
             for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
+        } else if (NC == 8 && bvec) {
+            // eight 16-bit biases are one aligned 16-byte run (c0 is a multiple of 8)
+            const uint4 q = *(const uint4 *)((const uint16_t *)bias + c0);
+            r.b[0] = q.x & 0xFFFFu; r.b[1 % NC] = q.x >> 16;
+            r.b[2 % NC] = q.y & 0xFFFFu; r.b[3 % NC] = q.y >> 16;
+            r.b[4 % NC] = q.z & 0xFFFFu; r.b[5 % NC] = q.z >> 16;
+            r.b[6 % NC] = q.w & 0xFFFFu; r.b[7 % NC] = q.w >> 16;
         } else {
 #pragma unroll
             for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
@@ -387,9 +476,9 @@ __device__ __forceinline__ void fetch_taps_uniform(const void *weight, const voi
             const uint32_t d = ((const uint32_t *)bias)[c >> 1];
             r.b[0] = (c & 1u) ? (d >> 16) : (d & 0xFFFFu);
         }
-        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, c, r);
+        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, false, c, r);
     } else {
-        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, c, r);
+        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, false, c, r);
     }
 }
 
@@ -429,7 +518,9 @@ __device__ __forceinline__ void decode_taps_typed(const RawTaps<NC> &r, bool vec
 template <int DT, int W, int NC>
 __device__ __forceinline__ void decode_taps(const RawTaps<NC> &r, int w_dtype, bool vec, bool has_bias, float (*w)[W], float *bv)
 {
-    if (w_dtype == CANON_DTYPE_F32) decode_taps_typed<DT, CANON_DTYPE_F32, W, NC>(r, vec, has_bias, w, bv);
+    // weights that already have the storage type of x need no rounding: decode them as if x were fp32
+    if (w_dtype == DT) decode_taps_typed<CANON_DTYPE_F32, DT, W, NC>(r, vec, has_bias, w, bv);
+    else if (w_dtype == CANON_DTYPE_F32) decode_taps_typed<DT, CANON_DTYPE_F32, W, NC>(r, vec, has_bias, w, bv);
     else if (w_dtype == CANON_DTYPE_BF16) decode_taps_typed<DT, CANON_DTYPE_BF16, W, NC>(r, vec, has_bias, w, bv);
     else decode_taps_typed<DT, CANON_DTYPE_F16, W, NC>(r, vec, has_bias, w, bv);
 }
@@ -512,7 +603,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
             float m[E];
 #pragma unroll
             for (int j = 0; j < E; ++j) m[j] = 0.0f;
-            if (v < a.nvec) load_mask_vec<E>(a.mask, b * a.m_sb + (int64_t)v * E * a.m_sl, a.m_sl, a.mask_dtype, m);
+            if (v < a.nvec) load_mask_vec<E>(a.mask, b * a.m_sb + (int64_t)v * E * a.m_sl, a.m_sl, a.mask_dtype, a.m_vec != 0, m);
 #pragma unroll
             for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], m[j]);
         }
@@ -633,30 +724,42 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         }
     }
 
+    // the three rows before the chunk and the taps: requested now, consumed
+    // only after everything has been issued (one memory round trip, not four)
+    uint4 H[3];
+    float mh[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int64_t t = t_begin - 3 + j;
+        H[j] = make_uint4(0, 0, 0, 0);
+        mh[j] = 0.0f;
+        if (j >= 3 - (W - 1) && t >= 0) {
+            H[j] = load_vec<false>(xb + t * xs);
+            if constexpr (MASK) mh[j] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+        }
+    }
+    RawTaps<E> raw;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+
     // hist[j] = masked row t_begin - 3 + j
     float hist[3][E];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-        const int64_t t = t_begin - 3 + j;
+        unpack_vec<DT>(H[j], hist[j]);
+        if constexpr (MASK) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) hist[j][e] = 0.0f;
-        if (j < 3 - (W - 1)) continue;
-        if (t >= 0) {
-            unpack_vec<DT>(load_vec<false>(xb + t * xs), hist[j]);
-            if constexpr (MASK) {
-                const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
-#pragma unroll
-                for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mm);
-            }
-        } else if (a.init && a.S_in + t >= 0) {
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
+            for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mh[j]);
         }
     }
-
-    RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
+    if (t_begin == 0 && a.init) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            if (j < 3 - (W - 1)) continue;
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+        }
+    }
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 
@@ -666,7 +769,7 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         uint4 Xn[R];
         float mn[R];
         const int64_t tn = t + R;
-        if (tn + R <= t_end) {
+        if (CANON_BLC_PREFETCH && tn + R <= t_end) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 Xn[r] = load_vec<NT>(xb + (tn + r) * xs);
@@ -676,10 +779,18 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t + r) * os);
+        if (CANON_BLC_PREFETCH) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            X[r] = Xn[r];
-            m[r] = mn[r];
+            for (int r = 0; r < R; ++r) {
+                X[r] = Xn[r];
+                m[r] = mn[r];
+            }
+        } else if (tn + R <= t_end) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                X[r] = load_vec<NT>(xb + (tn + r) * xs);
+                if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + (tn + r) * a.m_sl, a.mask_dtype);
+            }
         }
     }
     for (; t < t_end; ++t) {   // fewer than R rows left
@@ -850,7 +961,7 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
         }
     }
     RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 
@@ -996,11 +1107,23 @@ FastDiv make_fastdiv(uint32_t d)
     return f;
 }
 
+// a run of E consecutive mask entries (E = elements of x per 16 bytes) starting
+// at a multiple of E is contiguous and aligned to its own size
+bool mask_run_aligned(const canon_conv1d_fwd_params *p)
+{
+    if (!p->mask || p->mask_stride_l != 1) return false;
+    static const int msize[] = {1, 4, 8, 4, 2, 2};
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const int64_t run = (int64_t)E * msize[p->mask_dtype];
+    const int64_t align = run < 16 ? run : 16;
+    return ((uintptr_t)p->mask % align) == 0 && (p->mask_stride_b * msize[p->mask_dtype]) % align == 0;
+}
+
 enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
-constexpr int kBlcRows = 4;             // rows per batch (two batches in flight) in the channel-contiguous kernel
+constexpr int kBlcRows = CANON_BLC_ROWS;           // rows per batch in the channel-contiguous kernel
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update
 
@@ -1064,6 +1187,8 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.S_in = p->initial_state ? p->initial_len : 0;
     a.S_out = p->final_state ? p->final_len : 0;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
+    a.m_vec = mask_run_aligned(p);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
     plan->grid = 0;
@@ -1112,6 +1237,9 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
         uint32_t chunk = (uint32_t)((a.L + want_chunks - 1) / want_chunks);
         chunk = ((chunk + kBlcRows - 1) / kBlcRows) * kBlcRows;
         if (chunk < 2 * kBlcRows) chunk = 2 * kBlcRows;
+#ifdef CANON_TUNING
+        if (const char *e = getenv("CANON_BLC_CHUNK")) chunk = (uint32_t)atoi(e);
+#endif
         const uint32_t nseg = (a.L + chunk - 1) / chunk;
         const uint64_t nthreads = lanes_per_step * nseg;
         if (nthreads < (1ull << 31)) {
@@ -1226,6 +1354,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
     plan->kind = UPD_GENERIC;
     plan->grid = 0;
     if (empty) return CANON_OK;

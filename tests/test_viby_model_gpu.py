@@ -1,0 +1,122 @@
+"""BASELINE config 5: a Viby-shaped model (tests/viby_harness.py) run with the HIP Canon layers
+and with reference Canon back ends inside an otherwise identical network."""
+import time
+import types
+
+import pytest
+import torch
+from torch import nn
+
+from helpers import bits
+from oracle import canon_oracle as co
+from oracle.canon_eager import EagerCanon
+from viby_harness import VibyShaped, init_weights, viby_config
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+class TorchEagerCanon(nn.Module):
+    """The eager restatement (plain torch ops) on whatever device the input lives on."""
+
+    def __init__(self, C, cfg, name):
+        super().__init__()
+        self.name = name
+        self.weight = nn.Parameter(torch.randn(C, 1, cfg.canon_kernel))
+        self.act = cfg.canon_activation
+
+    def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
+        store = cache.__dict__.setdefault("eager_states", {})
+        return EagerCanon(self.weight, None, self.act).forward(x, attention_mask, store, (self.name, layer_idx))
+
+
+class OracleCanon(nn.Module):
+    """The C oracle on the host (eager rounding points), called with the semantics of the eager CanonLayer."""
+
+    def __init__(self, C, cfg, name, round_mode):
+        super().__init__()
+        self.name, self.K, self.round_mode = name, cfg.canon_kernel, round_mode
+        self.weight = nn.Parameter(torch.randn(C, 1, cfg.canon_kernel))
+
+    def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
+        store = cache.__dict__.setdefault("oracle_states", {})
+        key = (self.name, layer_idx)
+        xc, w = x.detach().cpu(), self.weight.detach().cpu().squeeze(1)
+        B, T, D = xc.shape
+        if T == 1 and key in store:
+            tok = xc[:, 0]
+            xt = (tok * attention_mask[:, -1].cpu().unsqueeze(-1).to(tok.dtype)) if attention_mask is not None else tok
+            y = co.conv1d_update(xt.contiguous(), store[key], w, None, round_mode=1)
+            return (tok + y).unsqueeze(1).to(x.device)     # residual on the unmasked token, rounded
+        mask = attention_mask.cpu() if attention_mask is not None else None
+        out, fs = co.conv1d_fwd(xc.transpose(1, 2), w, None, mask=mask, final_state_len=max(8, self.K),
+                                residual=1, round_mode=1)
+        store[key] = fs
+        return out.transpose(1, 2).contiguous().to(x.device)
+
+
+def hip_factory(cfg, rounding):
+    from causal_conv1d.canon import CanonLayer
+    return lambda C, name: CanonLayer(C, cfg, name, rounding=rounding)
+
+
+def test_small_model_hip_equals_oracle_bit_for_bit():
+    cfg = viby_config(hidden_size=64, num_hidden_layers=3, num_attention_heads=2, num_key_value_heads=1,
+                      head_dim=32, intermediate_size=96, vocab_size=512)
+    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(1)).to(DEV)
+    hip = init_weights(VibyShaped(cfg, hip_factory(cfg, "eager")), 7, torch.bfloat16, DEV)
+    ref = init_weights(VibyShaped(cfg, lambda C, n: OracleCanon(C, cfg, n, 1)), 7, torch.bfloat16, DEV)
+    toks_h, logits_h, cache_h = hip.generate(ids, 6)
+    toks_r, logits_r, cache_r = ref.generate(ids, 6)
+    assert torch.equal(toks_h, toks_r)
+    assert torch.equal(logits_h, logits_r)
+    for site in "abcd":
+        for layer in range(cfg.num_hidden_layers):
+            got = getattr(cache_h, f"canon_cache_{site}")[layer]
+            want = cache_r.oracle_states[(site, layer)]
+            assert torch.equal(bits(got), bits(want)), (site, layer)
+
+
+def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
+    cfg = viby_config()
+    B, T, steps = 16, 1024, 128
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(5)).to(DEV)
+    hip = init_weights(VibyShaped(cfg, hip_factory(cfg, "fused")), 11, torch.bfloat16, DEV)
+    hip.generate(ids[:2, :64], 2)                       # warm-up (library load, allocator)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    toks, logits, cache = hip.generate(ids, steps)
+    torch.cuda.synchronize()
+    t_hip = time.perf_counter() - t0
+    # shapes of the carried states: one [B, C, 8] tensor per (site, layer)
+    for site, C in (("a", 640), ("b", 960), ("c", 640), ("d", 3456)):
+        states = getattr(cache, f"canon_cache_{site}")
+        assert len(states) == cfg.num_hidden_layers
+        assert all(tuple(s.shape) == (B, C, 8) for s in states)
+    del hip, cache
+    torch.cuda.empty_cache()
+
+    # the same network with the eager torch Canon, fed the tokens the HIP run produced
+    ref = init_weights(VibyShaped(cfg, lambda C, n: TorchEagerCanon(C, cfg, n)), 11, torch.bfloat16, DEV)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    toks_r, logits_r, _ = ref.generate(ids, steps, forced=toks)
+    torch.cuda.synchronize()
+    t_ref = time.perf_counter() - t0
+
+    # the HIP layers round once where the eager module rounds three times: logits agree to bf16
+    # noise accumulated over 18 layers, and the greedy choice agrees wherever it is not a near tie
+    diff = (logits - logits_r).abs()
+    scale = logits_r.abs().max().item()
+    assert diff.max().item() <= 0.05 * scale, (diff.max().item(), scale)
+    top2 = logits_r.topk(2, dim=-1).values
+    margin = top2[..., 0] - top2[..., 1]
+    decided = margin > 4 * diff.max(dim=-1).values
+    agree = logits.argmax(-1) == logits_r.argmax(-1)
+    assert bool(agree[decided].all())
+    with capsys.disabled():
+        print(f"\n[config 5] B{B} x L{T} prefill + {steps} greedy steps, 18 layers bf16: "
+              f"HIP Canon {t_hip:.2f} s, eager torch Canon {t_ref:.2f} s; "
+              f"greedy tokens equal at {agree.float().mean().item() * 100:.1f} % of steps "
+              f"({decided.float().mean().item() * 100:.1f} % decided beyond rounding noise), "
+              f"max |dlogit| {diff.max().item():.4f} of scale {scale:.2f}")

@@ -352,7 +352,8 @@ struct UpdArgs {
     uint32_t B, C;
     int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec, b_vec;
     uint32_t nvec;      // channel vectors per batch row
-    uint32_t bgroups;   // batch groups (each thread walks NB batch rows)
+    uint32_t bgroups;   // batch groups (each thread walks nb batch rows)
+    uint32_t nb;
     uint32_t nthreads;
     FastDiv div_nvec;
 };
@@ -1125,7 +1126,7 @@ enum UpdKind { UPD_VEC, UPD_GENERIC };
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
 constexpr int kBlcRows = CANON_BLC_ROWS;           // rows per batch in the channel-contiguous kernel
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
-constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update
+constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work
 
 struct FwdPlan {
     FwdKind kind;
@@ -1368,7 +1369,9 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     if (vec_ok) {
         plan->kind = UPD_VEC;
         a.nvec = a.C / E;
-        a.bgroups = (a.B + kUpdNB - 1) / kUpdNB;
+        // two batch rows per lane halve the tap loads; with little work, more waves matter more
+        a.nb = ((uint64_t)a.nvec * a.B / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        a.bgroups = (a.B + a.nb - 1) / a.nb;
         a.nthreads = a.nvec * a.bgroups;
         a.div_nvec = make_fastdiv(a.nvec);
         plan->grid = (a.nthreads + 255) / 256;
@@ -1379,14 +1382,20 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     return CANON_OK;
 }
 
-template <int DT, int W> void launch_update_vec_w(const UpdPlan &pl, hipStream_t s)
+template <int DT, int W, int NB> void launch_update_vec_nb(const UpdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
     switch (pl.args.S) {
-    case 3: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 3, kUpdNB>), g, b, 0, s, pl.args); break;
-    case 4: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 4, kUpdNB>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 8, kUpdNB>), g, b, 0, s, pl.args); break;
+    case 3: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 3, NB>), g, b, 0, s, pl.args); break;
+    case 4: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 4, NB>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 8, NB>), g, b, 0, s, pl.args); break;
     }
+}
+
+template <int DT, int W> void launch_update_vec_w(const UpdPlan &pl, hipStream_t s)
+{
+    if (pl.args.nb == kUpdNB) launch_update_vec_nb<DT, W, kUpdNB>(pl, s);
+    else launch_update_vec_nb<DT, W, 1>(pl, s);
 }
 
 template <int DT> void launch_update(const UpdPlan &pl, hipStream_t s)

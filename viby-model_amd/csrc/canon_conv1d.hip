@@ -25,10 +25,7 @@
 
 // build-time tuning knobs of the channel-contiguous prefill kernel
 #ifndef CANON_BLC_ROWS
-#define CANON_BLC_ROWS 4
-#endif
-#ifndef CANON_BLC_PREFETCH
-#define CANON_BLC_PREFETCH 1
+#define CANON_BLC_ROWS 8
 #endif
 
 namespace {
@@ -331,11 +328,14 @@ struct FwdArgs {
     int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
-    uint32_t nseg;      // bcl: segments per row       blc: time chunks per sequence
-    uint32_t chunk;     // blc/generic: time steps per chunk
-    uint32_t ntasks;    // bcl: wave tasks             blc/generic: threads
-    uint32_t nblocks;   // logical blocks (grid may be padded to a multiple of 8)
-    FastDiv div_nseg, div_C, div_nvec;
+    uint32_t nseg;      // bcl: segments per row       generic: time chunks per row
+    uint32_t chunk;     // generic: time steps per chunk
+    uint32_t ntasks;    // bcl: wave tasks   blc: blocks   generic: threads
+    uint32_t nblocks;   // blocks to launch
+    FastDiv div_nseg, div_C;
+    // blc: tiles
+    uint32_t nct, ntt;  // channel tiles per row, time tiles per sequence
+    FastDiv div_nct, div_ntt;
 };
 
 struct UpdArgs {
@@ -357,15 +357,6 @@ struct UpdArgs {
     uint32_t nthreads;
     FastDiv div_nvec;
 };
-
-// Blocks are dealt round-robin to the 8 XCDs, each with its own L2.  Give XCD k
-// the k-th contiguous eighth of the logical blocks, so blocks that are
-// neighbours in memory (and share halo rows) share an L2.
-__device__ __forceinline__ uint32_t xcd_block(uint32_t nblocks)
-{
-    const uint32_t per = (nblocks + 7u) >> 3;
-    return (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
-}
 
 // The activated, residual-added output of one element (fused rounding mode).
 __device__ __forceinline__ float finish(float acc, int act, int res_mode, float xm, float xr)
@@ -409,6 +400,23 @@ __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias,
                                            int w_dtype, bool vec, bool bvec, uint32_t c0, RawTaps<NC> &r)
 {
     const bool wide = w_dtype == CANON_DTYPE_F32;
+    // bias first: whatever follows the tap loads may wait on them, and nothing must be issued after a wait
+    if (bias) {
+        if (wide) {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
+        } else if (NC == 8 && bvec) {
+            // eight 16-bit biases are one aligned 16-byte run (c0 is a multiple of 8)
+            const uint4 q = *(const uint4 *)((const uint16_t *)bias + c0);
+            r.b[0] = q.x & 0xFFFFu; r.b[1 % NC] = q.x >> 16;
+            r.b[2 % NC] = q.y & 0xFFFFu; r.b[3 % NC] = q.y >> 16;
+            r.b[4 % NC] = q.z & 0xFFFFu; r.b[5 % NC] = q.z >> 16;
+            r.b[6 % NC] = q.w & 0xFFFFu; r.b[7 % NC] = q.w >> 16;
+        } else {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
+        }
+    }
     if (W == 4 && vec) {
         if (wide) {
             const uint4 *p = (const uint4 *)weight + c0;
@@ -443,22 +451,6 @@ __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias,
         for (int e = 0; e < NC; ++e)
 #pragma unroll
             for (int k = 0; k < W; ++k) r.w[e][k] = ((const uint16_t *)weight)[(int64_t)(c0 + e) * w_sc + k * w_sk];
-    }
-    if (bias) {
-        if (wide) {
-#pragma unroll
-            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
-        } else if (NC == 8 && bvec) {
-            // eight 16-bit biases are one aligned 16-byte run (c0 is a multiple of 8)
-            const uint4 q = *(const uint4 *)((const uint16_t *)bias + c0);
-            r.b[0] = q.x & 0xFFFFu; r.b[1 % NC] = q.x >> 16;
-            r.b[2 % NC] = q.y & 0xFFFFu; r.b[3 % NC] = q.y >> 16;
-            r.b[4 % NC] = q.z & 0xFFFFu; r.b[5 % NC] = q.z >> 16;
-            r.b[6 % NC] = q.w & 0xFFFFu; r.b[7 % NC] = q.w >> 16;
-        } else {
-#pragma unroll
-            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
-        }
     }
 }
 
@@ -650,13 +642,20 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 // prefill, channel-contiguous rows ([B, L, C] memory, x_stride_c == 1): the
 // layout CanonLayer hands over (a transposed view of [B, T, D]).
 //
-// One lane owns E adjacent channels and walks `chunk` time steps, keeping the
-// three previous (masked) rows in registers; a wave's loads are contiguous
-// 1 KB row pieces.  Rows are fetched R at a time so R loads are in flight.
+// One lane owns E adjacent channels (16 bytes of every row) and R consecutive
+// time steps; the four waves of a block own four consecutive R-row slabs of
+// the same 64-lane channel tile, so a block streams a [4R rows] x [1 KB] tile
+// and consecutive blocks sweep memory in address order (short-lived waves over
+// a compact window: measured to be what HBM wants; long per-lane time runs
+// lose 10-20 %).  The three rows a wave needs from before its slab are the
+// last three rows of the previous wave: each wave publishes the raw tail of
+// its slab in LDS, one barrier, the next wave picks it up -- only the first
+// wave of a block reads its halo from memory.  All loads (slab, halo, taps)
+// are issued before the first wait.
 // ---------------------------------------------------------------------------
 template <int DT, int W, bool MASK, bool NT>
 __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias, float (*hist)[Elem<DT>::per_vec],
-                                        const uint4 &X, float m, char *optr)
+                                        const uint4 &X, float m, char *optr, bool active)
 {
     constexpr int E = Elem<DT>::per_vec;
     float xr[E], xm_store[MASK ? E : 1], o[E];
@@ -689,60 +688,84 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] += xm[e];
     }
-    store_vec<NT>(optr, pack_vec<DT>(o));
+    if (active) store_vec<NT>(optr, pack_vec<DT>(o));
 }
+
+constexpr int kBlcWaves = 4;   // waves (time slabs) per block
 
 template <int DT, int W, int R, bool MASK, bool NT>
 __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
-    const uint32_t blk = xcd_block(a.nblocks);
-    if (blk >= a.nblocks) return;
-    const uint32_t tid = blk * 256u + threadIdx.x;
-    if (tid >= a.ntasks) return;
-    const uint32_t bc = fdiv(tid, a.div_nvec);
-    const uint32_t cv = tid - bc * a.nvec;
-    const uint32_t b = fdiv(bc, a.div_nseg);
-    const uint32_t ch = bc - b * a.nseg;
-    const uint32_t c0 = cv * E;
+    static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
+    __shared__ uint4 tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
+
+    const uint32_t blk = blockIdx.x;   // plain memory order (an XCD-contiguous remap measured 3 % slower here)
+    // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
+    const uint32_t bt = fdiv(blk, a.div_nct);
+    const uint32_t ct = blk - bt * a.nct;
+    const uint32_t b = fdiv(bt, a.div_ntt);
+    const uint32_t tt = bt - b * a.ntt;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t cv = ct * 64u + lane;
+    const bool active = cv < a.nvec;
+    const uint32_t c0 = (active ? cv : a.nvec - 1u) * E;   // idle lanes shadow the last vector, loads need no predicate
 
     const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * Elem<DT>::bytes;
     char *ob = a.out + ((int64_t)b * a.o_sb + c0) * Elem<DT>::bytes;
     const int64_t xs = a.x_sl * Elem<DT>::bytes, os = a.o_sl * Elem<DT>::bytes;
-    const int64_t t_begin = (int64_t)ch * a.chunk;
-    const int64_t t_stop = t_begin + (int64_t)a.chunk;
-    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+    const int64_t t0 = ((int64_t)tt * kBlcWaves + wv) * R;
+    const int64_t left = (int64_t)a.L - t0;
+    const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
+    const int64_t t_last = (int64_t)a.L - 1;
 
-    // the first batch of rows is requested before the history rows and the taps
-    uint4 X[R];
-    float m[R];
-    if (t_begin + R <= t_end) {
+    // slab rows, then (first wave only) the three rows before the block, then the taps.
+    // Rows past the end of the sequence are clamped to the last row (loaded, never used).
+    uint4 X[R], H[3];
+    float m[R], mh[3];
+    RawTaps<E> raw;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            X[r] = load_vec<NT>(xb + (t_begin + r) * xs);
-            m[r] = 0.0f;
-            if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + (t_begin + r) * a.m_sl, a.mask_dtype);
-        }
+    for (int r = 0; r < R; ++r) {
+        X[r] = make_uint4(0, 0, 0, 0);
+        m[r] = 0.0f;
     }
-
-    // the three rows before the chunk and the taps: requested now, consumed
-    // only after everything has been issued (one memory round trip, not four)
-    uint4 H[3];
-    float mh[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-        const int64_t t = t_begin - 3 + j;
         H[j] = make_uint4(0, 0, 0, 0);
         mh[j] = 0.0f;
-        if (j >= 3 - (W - 1) && t >= 0) {
-            H[j] = load_vec<false>(xb + t * xs);
-            if constexpr (MASK) mh[j] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
-        }
     }
-    RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+    if (rows > 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t0 + r < t_last ? t0 + r : t_last;
+            X[r] = load_vec<NT>(xb + t * xs);
+            if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int64_t t = t0 - 3 + j;
+            if (j >= 3 - (W - 1) && t >= 0) {
+                if (wv == 0) H[j] = load_vec<false>(xb + t * xs);
+                if constexpr (MASK) mh[j] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+            }
+        }
+        // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
+        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+    }
 
-    // hist[j] = masked row t_begin - 3 + j
+    // hand the raw tail of this slab to the next wave
+#pragma unroll
+    for (int j = 0; j < 3; ++j) tail[wv][j][lane] = X[R - 3 + j];
+    __syncthreads();
+    if (wv > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (j >= 3 - (W - 1)) H[j] = tail[wv - 1][j][lane];
+    }
+    if (rows == 0) return;   // after the barrier
+
+    // hist[j] = masked row t0 - 3 + j
     float hist[3][E];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
@@ -752,7 +775,7 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
             for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mh[j]);
         }
     }
-    if (t_begin == 0 && a.init) {
+    if (t0 == 0 && a.init && active) {
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
             if (j < 3 - (W - 1)) continue;
@@ -764,44 +787,16 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 
-    int64_t t = t_begin;
-    for (; t + R <= t_end; t += R) {
-        // request the next full batch before working on this one
-        uint4 Xn[R];
-        float mn[R];
-        const int64_t tn = t + R;
-        if (CANON_BLC_PREFETCH && tn + R <= t_end) {
+    if (rows == R) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                Xn[r] = load_vec<NT>(xb + (tn + r) * xs);
-                mn[r] = 0.0f;
-                if constexpr (MASK) mn[r] = load_mask(a.mask, b * a.m_sb + (tn + r) * a.m_sl, a.mask_dtype);
-            }
-        }
+        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+    } else {
 #pragma unroll
-        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t + r) * os);
-        if (CANON_BLC_PREFETCH) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                X[r] = Xn[r];
-                m[r] = mn[r];
-            }
-        } else if (tn + R <= t_end) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                X[r] = load_vec<NT>(xb + (tn + r) * xs);
-                if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + (tn + r) * a.m_sl, a.mask_dtype);
-            }
-        }
-    }
-    for (; t < t_end; ++t) {   // fewer than R rows left
-        const uint4 xv = load_vec<NT>(xb + t * xs);
-        float mv = 0.0f;
-        if constexpr (MASK) mv = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
-        blc_row<DT, W, MASK, NT>(a, w, bias, hist, xv, mv, ob + t * os);
+        for (int r = 0; r < R; ++r)
+            if (r < rows) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
     }
 
-    if (a.fin && ch == a.nseg - 1) {
+    if (a.fin && active && t0 + rows == (int64_t)a.L) {
         for (int slot = 0; slot < a.S_out; ++slot) {
             const int64_t t = (int64_t)a.L - a.S_out + slot;
             float v[E];
@@ -1124,7 +1119,7 @@ enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
-constexpr int kBlcRows = CANON_BLC_ROWS;           // rows per batch in the channel-contiguous kernel
+constexpr int kBlcRows = CANON_BLC_ROWS;   // time steps per wave in the channel-contiguous kernel
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work
 
@@ -1230,25 +1225,15 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     }
     if (blc_ok) {
         const uint32_t nvec = a.C / E;
-        // time steps per lane: a multiple of the rows-in-flight count, sized so
-        // that the launch has about 8 waves per CU
-        const uint64_t lanes_per_step = (uint64_t)a.B * nvec;
-        uint64_t want_chunks = (256ull * 8 * 64 + lanes_per_step - 1) / lanes_per_step;
-        if (want_chunks < 1) want_chunks = 1;
-        uint32_t chunk = (uint32_t)((a.L + want_chunks - 1) / want_chunks);
-        chunk = ((chunk + kBlcRows - 1) / kBlcRows) * kBlcRows;
-        if (chunk < 2 * kBlcRows) chunk = 2 * kBlcRows;
-#ifdef CANON_TUNING
-        if (const char *e = getenv("CANON_BLC_CHUNK")) chunk = (uint32_t)atoi(e);
-#endif
-        const uint32_t nseg = (a.L + chunk - 1) / chunk;
-        const uint64_t nthreads = lanes_per_step * nseg;
-        if (nthreads < (1ull << 31)) {
+        const uint32_t nct = (nvec + 63) / 64;                                   // channel tiles per row
+        const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
+        const uint64_t nblocks = (uint64_t)a.B * ntt * nct;
+        if (nblocks < (1ull << 31) - 8) {
             plan->kind = FWD_BLC;
-            a.nvec = nvec; a.nseg = nseg; a.chunk = chunk; a.ntasks = (uint32_t)nthreads;
-            a.div_nvec = make_fastdiv(nvec); a.div_nseg = make_fastdiv(nseg);
-            a.nblocks = (uint32_t)((nthreads + 255) / 256);
-            plan->grid = ((a.nblocks + 7) / 8) * 8;
+            a.nvec = nvec; a.nct = nct; a.ntt = ntt; a.ntasks = (uint32_t)nblocks;
+            a.div_nct = make_fastdiv(nct); a.div_ntt = make_fastdiv(ntt);
+            a.nblocks = (uint32_t)nblocks;
+            plan->grid = a.nblocks;
             return CANON_OK;
         }
     }

@@ -371,3 +371,28 @@ def test_errors_surface(cc):
         cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 2, device=DEV), w)
     with pytest.raises(NotImplementedError, match="backward"):
         cc.causal_conv1d_fn(x.requires_grad_(), w)
+
+
+def test_integer_mask_narrowing_is_never_stale(cc):
+    """Large problems convert an int64 mask to x.dtype once and reuse it while the same mask
+    object comes back; a changed or different mask must never hit the cached copy."""
+    g = torch.Generator().manual_seed(91)
+    B, C, L = 4, 512, 1024          # 2M elements: above the narrowing threshold
+    x = torch.randn(B, C, L, generator=g).bfloat16()
+    w = torch.randn(C, 4, generator=g).bfloat16()
+    xg, wg = x.to(DEV), w.to(DEV)
+    m1 = right_padded_mask([1024, 700, 300, 5], L)
+    m2 = right_padded_mask([10, 1024, 64, 999], L)
+    mg = m1.to(DEV)
+    for m_cpu in (m1, m1, m2):
+        if m_cpu is m2:
+            mg.copy_(m2.to(DEV))     # same tensor object and address, new content
+        got = cc.causal_conv1d_fn(xg, wg, attention_mask=mg, residual=True)
+        assert_parity(got, co.conv1d_fwd(x, w, None, mask=m_cpu, residual=1), exact=True, what="narrowed mask")
+    del mg
+    other = m1.to(DEV)               # may land on the freed address
+    got = cc.causal_conv1d_fn(xg, wg, attention_mask=other, residual=True)
+    assert_parity(got, co.conv1d_fwd(x, w, None, mask=m1, residual=1), exact=True, what="narrowed mask, new tensor")
+    sliced = torch.cat([m2, m1], dim=1).to(DEV)[:, -L:]      # a view, as CanonLayer slices it
+    got = cc.causal_conv1d_fn(xg, wg, attention_mask=sliced, residual=True)
+    assert_parity(got, co.conv1d_fwd(x, w, None, mask=m1, residual=1), exact=True, what="narrowed mask view")

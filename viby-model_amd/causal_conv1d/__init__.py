@@ -111,6 +111,30 @@ def _prep_bias(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[t
     return bias
 
 
+_NARROW_MIN_ELEMENTS = 1 << 20
+_narrow_cache = [None, None, None]   # key, the source mask (kept alive so its address stays unique), converted mask
+
+
+def _narrow_mask(mask: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """An integer mask wider than x's element type is converted to x.dtype once.
+
+    Every (batch, channel) row re-reads its batch row of the mask, so an int64
+    mask moves four times the bytes of bf16 data through the caches.  The
+    conversion is what the multiply does anyway (``x * mask`` promotes the
+    integer to x.dtype, ``model/model.py:455``; the reference wrapper casts the
+    mask the same way, ``causal_conv1d_mps/__init__.py:244-247``).  The result
+    is cached on the mask's identity because a model passes one mask to every
+    Canon call of a forward.  Small problems keep the caller's mask as is.
+    """
+    if (mask.dtype.is_floating_point or mask.element_size() <= x.element_size()
+            or x.numel() < _NARROW_MIN_ELEMENTS):
+        return mask
+    key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, x.dtype, mask.device)
+    if _narrow_cache[0] != key:
+        _narrow_cache[:] = [key, mask, mask.to(x.dtype)]
+    return _narrow_cache[2]
+
+
 def _stream(dev: torch.device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
@@ -208,6 +232,7 @@ def causal_conv1d_fn(
             raise ValueError(f"Unsupported attention mask dtype {attention_mask.dtype}")
         if attention_mask.device != x.device:
             raise ValueError("Attention mask must be on the same device as x")
+        attention_mask = _narrow_mask(attention_mask, x)
     width = weight.shape[1]
     if initial_states is not None:
         if initial_states.dim() != 3 or tuple(initial_states.shape[:2]) != (batch, dim):

@@ -179,6 +179,50 @@ template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint
     else *(u32x4_t *)p = q;
 }
 
+// N mask entries of consecutive time steps t_first .. t_first+N-1 (clamped to
+// [0, L-1]) of one batch row.  The element-type switch sits outside the loops
+// and every case is straight-line code, so all N loads are issued back to back
+// and waited for once (a per-entry switch puts a wait after every load, which
+// also waits for -- and so serialises -- the row loads issued before it).
+template <int N>
+__device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
+                                               int dt, float *m)
+{
+    int64_t idx[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        int64_t t = t_first + j;
+        t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+        idx[j] = row_base + t * stride;
+    }
+    switch (dt) {
+    case CANON_MASK_U8:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[idx[j]];
+        break;
+    case CANON_MASK_I32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[idx[j]];
+        break;
+    case CANON_MASK_I64:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int64_t *)p)[idx[j]];
+        break;
+    case CANON_MASK_F32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[idx[j]];
+        break;
+    case CANON_MASK_BF16:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, idx[j]);
+        break;
+    default:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, idx[j]);
+        break;
+    }
+}
+
 // (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
 // the value almost always fits 32 bits and one conversion instruction does it
 __device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
@@ -187,63 +231,94 @@ __device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
     return (float)(int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-// N (4 or 8) consecutive mask entries starting at element `base`.  The
-// element-type switch sits outside the loops; `vec` (decided on the host)
-// says the entries are contiguous and the run is aligned to its own size, so
-// it is fetched with a few wide loads instead of N narrow ones.
-template <int N>
-__device__ __forceinline__ void load_mask_vec(const void *p, int64_t base, int64_t stride, int dt, bool vec, float *m)
+// U runs of N (4 or 8) consecutive mask entries, run u starting at element
+// base[u].  The element-type switch sits outside the loops and every case is
+// straight-line code, so all loads are issued back to back and waited for
+// once.  `vec` (decided on the host) says the entries are contiguous and each
+// run is aligned to its own size: it is fetched with a few wide loads instead
+// of N narrow ones.
+template <int N, int U>
+__device__ __forceinline__ void load_mask_vec(const void *p, const int64_t *base, int64_t stride, int dt, bool vec,
+                                              float (*m)[N])
 {
     if (vec) {
         switch (dt) {
         case CANON_MASK_U8: {
-            uint32_t q[N / 4];
+            uint32_t q[U][N / 4];
 #pragma unroll
-            for (int i = 0; i < N / 4; ++i) q[i] = ((const uint32_t *)((const uint8_t *)p + base))[i];
+            for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int j = 0; j < N; ++j) m[j] = (float)((q[j / 4] >> (8 * (j % 4))) & 0xFFu);
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint32_t *)((const uint8_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < N; ++j) m[u][j] = (float)((q[u][j / 4] >> (8 * (j % 4))) & 0xFFu);
             return;
         }
         case CANON_MASK_I32: {
+            uint4 q[U][N / 4];
 #pragma unroll
-            for (int i = 0; i < N / 4; ++i) {
-                const uint4 q = ((const uint4 *)((const int32_t *)p + base))[i];
-                m[4 * i] = (float)(int32_t)q.x; m[4 * i + 1] = (float)(int32_t)q.y;
-                m[4 * i + 2] = (float)(int32_t)q.z; m[4 * i + 3] = (float)(int32_t)q.w;
-            }
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint4 *)((const int32_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) {
+                    m[u][4 * i] = (float)(int32_t)q[u][i].x; m[u][4 * i + 1] = (float)(int32_t)q[u][i].y;
+                    m[u][4 * i + 2] = (float)(int32_t)q[u][i].z; m[u][4 * i + 3] = (float)(int32_t)q[u][i].w;
+                }
             return;
         }
         case CANON_MASK_I64: {
+            uint4 q[U][N / 2];
 #pragma unroll
-            for (int i = 0; i < N / 2; ++i) {
-                const uint4 q = ((const uint4 *)((const int64_t *)p + base))[i];
-                m[2 * i] = i64_words_to_float(q.x, q.y);
-                m[2 * i + 1] = i64_words_to_float(q.z, q.w);
-            }
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) q[u][i] = ((const uint4 *)((const int64_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) {
+                    m[u][2 * i] = i64_words_to_float(q[u][i].x, q[u][i].y);
+                    m[u][2 * i + 1] = i64_words_to_float(q[u][i].z, q[u][i].w);
+                }
             return;
         }
         case CANON_MASK_F32: {
+            uint4 q[U][N / 4];
 #pragma unroll
-            for (int i = 0; i < N / 4; ++i) {
-                const uint4 q = ((const uint4 *)((const float *)p + base))[i];
-                m[4 * i] = bits_f(q.x); m[4 * i + 1] = bits_f(q.y); m[4 * i + 2] = bits_f(q.z); m[4 * i + 3] = bits_f(q.w);
-            }
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint4 *)((const float *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) {
+                    m[u][4 * i] = bits_f(q[u][i].x); m[u][4 * i + 1] = bits_f(q[u][i].y);
+                    m[u][4 * i + 2] = bits_f(q[u][i].z); m[u][4 * i + 3] = bits_f(q[u][i].w);
+                }
             return;
         }
         default: {   // bf16 / fp16
-            uint32_t q[N / 2];
-            if constexpr (N == 8) {
-                const uint4 v = *(const uint4 *)((const uint16_t *)p + base);
-                q[0] = v.x; q[1] = v.y; q[2 % (N / 2)] = v.z; q[3 % (N / 2)] = v.w;
-            } else {
-                const uint2 v = *(const uint2 *)((const uint16_t *)p + base);
-                q[0] = v.x; q[1] = v.y;
+            uint32_t q[U][N / 2];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if constexpr (N == 8) {
+                    const uint4 v = *(const uint4 *)((const uint16_t *)p + base[u]);
+                    q[u][0] = v.x; q[u][1] = v.y; q[u][2 % (N / 2)] = v.z; q[u][3 % (N / 2)] = v.w;
+                } else {
+                    const uint2 v = *(const uint2 *)((const uint16_t *)p + base[u]);
+                    q[u][0] = v.x; q[u][1] = v.y;
+                }
             }
 #pragma unroll
-            for (int i = 0; i < N / 2; ++i) {
-                if (dt == CANON_MASK_BF16) unpack2<CANON_DTYPE_BF16>(q[i], m[2 * i], m[2 * i + 1]);
-                else unpack2<CANON_DTYPE_F16>(q[i], m[2 * i], m[2 * i + 1]);
-            }
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) {
+                    if (dt == CANON_MASK_BF16) unpack2<CANON_DTYPE_BF16>(q[u][i], m[u][2 * i], m[u][2 * i + 1]);
+                    else unpack2<CANON_DTYPE_F16>(q[u][i], m[u][2 * i], m[u][2 * i + 1]);
+                }
             return;
         }
         }
@@ -251,27 +326,39 @@ __device__ __forceinline__ void load_mask_vec(const void *p, int64_t base, int64
     switch (dt) {
     case CANON_MASK_U8:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[base + j * stride];
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const uint8_t *)p)[base[u] + j * stride];
         break;
     case CANON_MASK_I32:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[base + j * stride];
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const int32_t *)p)[base[u] + j * stride];
         break;
     case CANON_MASK_I64:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const int64_t *)p)[base + j * stride];
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const int64_t *)p)[base[u] + j * stride];
         break;
     case CANON_MASK_F32:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[base + j * stride];
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = ((const float *)p)[base[u] + j * stride];
         break;
     case CANON_MASK_BF16:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, base + j * stride);
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = load1<CANON_DTYPE_BF16>(p, base[u] + j * stride);
         break;
     default:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, base + j * stride);
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = load1<CANON_DTYPE_F16>(p, base[u] + j * stride);
         break;
     }
 }
@@ -562,6 +649,18 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     RawTaps<1> raw;
     fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
 
+    // all mask entries of the segment, requested before anything is consumed
+    float M[MASK ? U : 1][E];
+    if constexpr (MASK) {
+        int64_t mbase[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t v = v0 + u * 64u;
+            mbase[u] = b * a.m_sb + (int64_t)(v < a.nvec ? v : a.nvec - 1u) * E * a.m_sl;   // idle lanes shadow the last vector
+        }
+        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+    }
+
     float w[1][W], bvv[1];
     decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
     const float bv = bvv[0];
@@ -593,12 +692,8 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
         float *xm = MASK ? xm_store : xr;
         unpack_vec<DT>(X[u], xr);
         if constexpr (MASK) {
-            float m[E];
 #pragma unroll
-            for (int j = 0; j < E; ++j) m[j] = 0.0f;
-            if (v < a.nvec) load_mask_vec<E>(a.mask, b * a.m_sb + (int64_t)v * E * a.m_sl, a.m_sl, a.mask_dtype, a.m_vec != 0, m);
-#pragma unroll
-            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], m[j]);
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
         }
         // seq[0..2] = the three masked inputs before this vector
         float seq[E + 3];
@@ -740,18 +835,25 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
         for (int r = 0; r < R; ++r) {
             const int64_t t = t0 + r < t_last ? t0 + r : t_last;
             X[r] = load_vec<NT>(xb + t * xs);
-            if constexpr (MASK) m[r] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
         }
+        if (wv == 0) {
 #pragma unroll
-        for (int j = 0; j < 3; ++j) {
-            const int64_t t = t0 - 3 + j;
-            if (j >= 3 - (W - 1) && t >= 0) {
-                if (wv == 0) H[j] = load_vec<false>(xb + t * xs);
-                if constexpr (MASK) mh[j] = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = t0 - 3 + j;
+                if (j >= 3 - (W - 1) && t >= 0) H[j] = load_vec<false>(xb + t * xs);
             }
         }
         // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
         fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+        if constexpr (MASK) {
+            // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
+            float mm[R + 3];
+            load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mm);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) mh[j] = mm[j];
+#pragma unroll
+            for (int r = 0; r < R; ++r) m[r] = mm[3 + r];
+        }
     }
 
     // hand the raw tail of this slab to the next wave

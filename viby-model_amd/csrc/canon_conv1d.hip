@@ -1055,11 +1055,23 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
             const uint4 *sp = (const uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
 #pragma unroll
             for (int k = 0; k < S; ++k) ST[n][k] = sp[k];
-            if (a.tmask) tm[n] = load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype);
         }
     }
     RawTaps<E> raw;
     fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+    if (a.tmask) {
+        // token masks last and in one go (one element-type switch, one wait)
+        int64_t mbase[NB];
+        float tmv[NB][1];
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = bg * NB + n;
+            mbase[n] = (int64_t)(b < a.B ? b : a.B - 1u) * a.m_sb;
+        }
+        load_mask_vec<1, NB>(a.tmask, mbase, 0, a.mask_dtype, false, tmv);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) tm[n] = tmv[n][0];
+    }
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 

@@ -2,10 +2,11 @@
  * canon_conv1d.h -- C ABI of the MI355X (gfx950) Canon causal depthwise conv1d.
  *
  * Two operators, the two calls Viby's CanonLayer makes into an accelerated
- * backend (reference = JohanLi233/Viby-Model):
+ * backend (reference = JohanLi233/Viby-Model), plus the backward of the first:
  *
  *   canon_conv1d_fwd     replaces  causal_conv1d_fn      (prefill)
  *   canon_conv1d_update  replaces  causal_conv1d_update  (one decode token)
+ *   canon_conv1d_bwd     gradient of canon_conv1d_fwd    (training)
  *
  * Plain pointers, sizes and element strides only; no framework types.  Every
  * pointer is a DEVICE pointer owned by the caller.  Kernels are enqueued on
@@ -154,6 +155,51 @@ typedef struct canon_conv1d_update_params {
     const int32_t *conv_state_indices;   /* upstream's batch indirection:    must be NULL */
 } canon_conv1d_update_params;
 
+/*
+ * Backward of canon_conv1d_fwd (no initial/final state): the gradient a
+ * training step needs so that the fused forward can stay on the accelerated
+ * path (trainer/base_trainer.py:274 calls backward through every Canon
+ * layer).  Same role as the reference's own backward kernels
+ * (causal_conv1d_mps/autograd.py:116-151 and :305-338,
+ * causal_conv1d.metal:803-958, 1354-1735), which return dx, dweight, dbias.
+ *
+ * With z = bias + conv(xm), xm = x * mask, out = act(z) (+ xm | + x):
+ *   dz[t]  = dout[t] * act'(z[t])                         (z is recomputed from x)
+ *   dxm[t] = sum_k weight[k] * dz[t + (W-1) - k]  (+ dout[t] for RESIDUAL_MASKED)
+ *   dx[t]  = dxm[t] * mask[t]                     (+ dout[t] for RESIDUAL_UNMASKED)
+ *   dweight[c,k] = sum_{b,t} dz[b,c,t] * xm[b,c,t-(W-1)+k],   dbias[c] = sum_{b,t} dz[b,c,t]
+ * All arithmetic in fp32; dx is rounded once to the storage type.  dweight and
+ * dbias are fp32, OVERWRITTEN (not accumulated into), and reduced in a fixed
+ * order in two stages through `workspace` (no float atomics: results are
+ * reproducible run to run).
+ */
+typedef struct canon_conv1d_bwd_params {
+    uint32_t struct_size;           /* sizeof(canon_conv1d_bwd_params) */
+    int32_t x_dtype;                /* x, dout, dx */
+    int32_t w_dtype;                /* weight and bias as used by the forward */
+    int32_t mask_dtype;
+    int32_t width;
+    int32_t activation;
+    int32_t residual_mode;
+    int32_t reserved0;
+    int64_t batch, channels, seqlen;
+    const void *x;
+    int64_t x_stride_b, x_stride_c, x_stride_l;
+    const void *dout;
+    int64_t dout_stride_b, dout_stride_c, dout_stride_l;
+    void *dx;                       /* must not alias x or dout */
+    int64_t dx_stride_b, dx_stride_c, dx_stride_l;
+    const void *weight;
+    int64_t w_stride_c, w_stride_k;
+    const void *bias;               /* or NULL */
+    const void *mask;               /* or NULL */
+    int64_t mask_stride_b, mask_stride_l;
+    float *dweight;                 /* [channels, width] contiguous fp32 */
+    float *dbias;                   /* [channels] fp32, or NULL */
+    void *workspace;                /* canon_conv1d_bwd_workspace_bytes() bytes, 16-byte aligned */
+    int64_t workspace_bytes;
+} canon_conv1d_bwd_params;
+
 int canon_conv1d_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none). */
@@ -162,6 +208,11 @@ const char *canon_conv1d_last_error(void);
 /* Enqueue on `stream` (a hipStream_t; NULL = the default stream). */
 int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream);
 int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
+int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream);
+
+/* Scratch bytes canon_conv1d_bwd needs for these sizes and strides (the
+ * pointers in *p are not read); negative if the arguments are rejected. */
+int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
 
 /*
  * Name of the kernel family the call above would launch for these arguments
@@ -171,6 +222,7 @@ int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
  */
 const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p);
 const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p);
+const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p);   /* "bwd_blc_vec" | "bwd_bcl_vec" | "bwd_generic" */
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@ HEADER = os.path.join(ROOT, "include", "canon_conv1d.h")
 
 import causal_conv1d as cc                      # noqa: E402
 from causal_conv1d import _lib                  # noqa: E402
-from causal_conv1d._lib import FwdParams, UpdateParams  # noqa: E402
+from causal_conv1d._lib import BwdParams, FwdParams, UpdateParams  # noqa: E402
 
 
 def test_library_exports_every_declared_function():
@@ -39,7 +39,9 @@ def test_library_exports_every_declared_function():
 
 def test_ctypes_structs_match_the_header(tmp_path):
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){']
-    for cname, cls in (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams)):
+    structs = (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams),
+               ("canon_conv1d_bwd_params", BwdParams))
+    for cname, cls in structs:
         lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')
         for fname, _ in cls._fields_:
             lines.append(f'printf("{cname} {fname} %zu\\n", offsetof({cname}, {fname}));')
@@ -50,7 +52,7 @@ def test_ctypes_structs_match_the_header(tmp_path):
     subprocess.check_call(["gcc", "-o", str(exe), str(src)])
     out = subprocess.check_output([str(exe)], text=True).split("\n")
     got = {tuple(l.split()[:2]): int(l.split()[2]) for l in out if l}
-    for cname, cls in (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams)):
+    for cname, cls in structs:
         assert got[(cname, "size")] == ctypes.sizeof(cls)
         for fname, _ in cls._fields_:
             assert got[(cname, fname)] == getattr(cls, fname).offset, (cname, fname)
@@ -245,3 +247,38 @@ def test_canon_layer_module_mirrors_the_reference_class():
     assert nobias._slot(cache) is cache.canon_cache_a and len(cache.canon_cache_a) == 18
     with pytest.raises(ValueError, match="must be on a ROCm GPU device"):
         layer(torch.randn(1, 4, 640))
+
+
+def bwd_params(B=8, C=3456, L=1024, layout="blc", dtype=1, **over):
+    p = BwdParams()
+    p.struct_size = ctypes.sizeof(BwdParams)
+    p.x_dtype = p.w_dtype = dtype
+    p.width = 4
+    p.batch, p.channels, p.seqlen = B, C, L
+    p.x, p.dout, p.dx, p.weight, p.dweight = FAKE_X, FAKE_OUT, FAKE_STATE, FAKE_W, FAKE_W + 0x100000
+    strides = (C * L, L, 1) if layout == "bcl" else (C * L, 1, C)
+    for name in ("x", "dout", "dx"):
+        for s, v in zip(("b", "c", "l"), strides):
+            setattr(p, f"{name}_stride_{s}", v)
+    p.w_stride_c, p.w_stride_k = 4, 1
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_bwd_plan_and_workspace():
+    L = _lib.lib()
+    p = bwd_params()
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(p)) == b"bwd_blc_vec"
+    ws = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(p))
+    assert 0 < ws <= 20 << 20 and ws % (3456 * 5 * 4) == 0        # whole partial sets, bounded scratch
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl"))) == b"bwd_generic"
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(C=3457))) == b"bwd_generic"
+    assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(width=9))) == -1
+    assert "width 9" in last_error()
+    assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(B=0))) == 0
+    # the launching call validates what the planner cannot: pointers and the scratch itself
+    assert L.canon_conv1d_bwd(ctypes.byref(bwd_params(workspace=0)), None) == _lib.ERR_INVALID_ARGUMENT
+    assert "workspace" in last_error()
+    assert L.canon_conv1d_bwd(ctypes.byref(bwd_params(dx=FAKE_X)), None) == _lib.ERR_INVALID_ARGUMENT
+    assert "alias" in last_error()

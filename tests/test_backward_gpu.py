@@ -1,0 +1,185 @@
+"""Backward of the prefill (dx, dweight, dbias) against torch autograd of the reference's eager
+formulation (oracle/canon_grad.py, float64), by finite differences as the reference's own tests
+do (causal-conv1d-mps/test.py:8-80, 259-291), and through the drop-in CanonLayer."""
+import itertools
+import types
+
+import pytest
+import torch
+
+from helpers import bits, right_padded_mask
+from oracle.canon_grad import conv1d_grads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def cc():
+    import causal_conv1d
+    return causal_conv1d
+
+
+def gpu_grads(cc, x_cpu, w, b, dout_cpu, layout, mask=None, act=None, residual=False):
+    xg = x_cpu.to(DEV)
+    dg = dout_cpu.to(DEV)
+    if layout == "blc":
+        xg = xg.transpose(1, 2).contiguous().transpose(1, 2)
+        dg = dg.transpose(1, 2).contiguous().transpose(1, 2)
+    xg.requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True) if b is not None else None
+    out = cc.causal_conv1d_fn(xg, wg, bg, activation=act,
+                              attention_mask=None if mask is None else mask.to(DEV), residual=residual)
+    out.backward(dg)
+    torch.cuda.synchronize()
+    return xg.grad, wg.grad, (bg.grad if bg is not None else None), out.detach()
+
+
+def check(got, want64, dtype, what, sum_terms=1):
+    """dx-like tensors: fp32 to 2e-5 of the tensor's scale; 16-bit to 1 ulp of the rounded float64
+    value.  Sums over `sum_terms` products are compared relative to the magnitude of the sum."""
+    got = got.detach().cpu()
+    if sum_terms > 1:
+        # fp32 accumulation in a fixed order vs exact: 1e-4 of the tensor's scale; a 16-bit result is
+        # additionally rounded once to its storage type (one ulp of its own value)
+        scale = want64.abs().max().item() + 1e-30
+        ulp = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+        err = (got.double() - want64).abs()
+        bound = 1e-4 * scale + ulp * want64.abs()
+        assert bool((err <= bound).all()), f"{what}: worst excess {(err - bound).max().item():.3e} (scale {scale:.3e})"
+    elif dtype == torch.float32:
+        scale = want64.abs().max().item() + 1e-30
+        err = (got.double() - want64).abs().max().item() / scale
+        assert err <= 2e-5, f"{what}: {err:.3e}"
+    else:
+        # one rounding to the storage type of a value computed in fp32 from a handful of terms that
+        # may cancel: one ulp of the value plus 1e-5 of the tensor's scale
+        scale = want64.abs().max().item() + 1e-30
+        ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+        err = (got.double() - want64).abs()
+        bound = ulp * want64.abs() + 1e-5 * scale
+        assert bool((err <= bound).all()), f"{what}: worst excess {(err - bound).max().item():.3e} (scale {scale:.3e})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["bcl", "blc"])
+def test_backward_matches_autograd_of_the_eager_formulation(cc, dtype, layout):
+    g = torch.Generator().manual_seed(17)
+    shapes = [(2, 16, 40), (3, 24, 129), (1, 8, 5), (2, 40, 3), (4, 64, 256)]
+    for (B, C, L), W in itertools.product(shapes, [2, 3, 4]):
+        for has_bias, act, residual, has_mask in [(False, None, False, False), (True, "silu", "masked", True),
+                                                  (True, None, "unmasked", True), (False, "silu", True, False)]:
+            x = torch.randn(B, C, L, generator=g).to(dtype)
+            w = (torch.randn(C, W, generator=g) * 0.5).to(dtype)
+            b = (torch.randn(C, generator=g) * 0.2).to(dtype) if has_bias else None
+            dout = torch.randn(B, C, L, generator=g).to(dtype)
+            mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L) if has_mask else None
+            dx, dw, db, out = gpu_grads(cc, x, w, b, dout, layout, mask, act, residual)
+            rdx, rdw, rdb, _ = conv1d_grads(x, w, b, dout, mask, act, residual)
+            what = f"{dtype} {layout} {B}x{C}x{L} W{W} bias{has_bias} {act} {residual} mask{has_mask}"
+            assert dx.stride() == (x.to(DEV).stride() if layout == "bcl" else dx.stride())
+            check(dx, rdx, dtype, what + " dx")
+            check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
+            if has_bias:
+                check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
+def test_backward_finite_differences_like_the_reference_tests(cc):
+    """causal-conv1d-mps/test.py:259-272 and :275-291: eps 1e-3, atol 1e-3, rtol 1e-2, loss = out.sum()."""
+    torch.manual_seed(0)
+    for layout, (B, C, L) in itertools.product(["bcl", "blc"], [(2, 8, 16)]):
+        x = torch.randn(B, C, L, device=DEV)
+        if layout == "blc":
+            x = x.transpose(1, 2).contiguous().transpose(1, 2)
+        w = torch.randn(C, 4, device=DEV)
+        b = torch.randn(C, device=DEV)
+        mask = torch.ones(B, L, device=DEV)
+        mask[1, 11:] = 0
+        params = [x, w, b]
+
+        def f():
+            return cc.causal_conv1d_fn(x, w, b, activation="silu", attention_mask=mask, residual="unmasked")
+
+        for p in params:
+            p.requires_grad_(True)
+            p.grad = None
+        f().sum().backward()
+        analytic = [p.grad.clone() for p in params]
+        eps = 1e-3
+        with torch.no_grad():
+            for p, a in zip(params, analytic):
+                num = torch.zeros_like(p)
+                flat, nflat = p.view(-1) if p.is_contiguous() else None, None
+                idx = list(itertools.product(*[range(s) for s in p.shape]))
+                for i in idx:
+                    old = p[i].item()
+                    p[i] = old + eps
+                    lp = f().double().sum().item()
+                    p[i] = old - eps
+                    lm = f().double().sum().item()
+                    p[i] = old
+                    num[i] = (lp - lm) / (2 * eps)
+                assert torch.allclose(a, num, atol=1e-3, rtol=1e-2), (layout, (a - num).abs().max().item())
+
+
+@pytest.mark.parametrize("layout", ["blc", "bcl"])
+def test_backward_at_model_shape_is_deterministic_and_correct(cc, layout):
+    g = torch.Generator().manual_seed(23)
+    B, C, L = 4, 3456, 1024                      # Canon-D channel count, BASELINE sequence length
+    x = torch.randn(B, C, L, generator=g).bfloat16()
+    w = (torch.randn(C, 4, generator=g) * 0.3).bfloat16()
+    b = (torch.randn(C, generator=g) * 0.1).bfloat16()
+    dout = torch.randn(B, C, L, generator=g).bfloat16()
+    mask = right_padded_mask([1024, 800, 333, 128], L)
+    dx, dw, db, _ = gpu_grads(cc, x, w, b, dout, layout, mask, None, "masked")
+    dx2, dw2, db2, _ = gpu_grads(cc, x, w, b, dout, layout, mask, None, "masked")
+    assert torch.equal(bits(dx), bits(dx2)) and torch.equal(bits(dw), bits(dw2)) and torch.equal(bits(db), bits(db2))
+    rdx, rdw, rdb, _ = conv1d_grads(x, w, b, dout, mask, None, "masked")
+    check(dx, rdx, torch.bfloat16, "model shape dx")
+    check(dw, rdw, torch.bfloat16, "model shape dweight", sum_terms=B * L)
+    check(db, rdb, torch.bfloat16, "model shape dbias", sum_terms=B * L)
+    # fp32 master weights with bf16 activations (autocast-style): gradients come back in fp32
+    xg = x.to(DEV).requires_grad_(True)
+    w32 = w.float().to(DEV).requires_grad_(True)
+    cc.causal_conv1d_fn(xg, w32, None, residual=True).backward(dout.to(DEV))
+    assert w32.grad.dtype == torch.float32
+    rdx, rdw, _, _ = conv1d_grads(x, w.float(), None, dout, None, None, 1)
+    check(w32.grad, rdw, torch.float32, "fp32 weight grad", sum_terms=B * L)
+
+
+def test_canon_layer_trains(cc):
+    """One SGD step through the drop-in CanonLayer equals the same step through the eager restatement."""
+    from causal_conv1d.canon import CanonLayer
+    from oracle.canon_eager import EagerCanon
+    torch.manual_seed(3)
+    B, T, D = 3, 64, 96
+    cfg = types.SimpleNamespace(canon_kernel=4, canon_bias=True, canon_activation=True)
+    layer = CanonLayer(D, cfg, "a").to(DEV)
+    layer.reset_parameters()
+    x = torch.randn(B, T, D)
+    mask = right_padded_mask([64, 40, 9], T)
+    target = torch.randn(B, T, D)
+    xg = x.to(DEV).requires_grad_(True)
+    loss = ((layer(xg, attention_mask=mask.to(DEV)) - target.to(DEV)) ** 2).mean()
+    loss.backward()
+    w_ref = layer.weight.detach().cpu().double().requires_grad_(True)
+    b_ref = layer.bias_param.detach().cpu().double().requires_grad_(True)
+    x_ref = x.double().requires_grad_(True)
+    ref_out = EagerCanon(w_ref, b_ref, True).forward(x_ref, mask.double())
+    ((ref_out - target.double()) ** 2).mean().backward()
+    torch.testing.assert_close(loss.item(), ((ref_out - target.double()) ** 2).mean().item(), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(xg.grad.cpu().double(), x_ref.grad, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(layer.weight.grad.cpu().double(), w_ref.grad, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(layer.bias_param.grad.cpu().double(), b_ref.grad, rtol=1e-4, atol=1e-7)
+
+
+def test_unsupported_gradients_raise(cc):
+    x = torch.randn(2, 8, 16, device=DEV, requires_grad=True)
+    w = torch.randn(8, 4, device=DEV)
+    with pytest.raises(NotImplementedError, match="initial_states"):
+        cc.causal_conv1d_fn(x, w, initial_states=torch.zeros(2, 8, 3, device=DEV))
+    with pytest.raises(NotImplementedError, match="backward of the decode step"):
+        cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 4, device=DEV), w)
+    out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
+    assert out.requires_grad and not fs.requires_grad

@@ -73,8 +73,8 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
 def _no_grad_needed(*tensors) -> None:
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise NotImplementedError(
-            "causal_conv1d (gfx950): backward is not implemented; call under torch.no_grad() "
-            "or detach the inputs")
+            "causal_conv1d_update (gfx950): backward of the decode step is not implemented; call under "
+            "torch.no_grad() or detach the inputs")
 
 
 def _check_shapes(x_dim: int, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
@@ -219,7 +219,6 @@ def causal_conv1d_fn(
     _check_shapes(dim, weight, bias)
     _require_gpu(x, "Input tensor")
     _check_devices(weight, bias, x.device)
-    _no_grad_needed(x, weight, bias, initial_states)
     bias = _prep_bias(weight, bias)
 
     if attention_mask is not None:
@@ -253,17 +252,97 @@ def causal_conv1d_fn(
 
     if x.stride(2) != 1 and x.stride(1) != 1:
         x = x.contiguous()
+    if x.numel() == 0 and final_states is not None and final_states.numel():
+        raise ValueError("cannot produce final states from an empty input")
+
+    if _wants_grad(x, weight, bias):
+        if initial_states is not None:
+            raise NotImplementedError("gradients through a call with initial_states are not implemented")
+        result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd)
+    else:
+        result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+        if final_states is not None:
+            result = (result, final_states)
+    return result
+
+
+def _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd) -> torch.Tensor:
     out = torch.empty_like(x)
     if x.numel() == 0:
-        if final_states is not None and final_states.numel():
-            raise ValueError("cannot produce final states from an empty input")
-        return out if final_states is None else (out, final_states)
-
-    p = _fill_fwd(x, out, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+        return out
+    p = _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd)
     with torch.cuda.device(x.device):
         rc = _lib.lib().canon_conv1d_fwd(ctypes.byref(p), _stream(x.device))
     _lib.check(rc, "causal_conv1d_fn")
-    return out if final_states is None else (out, final_states)
+    return out
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+class _CanonConvFn(torch.autograd.Function):
+    """Autograd node of the prefill: forward and backward are one fused launch each
+    (the backward recomputes the pre-activation from x, nothing but the inputs is saved).
+    Mirrors the role of CausalConv1dMPSFunction / ShortConvFusedMPSFunction
+    (causal_conv1d_mps/autograd.py:13-160, 162-338)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd):
+        out = _launch_fwd(x, weight, bias, mask, None, final_states, act, res, rnd)
+        ctx.save_for_backward(x, weight, bias, mask)
+        ctx.flags = (act, res)
+        if final_states is not None:
+            ctx.mark_non_differentiable(final_states)
+            return out, final_states
+        return out
+
+    @staticmethod
+    def backward(ctx, dout, *unused):
+        x, weight, bias, mask = ctx.saved_tensors
+        act, res = ctx.flags
+        if dout.dtype != x.dtype:
+            dout = dout.to(x.dtype)
+        if dout.stride() != x.stride():
+            dout = torch.empty_like(x).copy_(dout)       # same layout as x: keeps the vector kernel
+        dx = torch.empty_like(x)
+        channels, width = weight.shape
+        dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
+        dbias = torch.empty(channels, dtype=torch.float32, device=x.device) if bias is not None else None
+        p = _lib.BwdParams()
+        p.struct_size = ctypes.sizeof(_lib.BwdParams)
+        p.x_dtype = _lib.DTYPE_CODE[x.dtype]
+        p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
+        p.width = width
+        p.activation, p.residual_mode = act, res
+        p.batch, p.channels, p.seqlen = x.shape
+        p.x = x.data_ptr()
+        p.x_stride_b, p.x_stride_c, p.x_stride_l = x.stride()
+        p.dout = dout.data_ptr()
+        p.dout_stride_b, p.dout_stride_c, p.dout_stride_l = dout.stride()
+        p.dx = dx.data_ptr()
+        p.dx_stride_b, p.dx_stride_c, p.dx_stride_l = dx.stride()
+        p.weight = weight.data_ptr()
+        p.w_stride_c, p.w_stride_k = weight.stride()
+        p.bias = bias.data_ptr() if bias is not None else None
+        if mask is not None:
+            p.mask = mask.data_ptr()
+            p.mask_dtype = _lib.MASK_CODE[mask.dtype]
+            p.mask_stride_b, p.mask_stride_l = mask.stride()
+        p.dweight = dweight.data_ptr()
+        p.dbias = dbias.data_ptr() if dbias is not None else None
+        L = _lib.lib()
+        nbytes = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(p))
+        if nbytes < 0:
+            _lib.check(_lib.ERR_INVALID_ARGUMENT, "causal_conv1d_fn backward")
+        workspace = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=x.device)
+        p.workspace = workspace.data_ptr()
+        p.workspace_bytes = workspace.numel()
+        with torch.cuda.device(x.device):
+            rc = L.canon_conv1d_bwd(ctypes.byref(p), _stream(x.device))
+        _lib.check(rc, "causal_conv1d_fn backward")
+        return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
+                None, None, None, None, None)
 
 
 def _fill_update(x2, out2, conv_state, weight, bias, token_mask, act, res, rnd) -> UpdateParams:

@@ -61,6 +61,23 @@ class UpdateParams(ctypes.Structure):
     ]
 
 
+class BwdParams(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", _u32),
+        ("x_dtype", _i32), ("w_dtype", _i32), ("mask_dtype", _i32),
+        ("width", _i32), ("activation", _i32), ("residual_mode", _i32), ("reserved0", _i32),
+        ("batch", _i64), ("channels", _i64), ("seqlen", _i64),
+        ("x", _vp), ("x_stride_b", _i64), ("x_stride_c", _i64), ("x_stride_l", _i64),
+        ("dout", _vp), ("dout_stride_b", _i64), ("dout_stride_c", _i64), ("dout_stride_l", _i64),
+        ("dx", _vp), ("dx_stride_b", _i64), ("dx_stride_c", _i64), ("dx_stride_l", _i64),
+        ("weight", _vp), ("w_stride_c", _i64), ("w_stride_k", _i64),
+        ("bias", _vp),
+        ("mask", _vp), ("mask_stride_b", _i64), ("mask_stride_l", _i64),
+        ("dweight", _vp), ("dbias", _vp),
+        ("workspace", _vp), ("workspace_bytes", _i64),
+    ]
+
+
 EXPORTS = (
     "canon_conv1d_abi_version",
     "canon_conv1d_last_error",
@@ -68,6 +85,9 @@ EXPORTS = (
     "canon_conv1d_update",
     "canon_conv1d_fwd_plan",
     "canon_conv1d_update_plan",
+    "canon_conv1d_bwd",
+    "canon_conv1d_bwd_workspace_bytes",
+    "canon_conv1d_bwd_plan",
 )
 
 _lib = None
@@ -94,6 +114,12 @@ def lib() -> ctypes.CDLL:
         L.canon_conv1d_fwd_plan.argtypes = [ctypes.POINTER(FwdParams)]
         L.canon_conv1d_update_plan.restype = ctypes.c_char_p
         L.canon_conv1d_update_plan.argtypes = [ctypes.POINTER(UpdateParams)]
+        L.canon_conv1d_bwd.restype = ctypes.c_int
+        L.canon_conv1d_bwd.argtypes = [ctypes.POINTER(BwdParams), _vp]
+        L.canon_conv1d_bwd_workspace_bytes.restype = ctypes.c_int64
+        L.canon_conv1d_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdParams)]
+        L.canon_conv1d_bwd_plan.restype = ctypes.c_char_p
+        L.canon_conv1d_bwd_plan.argtypes = [ctypes.POINTER(BwdParams)]
         got = L.canon_conv1d_abi_version()
         if got != ABI_VERSION:
             raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}")

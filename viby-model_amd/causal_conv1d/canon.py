@@ -26,8 +26,10 @@ package is installed and the one the parity vectors come from:
 ``rounding='eager'`` reproduces that branch's intermediate bf16/fp16 roundings
 bit for bit; the default ``'fused'`` rounds once.
 
-Forward only: with gradients enabled and parameters that require them the
-underlying calls raise (use ``torch.no_grad()`` / ``torch.inference_mode()``).
+Training: a block call without a cache is differentiable (fused backward
+kernel); the cached paths (prefill with state capture continues to work, the
+single-token step does not) are inference paths: run them under
+``torch.no_grad()`` / ``torch.inference_mode()``.
 """
 from __future__ import annotations
 

@@ -20,6 +20,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <type_traits>
 
 #include "canon_conv1d.h"
 
@@ -995,6 +996,271 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// backward of the prefill: dx, and per-chunk partial sums of dweight / dbias
+//
+// One lane owns E channels and walks a chunk of time steps from its END to its
+// start: dx[t] needs dz[t .. t+W-1] (the three later steps are carried in
+// registers), z[t] needs xm[t-3 .. t] (a sliding window refilled with one row
+// per step, fetched R rows ahead).  The three dz values just past the chunk are
+// recomputed from memory.  dweight / dbias accumulate in registers over the
+// chunk and go to partial[(b * nchunk + chunk) * C + c][5] (w0..w3, bias);
+// canon_bwd_reduce_kernel sums the partial sets in a fixed order.
+//   VEC:  channel-contiguous tensors, E = elements per 16 bytes, vector access
+//   !VEC: E = 1, any strides (the fallback for every other layout)
+// ---------------------------------------------------------------------------
+struct BwdArgs {
+    const char *x;
+    const char *dy;
+    char *dx;
+    const void *weight;
+    const void *bias;
+    const void *mask;
+    float *partial;
+    float *dweight;
+    float *dbias;
+    int64_t x_sb, x_sc, x_sl;
+    int64_t g_sb, g_sc, g_sl;
+    int64_t d_sb, d_sc, d_sl;
+    int64_t w_sc, w_sk;
+    int64_t m_sb, m_sl;
+    uint32_t B, C, L;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_vec;
+    uint32_t nvec;      // channel groups per row (C / E)
+    uint32_t nchunk;    // time chunks per sequence
+    uint32_t chunk;     // time steps per chunk
+    uint32_t nthreads;
+    uint32_t nsets;     // partial sets = B * nchunk
+    FastDiv div_nvec, div_nchunk;
+};
+
+__device__ __forceinline__ float silu_grad(float z)
+{
+    const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+    return s * (1.0f + z * (1.0f - s));
+}
+
+template <int DT, int E, bool VEC>
+__device__ __forceinline__ void bwd_load_row(const char *base, int64_t row_off, int64_t sc, float *f)
+{
+    // E values of one time step; VEC: 16 contiguous bytes at base + row_off (bytes)
+    if constexpr (VEC) {
+        unpack_vec<DT>(load_vec<false>(base + row_off), f);
+    } else {
+        f[0] = load1<DT>(base + row_off, 0);
+    }
+}
+
+template <int DT, int W, int E, bool VEC, bool MASK, int R>
+__global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
+{
+    constexpr int BY = Elem<DT>::bytes;
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.nthreads) return;
+    const uint32_t bc = fdiv(tid, a.div_nvec);
+    const uint32_t cv = tid - bc * a.nvec;
+    const uint32_t b = fdiv(bc, a.div_nchunk);
+    const uint32_t ch = bc - b * a.nchunk;
+    const uint32_t c0 = cv * E;
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + (int64_t)c0 * a.x_sc) * BY;
+    const char *gb = a.dy + ((int64_t)b * a.g_sb + (int64_t)c0 * a.g_sc) * BY;
+    char *db_ = a.dx + ((int64_t)b * a.d_sb + (int64_t)c0 * a.d_sc) * BY;
+    const int64_t xs = a.x_sl * BY, gs = a.g_sl * BY, ds = a.d_sl * BY;
+    const int64_t t_begin = (int64_t)ch * a.chunk;
+    const int64_t t_stop = t_begin + (int64_t)a.chunk;
+    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+    const int64_t Lm1 = (int64_t)a.L - 1;
+
+    RawTaps<E> raw;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, VEC && a.w_vec != 0, VEC && a.b_vec != 0, c0, raw);
+
+    // rows t_end-4 .. t_end+2 of xm (window for the last step + the three steps past the chunk)
+    float xr7[7][E], m7[7];
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+        const int64_t t = t_end - 4 + j;
+        const int64_t tc = t < 0 ? 0 : (t > Lm1 ? Lm1 : t);
+        bwd_load_row<DT, E, VEC>(xb, tc * xs, a.x_sc, xr7[j]);
+        m7[j] = 1.0f;
+    }
+    float g3[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int64_t t = t_end + j;
+        bwd_load_row<DT, E, VEC>(gb, (t > Lm1 ? Lm1 : t) * gs, a.g_sc, g3[j]);
+    }
+    if constexpr (MASK) load_mask_rows<7>(a.mask, (int64_t)b * a.m_sb, t_end - 4, a.L, a.m_sl, a.mask_dtype, m7);
+
+    float w[E][W], bias[E];
+    decode_taps<DT, W, E>(raw, a.w_dtype, VEC && a.w_vec != 0, a.bias != nullptr, w, bias);
+
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+        const int64_t t = t_end - 4 + j;
+        const bool inside = t >= 0 && t <= Lm1;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float v = MASK ? mul_round<DT>(xr7[j][e], m7[j]) : xr7[j][e];
+            xr7[j][e] = inside ? v : 0.0f;
+        }
+    }
+    // dzf[j] = dz[t_end + j]
+    float dzf[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const bool inside = t_end + j <= Lm1;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float z = bias[e];
+#pragma unroll
+            for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xr7[j + 1 + (4 - W) + k][e], z);   // xm[t_end+j-(W-1)+k]
+            const float d = a.act ? g3[j][e] * silu_grad(z) : g3[j][e];
+            dzf[j][e] = inside ? d : 0.0f;
+        }
+    }
+    // xw[k] = xm[t-3+k] for the step being processed, starting with t = t_end - 1
+    float xw[4][E];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) xw[k][e] = xr7[k][e];
+
+    float dw[E][W], dbs[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        dbs[e] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) dw[e][k] = 0.0f;
+    }
+
+    for (int64_t t_hi = t_end - 1; t_hi >= t_begin; t_hi -= R) {
+        // this batch: steps t_hi, t_hi-1, .., t_hi-R+1; needs dout of those steps and x rows t-4.
+        // Rows are kept as loaded (raw) until their step, to keep the register count down.
+        typename std::conditional<VEC, uint4, float>::type G[R], XN[R];
+        float mk[R], mn[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t_hi - r;
+            const int64_t tg = t < 0 ? 0 : t;
+            const int64_t tn = t - 4 < 0 ? 0 : t - 4;
+            if constexpr (VEC) {
+                G[r] = load_vec<false>(gb + tg * gs);
+                XN[r] = load_vec<false>(xb + tn * xs);
+            } else {
+                G[r] = load1<DT>(gb + tg * gs, 0);
+                XN[r] = load1<DT>(xb + tn * xs, 0);
+            }
+            mk[r] = 1.0f;
+            mn[r] = 1.0f;
+        }
+        if constexpr (MASK) {
+            // masks of steps t_hi-R+1 .. t_hi (for dx) and of rows t_hi-R-3 .. t_hi-4 (for the window)
+            float mm[R + 4];
+            load_mask_rows<R + 4>(a.mask, (int64_t)b * a.m_sb, t_hi - R - 3, a.L, a.m_sl, a.mask_dtype, mm);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                mk[r] = mm[R + 3 - r];      // step t_hi - r
+                mn[r] = mm[R - 1 - r];      // row  t_hi - r - 4
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t_hi - r;
+            if (t < t_begin) break;
+            float g[E], xn[E], dz[E], o[E];
+            if constexpr (VEC) {
+                unpack_vec<DT>(G[r], g);
+                unpack_vec<DT>(XN[r], xn);
+            } else {
+                g[0] = G[r];
+                xn[0] = XN[r];
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float z = bias[e];
+#pragma unroll
+                for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xw[(4 - W) + k][e], z);
+                dz[e] = z;
+            }
+            if (a.act) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = g[e] * silu_grad(dz[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = g[e];
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                // dxm[t] = sum_k w[k] * dz[t + (W-1) - k]
+                float acc = w[e][W - 1] * dz[e];
+                acc = fmaf(w[e][W - 2], dzf[0][e], acc);
+                if constexpr (W >= 3) acc = fmaf(w[e][W - 3], dzf[1][e], acc);
+                if constexpr (W == 4) acc = fmaf(w[e][0], dzf[2][e], acc);
+                o[e] = acc;
+#pragma unroll
+                for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xw[(4 - W) + k][e], dw[e][k]);
+                dbs[e] += dz[e];
+                dzf[2][e] = dzf[1][e];
+                dzf[1][e] = dzf[0][e];
+                dzf[0][e] = dz[e];
+            }
+            if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] += g[e];
+            }
+            if constexpr (MASK) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] *= mk[r];
+            }
+            if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] += g[e];
+            }
+            // slide the window one step back: the new oldest row is t - 4
+            const bool has_row = t - 4 >= 0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float v = xn[e];
+                if constexpr (MASK) v = mul_round<DT>(v, mn[r]);
+                xw[3][e] = xw[2][e];
+                xw[2][e] = xw[1][e];
+                xw[1][e] = xw[0][e];
+                xw[0][e] = has_row ? v : 0.0f;
+            }
+            if constexpr (VEC) {
+                store_vec<false>(db_ + t * ds, pack_vec<DT>(o));
+            } else {
+                store1<DT>(db_ + t * ds, 0, o[0]);
+            }
+        }
+    }
+
+    float *pp = a.partial + (((int64_t)b * a.nchunk + ch) * a.C + c0) * 5;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) pp[e * 5 + k] = k < W ? dw[e][k] : 0.0f;
+        pp[e * 5 + 4] = dbs[e];
+    }
+}
+
+// dweight[c, k] = sum over partial sets, in set order (fp64 accumulator, one rounding)
+__global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *partial, float *dweight, float *dbias,
+                                                              uint32_t C, uint32_t nsets, int W)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;   // (c, j), j in 0..4
+    if (i >= C * 5u) return;
+    const uint32_t c = i / 5u, j = i - c * 5u;
+    double acc = 0.0;
+    for (uint32_t s = 0; s < nsets; ++s) acc += (double)partial[(int64_t)s * C * 5 + i];
+    if (j < 4) {
+        if ((int)j < W) dweight[c * W + j] = (float)acc;
+    } else if (dbias) {
+        dbias[c] = (float)acc;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // decode update, vectorised: contiguous [B, C, S] state, channel-contiguous
 // x / out.  One lane owns E adjacent channels: it reads the E*S state
 // elements as S 16-byte vectors (they are one contiguous 16*S-byte run),
@@ -1510,6 +1776,125 @@ template <int DT> void launch_update(const UpdPlan &pl, hipStream_t s)
     }
 }
 
+// ---------------------------------------------------------------------------
+// backward: planning and launch
+// ---------------------------------------------------------------------------
+enum BwdKind { BWD_BLC_VEC, BWD_GENERIC };
+constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
+
+struct BwdPlan {
+    BwdKind kind;
+    BwdArgs args;
+    uint32_t grid;
+    int64_t workspace_bytes;
+};
+
+int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointers)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_bwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_bwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_bwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->batch < 0 || p->channels < 0 || p->seqlen < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld, seqlen %lld)",
+                    (long long)p->batch, (long long)p->channels, (long long)p->seqlen);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->seqlen >= (1ll << 31) ||
+        p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    if (p->mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
+    if (check_pointers) {
+        if (p->channels > 0 && (!p->weight || !p->dweight))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "weight and dweight must not be NULL");
+        if (!empty && (!p->x || !p->dout || !p->dx))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "x, dout and dx must not be NULL");
+        if (!empty && (p->dx == p->x || p->dx == p->dout))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "dx must not alias x or dout");
+    }
+
+    BwdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.dy = (const char *)p->dout; a.dx = (char *)p->dx;
+    a.weight = p->weight; a.bias = p->bias; a.mask = p->mask;
+    a.partial = (float *)p->workspace; a.dweight = p->dweight; a.dbias = p->dbias;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.x_sl = p->x_stride_l;
+    a.g_sb = p->dout_stride_b; a.g_sc = p->dout_stride_c; a.g_sl = p->dout_stride_l;
+    a.d_sb = p->dx_stride_b; a.d_sc = p->dx_stride_c; a.d_sl = p->dx_stride_l;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
+    a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
+    a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
+    plan->kind = BWD_GENERIC;
+    plan->grid = 0;
+    plan->workspace_bytes = 0;
+    if (empty) return CANON_OK;   // the caller's dweight/dbias are zero filled by canon_conv1d_bwd
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E == 0 && a.x_sl != 1 &&
+                     a.x_sb % E == 0 && a.x_sl % E == 0 && a.g_sb % E == 0 && a.g_sl % E == 0 &&
+                     a.d_sb % E == 0 && a.d_sl % E == 0 &&
+                     (!check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx)));
+    plan->kind = vec ? BWD_BLC_VEC : BWD_GENERIC;
+    a.nvec = vec ? a.C / E : a.C;
+    // time steps per lane: about 8 waves per CU, a multiple of the look-ahead, and few enough
+    // partial sets that the scratch stays below ~16 MB
+    const uint64_t lanes_per_step = (uint64_t)a.B * a.nvec;
+    uint64_t want_chunks = (256ull * 8 * 64 + lanes_per_step - 1) / lanes_per_step;
+    const uint64_t max_sets = (16ull << 20) / ((uint64_t)a.C * 20) + 1;
+    if ((uint64_t)a.B * want_chunks > max_sets) want_chunks = max_sets / a.B;
+    if (want_chunks < 1) want_chunks = 1;
+    uint32_t chunk = (uint32_t)((a.L + want_chunks - 1) / want_chunks);
+    chunk = ((chunk + kBwdRows - 1) / kBwdRows) * kBwdRows;
+    if (chunk < 4 * kBwdRows) chunk = 4 * kBwdRows;
+    a.chunk = chunk;
+    a.nchunk = (a.L + chunk - 1) / chunk;
+    const uint64_t nthreads = lanes_per_step * a.nchunk;
+    if (nthreads >= (1ull << 32)) return fail(CANON_ERR_UNSUPPORTED, "problem too large for the backward kernel");
+    a.nthreads = (uint32_t)nthreads;
+    a.nsets = a.B * a.nchunk;
+    a.div_nvec = make_fastdiv(a.nvec);
+    a.div_nchunk = make_fastdiv(a.nchunk);
+    plan->grid = (uint32_t)((nthreads + 255) / 256);
+    plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+    if (check_pointers) {
+        if (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes)
+            return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                        (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+    }
+    return CANON_OK;
+}
+
+template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStream_t s)
+{
+    const dim3 g(pl.grid), b(256);
+    if (pl.kind == BWD_BLC_VEC)
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, Elem<DT>::per_vec, true, MASK, kBwdRows>), g, b, 0, s, pl.args);
+    else
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, 1, false, MASK, kBwdRows>), g, b, 0, s, pl.args);
+}
+
+template <int DT> void launch_bwd(const BwdPlan &pl, hipStream_t s)
+{
+    const bool m = pl.args.mask != nullptr;
+    switch (pl.args.W) {
+    case 2: m ? launch_bwd_m<DT, 2, true>(pl, s) : launch_bwd_m<DT, 2, false>(pl, s); break;
+    case 3: m ? launch_bwd_m<DT, 3, true>(pl, s) : launch_bwd_m<DT, 3, false>(pl, s); break;
+    default: m ? launch_bwd_m<DT, 4, true>(pl, s) : launch_bwd_m<DT, 4, false>(pl, s); break;
+    }
+}
+
 int check_launch(const char *what)
 {
     const hipError_t e = hipGetLastError();
@@ -1553,6 +1938,46 @@ int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream)
     default: launch_update<CANON_DTYPE_F16>(pl, s); break;
     }
     return check_launch("canon_conv1d_update");
+}
+
+int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream)
+{
+    BwdPlan pl;
+    const int rc = plan_bwd(p, &pl, true);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (pl.grid == 0) {
+        // nothing to sum: the gradients of the parameters are zero
+        if (p->channels > 0) {
+            if (hipMemsetAsync(p->dweight, 0, (size_t)p->channels * p->width * sizeof(float), s) != hipSuccess)
+                return check_launch("canon_conv1d_bwd");
+            if (p->dbias && hipMemsetAsync(p->dbias, 0, (size_t)p->channels * sizeof(float), s) != hipSuccess)
+                return check_launch("canon_conv1d_bwd");
+        }
+        return CANON_OK;
+    }
+    switch (p->x_dtype) {
+    case CANON_DTYPE_F32: launch_bwd<CANON_DTYPE_F32>(pl, s); break;
+    case CANON_DTYPE_BF16: launch_bwd<CANON_DTYPE_BF16>(pl, s); break;
+    default: launch_bwd<CANON_DTYPE_F16>(pl, s); break;
+    }
+    hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 255u) / 256u), dim3(256), 0, s,
+                       pl.args.partial, pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.nsets, pl.args.W);
+    return check_launch("canon_conv1d_bwd");
+}
+
+int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p)
+{
+    BwdPlan pl;
+    if (plan_bwd(p, &pl, false) != CANON_OK) return -1;
+    return pl.workspace_bytes;
+}
+
+const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p)
+{
+    BwdPlan pl;
+    if (plan_bwd(p, &pl, false) != CANON_OK) return nullptr;
+    return pl.kind == BWD_BLC_VEC ? "bwd_blc_vec" : "bwd_generic";
 }
 
 const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)

@@ -130,6 +130,53 @@ def bench_decode(reps, warmup):
     return ms_eager * 1e3, ms_graph * 1e3, plan
 
 
+def bench_backward(steps, warmup, nbuf):
+    """Backward of the same prefill step (channel-contiguous, as a training step through the model
+    produces it): reads x and dout, writes dx, reduces dweight / dbias."""
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(2)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    dw = torch.empty(C, W, dtype=torch.float32, device=dev)
+    db = torch.empty(C, dtype=torch.float32, device=dev)
+    keep, params = [], []
+    for _ in range(nbuf):
+        x = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        dy = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        dx = torch.empty_like(x)
+        p = _lib.BwdParams()
+        p.struct_size = ctypes.sizeof(_lib.BwdParams)
+        p.x_dtype = p.w_dtype = 1
+        p.width, p.residual_mode = W, 1
+        p.batch, p.channels, p.seqlen = B, C, L
+        for name, t in (("x", x), ("dout", dy), ("dx", dx)):
+            setattr(p, name, t.data_ptr())
+            for sname, v in zip(("b", "c", "l"), t.stride()):
+                setattr(p, f"{name}_stride_{sname}", v)
+        p.weight, p.w_stride_c, p.w_stride_k, p.bias = w.data_ptr(), W, 1, bias.data_ptr()
+        p.dweight, p.dbias = dw.data_ptr(), db.data_ptr()
+        keep.append((x, dy, dx))
+        params.append(p)
+    L_ = _lib.lib()
+    ws = torch.empty(L_.canon_conv1d_bwd_workspace_bytes(ctypes.byref(params[0])), dtype=torch.uint8, device=dev)
+    for p in params:
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    plan = L_.canon_conv1d_bwd_plan(ctypes.byref(params[0])).decode()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    refs = [ctypes.byref(p) for p in params]
+
+    def step(i):
+        rc = L_.canon_conv1d_bwd(refs[i % nbuf], stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_bwd")
+
+    ms = time_region(step, steps, warmup)
+    return ms, plan, ws.numel()
+
+
 def cpu_baseline(budget_s=12.0):
     """The reference's eager formulation (mask-free Canon-D call: pad + grouped
     conv1d + residual, model/model.py:604-675) on the host cores, same shape."""
@@ -187,6 +234,7 @@ def main():
     ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
     dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
+    ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
     nbytes = prefill_bytes(B, C, L)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -205,6 +253,10 @@ def main():
                    "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
                    "us_per_step_hipgraph": round(dec_graph_us, 3),
                    "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1)},
+        "backward_channel_last": {"kernel": plan_bwd, "ms_per_step": round(ms_bwd, 6),
+                                  "GB/s": round(1.5 * nbytes / (ms_bwd * 1e-3) / 1e9, 1),
+                                  "bytes": "x and dout read, dx written (3 tensor passes)",
+                                  "scratch_bytes": ws_bwd},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
     }

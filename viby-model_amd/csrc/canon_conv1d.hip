@@ -1244,19 +1244,30 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     }
 }
 
-// dweight[c, k] = sum over partial sets, in set order (fp64 accumulator, one rounding)
+// dweight[c, k] / dbias[c] = sum over the partial sets, in a fixed order: a block owns 32 adjacent
+// (c, j) columns; its 8 slices each sum every 8th set in set order (fp64), then the slices are added
+// in slice order.  Reads are 128 contiguous bytes per set and slice.
 __global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *partial, float *dweight, float *dbias,
                                                               uint32_t C, uint32_t nsets, int W)
 {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;   // (c, j), j in 0..4
-    if (i >= C * 5u) return;
-    const uint32_t c = i / 5u, j = i - c * 5u;
+    __shared__ double part[8][32];
+    const uint32_t col = threadIdx.x & 31u, slice = threadIdx.x >> 5;
+    const uint32_t ncols = C * 5u;
+    const uint32_t i = blockIdx.x * 32u + col;   // (c, j), j in 0..4
     double acc = 0.0;
-    for (uint32_t s = 0; s < nsets; ++s) acc += (double)partial[(int64_t)s * C * 5 + i];
+    if (i < ncols)
+        for (uint32_t s = slice; s < nsets; s += 8u) acc += (double)partial[(int64_t)s * ncols + i];
+    part[slice][col] = acc;
+    __syncthreads();
+    if (slice != 0 || i >= ncols) return;
+    double total = part[0][col];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) total += part[k][col];
+    const uint32_t c = i / 5u, j = i - c * 5u;
     if (j < 4) {
-        if ((int)j < W) dweight[c * W + j] = (float)acc;
+        if ((int)j < W) dweight[c * W + j] = (float)total;
     } else if (dbias) {
-        dbias[c] = (float)acc;
+        dbias[c] = (float)total;
     }
 }
 
@@ -1961,7 +1972,7 @@ int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream)
     case CANON_DTYPE_BF16: launch_bwd<CANON_DTYPE_BF16>(pl, s); break;
     default: launch_bwd<CANON_DTYPE_F16>(pl, s); break;
     }
-    hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 255u) / 256u), dim3(256), 0, s,
+    hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 31u) / 32u), dim3(256), 0, s,
                        pl.args.partial, pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.nsets, pl.args.W);
     return check_launch("canon_conv1d_bwd");
 }

@@ -272,7 +272,8 @@ def test_bwd_plan_and_workspace():
     assert L.canon_conv1d_bwd_plan(ctypes.byref(p)) == b"bwd_blc_vec"
     ws = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(p))
     assert 0 < ws <= 20 << 20 and ws % (3456 * 5 * 4) == 0        # whole partial sets, bounded scratch
-    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl"))) == b"bwd_generic"
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl"))) == b"bwd_bcl_vec"
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl", L=1023))) == b"bwd_generic"
     assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(C=3457))) == b"bwd_generic"
     assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(width=9))) == -1
     assert "width 9" in last_error()

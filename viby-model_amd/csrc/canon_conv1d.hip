@@ -1024,7 +1024,7 @@ struct BwdArgs {
     int64_t w_sc, w_sk;
     int64_t m_sb, m_sl;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_vec;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_vec, b_pair, m_vec;
     uint32_t nvec;      // channel groups per row (C / E)
     uint32_t nchunk;    // time chunks per sequence
     uint32_t chunk;     // time steps per chunk
@@ -1241,6 +1241,226 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 #pragma unroll
         for (int k = 0; k < 4; ++k) pp[e * 5 + k] = k < W ? dw[e][k] : 0.0f;
         pp[e * 5 + 4] = dbs[e];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, time-contiguous rows ([B, C, L]): one wave owns one segment of one
+// (b, c) row, U vectors of E time steps per lane, exactly as the forward
+// kernel.  Pass 1 recomputes z and dz = dout * act'(z) for the lane's own
+// steps (history from lane l-1 by wave shift) and accumulates the lane's share
+// of dweight / dbias; pass 2 forms dx[t] = sum_k w[k] * dz[t+(W-1)-k] with the
+// three later dz values taken from lane l+1 (wave shift the other way), from
+// the next vector's lane 0, or -- for the last lane of a segment that is not
+// the end of the row -- recomputed from memory.  The wave's dweight / dbias
+// are reduced across lanes in a fixed butterfly order and written as one
+// partial set entry; canon_bwd_reduce_kernel sums the sets.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_shift_down(float v, float last)
+{
+    // lane i <- lane i+1 across the whole wave; lane 63 <- `last`
+    return bits_f((uint32_t)__builtin_amdgcn_update_dpp((int)f_bits(last), (int)f_bits(v),
+                                                        0x130 /* wave_shl:1 */, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float read_lane0(float v)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_readfirstlane((int)f_bits(v)));
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+    // fixed-order butterfly: every lane ends with the same total
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <int DT, int W, int U, bool MASK>
+__global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    constexpr int BY = Elem<DT>::bytes;
+    const int lane = threadIdx.x & 63;
+    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    if (task >= a.nthreads) return;          // nthreads = wave tasks in this kernel
+    uint32_t row = task, seg = 0;
+    if (a.nchunk > 1) {                      // nchunk = segments per row
+        row = fdiv(task, a.div_nchunk);
+        seg = task - row * a.nchunk;
+    }
+    const uint32_t b = fdiv(row, a.div_nvec);   // div_nvec divides by C here
+    const uint32_t c = row - b * a.C;
+
+    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * BY;
+    const char *grow = a.dy + ((int64_t)b * a.g_sb + (int64_t)c * a.g_sc) * BY;
+    char *drow = a.dx + ((int64_t)b * a.d_sb + (int64_t)c * a.d_sc) * BY;
+    const uint32_t nvec = a.L / E;
+    const uint32_t v0 = seg * (64u * U) + lane;
+
+    uint4 X[U], G[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        const uint32_t vc = v < nvec ? v : nvec - 1u;
+        X[u] = load_vec<false>(xrow + (int64_t)vc * 16);
+        G[u] = load_vec<false>(grow + (int64_t)vc * 16);
+    }
+    RawTaps<1> raw;
+    fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
+    float M[MASK ? U : 1][E];
+    if constexpr (MASK) {
+        int64_t mbase[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t v = v0 + u * 64u;
+            mbase[u] = b * a.m_sb + (int64_t)(v < nvec ? v : nvec - 1u) * E * a.m_sl;
+        }
+        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+    }
+    float w[1][W], bvv[1];
+    decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
+    const float bv = bvv[0];
+
+    // left history of the segment's first vector (lane 0 only), right dz of its last vector (lane 63 only)
+    float carry[3] = {0.0f, 0.0f, 0.0f};
+    float edge[3] = {0.0f, 0.0f, 0.0f};
+    const int64_t t_seg0 = (int64_t)seg * (64 * U) * E;
+    const int64_t t_seg1 = t_seg0 + (int64_t)(64 * U) * E;      // first step after the segment
+    if (lane == 0 && seg > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            float v = load1<DT>(xrow, t_seg0 - 3 + j);
+            if constexpr (MASK) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + (t_seg0 - 3 + j) * a.m_sl, a.mask_dtype));
+            carry[j] = v;
+        }
+    }
+    if (lane == 63 && t_seg1 < (int64_t)a.L) {
+        // dz[t_seg1 + j], j = 0..2, from x[t_seg1-3 .. t_seg1+2] and dout[t_seg1 .. t_seg1+2]
+        float xs6[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            const int64_t t = t_seg1 - 3 + i;
+            float v = 0.0f;
+            if (t < (int64_t)a.L) {
+                v = load1<DT>(xrow, t);
+                if constexpr (MASK) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            }
+            xs6[i] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int64_t t = t_seg1 + j;
+            if (t < (int64_t)a.L) {
+                float z = bv;
+#pragma unroll
+                for (int k = 0; k < W; ++k) z = fmaf(w[0][k], xs6[j + (4 - W) + k], z);
+                const float g = load1<DT>(grow, t);
+                edge[j] = a.act ? g * silu_grad(z) : g;
+            }
+        }
+    }
+
+    // pass 1: dz of the lane's own steps, and its share of dweight / dbias
+    float dz[U][E], gg[U][E];
+    float dwl[W], dbl = 0.0f;
+#pragma unroll
+    for (int k = 0; k < W; ++k) dwl[k] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool valid = v0 + u * 64u < nvec;
+        float xr[E], xm_store[MASK ? E : 1];
+        float *xm = MASK ? xm_store : xr;
+        unpack_vec<DT>(X[u], xr);
+        unpack_vec<DT>(G[u], gg[u]);
+        if constexpr (MASK) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
+        }
+        float seq[E + 3];
+        seq[0] = wave_shift_up(xm[E - 3], carry[0]);
+        seq[1] = wave_shift_up(xm[E - 2], carry[1]);
+        seq[2] = wave_shift_up(xm[E - 1], carry[2]);
+        if (u + 1 < U) {
+            carry[0] = read_lane63(xm[E - 3]);
+            carry[1] = read_lane63(xm[E - 2]);
+            carry[2] = read_lane63(xm[E - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) seq[3 + j] = xm[j];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float z = bv;
+#pragma unroll
+            for (int k = 0; k < W; ++k) z = fmaf(w[0][k], seq[j + (4 - W) + k], z);
+            dz[u][j] = z;
+        }
+        if (a.act) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = gg[u][j] * silu_grad(dz[u][j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = gg[u][j];
+        }
+        if (!valid) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) dwl[k] = fmaf(dz[u][j], seq[j + (4 - W) + k], dwl[k]);
+            dbl += dz[u][j];
+        }
+    }
+
+    // pass 2: dx
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        // the three dz values after this vector: lane l+1 of the same step, for lane 63 lane 0 of the next
+        float nx[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const float last = (u + 1 < U) ? read_lane0(dz[u + 1 < U ? u + 1 : u][j]) : edge[j];
+            nx[j] = wave_shift_down(dz[u][j], last);
+        }
+        float dq[E + 3];
+#pragma unroll
+        for (int j = 0; j < E; ++j) dq[j] = dz[u][j];
+        dq[E] = nx[0]; dq[E + 1] = nx[1]; dq[E + 2] = nx[2];
+        float o[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float acc = w[0][W - 1] * dq[j];
+#pragma unroll
+            for (int k = W - 2; k >= 0; --k) acc = fmaf(w[0][k], dq[j + (W - 1) - k], acc);
+            o[j] = acc;
+        }
+        if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += gg[u][j];
+        }
+        if constexpr (MASK) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] *= M[u][j];
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += gg[u][j];
+        }
+        if (v < nvec) store_vec<false>(drow + (int64_t)v * 16, pack_vec<DT>(o));
+    }
+
+    // the wave's dweight / dbias -> partial[(b * nseg + seg) * C + c][5]
+    float tot[5];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) tot[k] = k < W ? wave_sum(dwl[k < W ? k : 0]) : 0.0f;
+    tot[4] = wave_sum(dbl);
+    if (lane == 0) {
+        float *pp = a.partial + (((int64_t)b * a.nchunk + seg) * a.C + c) * 5;
+#pragma unroll
+        for (int k = 0; k < 5; ++k) pp[k] = tot[k];
     }
 }
 
@@ -1496,14 +1716,14 @@ FastDiv make_fastdiv(uint32_t d)
 
 // a run of E consecutive mask entries (E = elements of x per 16 bytes) starting
 // at a multiple of E is contiguous and aligned to its own size
-bool mask_run_aligned(const canon_conv1d_fwd_params *p)
+bool mask_run_aligned(const void *mask, int mask_dtype, int64_t stride_b, int64_t stride_l, int x_dtype)
 {
-    if (!p->mask || p->mask_stride_l != 1) return false;
+    if (!mask || stride_l != 1) return false;
     static const int msize[] = {1, 4, 8, 4, 2, 2};
-    const int E = 16 / elem_bytes(p->x_dtype);
-    const int64_t run = (int64_t)E * msize[p->mask_dtype];
+    const int E = 16 / elem_bytes(x_dtype);
+    const int64_t run = (int64_t)E * msize[mask_dtype];
     const int64_t align = run < 16 ? run : 16;
-    return ((uintptr_t)p->mask % align) == 0 && (p->mask_stride_b * msize[p->mask_dtype]) % align == 0;
+    return ((uintptr_t)mask % align) == 0 && (stride_b * msize[mask_dtype]) % align == 0;
 }
 
 enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
@@ -1575,7 +1795,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.S_out = p->final_state ? p->final_len : 0;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
     a.b_vec = p->bias && aligned16(p->bias);
-    a.m_vec = mask_run_aligned(p);
+    a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
     plan->grid = 0;
@@ -1790,11 +2010,12 @@ template <int DT> void launch_update(const UpdPlan &pl, hipStream_t s)
 // ---------------------------------------------------------------------------
 // backward: planning and launch
 // ---------------------------------------------------------------------------
-enum BwdKind { BWD_BLC_VEC, BWD_GENERIC };
+enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
 constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
 
 struct BwdPlan {
     BwdKind kind;
+    int U;
     BwdArgs args;
     uint32_t grid;
     int64_t workspace_bytes;
@@ -1848,15 +2069,46 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
     a.b_vec = p->bias && aligned16(p->bias);
     plan->kind = BWD_GENERIC;
+    plan->U = 1;
     plan->grid = 0;
     plan->workspace_bytes = 0;
     if (empty) return CANON_OK;   // the caller's dweight/dbias are zero filled by canon_conv1d_bwd
 
     const int E = 16 / elem_bytes(p->x_dtype);
+    a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
+    a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
+    const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
+    const bool rows = ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
+                      a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
+                      a.d_sb % E == 0 && a.d_sc % E == 0;
+    if (rows) {
+        const uint32_t nvec = a.L / E;
+        const uint64_t nrows = (uint64_t)a.B * a.C;
+        int U = 1;
+        for (int cand = 2; cand <= 4; cand *= 2) {
+            const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
+            if (nvec >= 64u * cand && nrows * nseg >= 2048) U = cand;
+        }
+        const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
+        const uint64_t ntasks = nrows * nseg;
+        if (ntasks < (1ull << 31)) {
+            plan->kind = BWD_BCL_VEC;
+            plan->U = U;
+            // field use in this kernel family: nthreads = wave tasks, nchunk = segments per row
+            a.nvec = nvec; a.nchunk = (uint32_t)nseg; a.nthreads = (uint32_t)ntasks;
+            a.nsets = a.B * a.nchunk;
+            a.div_nchunk = make_fastdiv(a.nchunk); a.div_nvec = make_fastdiv(a.C);
+            plan->grid = (uint32_t)((ntasks + 3) / 4);
+            plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+            if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
+                return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                            (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+            return CANON_OK;
+        }
+    }
     const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E == 0 && a.x_sl != 1 &&
                      a.x_sb % E == 0 && a.x_sl % E == 0 && a.g_sb % E == 0 && a.g_sl % E == 0 &&
-                     a.d_sb % E == 0 && a.d_sl % E == 0 &&
-                     (!check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx)));
+                     a.d_sb % E == 0 && a.d_sl % E == 0 && ptrs16;
     plan->kind = vec ? BWD_BLC_VEC : BWD_GENERIC;
     a.nvec = vec ? a.C / E : a.C;
     // time steps per lane: about 8 waves per CU, a multiple of the look-ahead, and few enough
@@ -1890,7 +2142,13 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
 template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
-    if (pl.kind == BWD_BLC_VEC)
+    if (pl.kind == BWD_BCL_VEC) {
+        switch (pl.U) {
+        case 4: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 4, MASK>), g, b, 0, s, pl.args); break;
+        case 2: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 2, MASK>), g, b, 0, s, pl.args); break;
+        default: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 1, MASK>), g, b, 0, s, pl.args); break;
+        }
+    } else if (pl.kind == BWD_BLC_VEC)
         hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, Elem<DT>::per_vec, true, MASK, kBwdRows>), g, b, 0, s, pl.args);
     else
         hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, 1, false, MASK, kBwdRows>), g, b, 0, s, pl.args);
@@ -1988,7 +2246,7 @@ const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p)
 {
     BwdPlan pl;
     if (plan_bwd(p, &pl, false) != CANON_OK) return nullptr;
-    return pl.kind == BWD_BLC_VEC ? "bwd_blc_vec" : "bwd_generic";
+    return pl.kind == BWD_BLC_VEC ? "bwd_blc_vec" : pl.kind == BWD_BCL_VEC ? "bwd_bcl_vec" : "bwd_generic";
 }
 
 const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)

@@ -96,3 +96,47 @@ def test_canon_layer_prefill_then_decode_at_model_shapes(site, C):
             assert cache.canon_cache_a[3] is state            # updated in place, same object
             assert torch.equal(bits(state), bits(ref_cache[0])), step
             assert_parity(got, want, exact=False, what=f"site {site} step {step}")
+
+
+def test_decode_token_as_one_hip_graph():
+    """All 72 Canon update launches of one generated token (18 layers x sites a, b, c, d) captured into
+    one HIP graph and replayed with eager work and synchronisations in between: every replay must give
+    the bits of the eager launches (states are carried in place from replay to replay)."""
+    import causal_conv1d as cc
+    torch.manual_seed(12)
+    B, S, layers = 16, 4, 18
+    sites = [("a", 640), ("b", 960), ("c", 640), ("d", 3456)]
+    dtype = torch.bfloat16
+    weights = {n: (torch.randn(C, 4) * 0.3).to(dtype).to(DEV) for n, C in sites}
+    toks = {n: torch.randn(B, C).to(dtype).to(DEV) for n, C in sites}          # static input buffers
+    states_g = {(n, l): torch.randn(B, C, S).to(dtype).to(DEV) for n, C in sites for l in range(layers)}
+    states_e = {k: v.clone() for k, v in states_g.items()}
+    outs_g = {}
+
+    def one_token(states, outs):
+        for l in range(layers):
+            for n, _ in sites:
+                outs[(n, l)] = cc.causal_conv1d_update(toks[n], states[(n, l)], weights[n], residual=True)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one_token({k: v.clone() for k, v in states_g.items()}, {})              # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_token(states_g, outs_g)
+    for k in states_g:                    # capture does not run the kernels; start both from the same state
+        assert torch.equal(bits(states_g[k]), bits(states_e[k]))
+    for replay in range(4):
+        for n, C in sites:
+            toks[n].copy_(torch.randn(B, C).to(dtype))                          # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        outs_e = {}
+        one_token(states_e, outs_e)
+        torch.cuda.synchronize()
+        for k in states_g:
+            assert torch.equal(bits(states_g[k]), bits(states_e[k])), (replay, k)
+            assert torch.equal(bits(outs_g[k]), bits(outs_e[k])), (replay, k)

@@ -200,6 +200,24 @@ typedef struct canon_conv1d_bwd_params {
     int64_t workspace_bytes;
 } canon_conv1d_bwd_params;
 
+/*
+ * One channel range of a logical [batch, channels, seqlen] input that lives in
+ * a tensor of its own.  Canon-B convolves cat(q, k, v) and Canon-D
+ * cat(gate, up) along the channels (model/model.py:772-789, 962-971): with
+ * parts, the projections are read where they are and the results written to
+ * separate tensors, so neither the cat nor a split copy is made.  Part i covers
+ * channels [sum of channels of parts < i, + channels) of weight, bias and the
+ * states.  For the decode update only the _b and _c strides are read.
+ */
+#define CANON_CONV1D_MAX_PARTS 4
+typedef struct canon_conv1d_part {
+    const void *x;
+    int64_t x_stride_b, x_stride_c, x_stride_l;
+    void *out;
+    int64_t out_stride_b, out_stride_c, out_stride_l;
+    int64_t channels;
+} canon_conv1d_part;
+
 int canon_conv1d_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none). */
@@ -209,6 +227,18 @@ const char *canon_conv1d_last_error(void);
 int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream);
 int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
 int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream);
+
+/*
+ * The same operators with x / out given as 1..CANON_CONV1D_MAX_PARTS channel
+ * ranges (p->x, p->out and their strides are ignored; p->channels must equal
+ * the sum over the parts; weight, bias, mask and the states are those of the
+ * whole problem).  Channel-contiguous parts of width 4 run as ONE launch;
+ * other layouts are launched part by part.  Results equal the single-tensor
+ * call on the concatenated input bit for bit.
+ */
+int canon_conv1d_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts, void *stream);
+int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts,
+                              void *stream);
 
 /* Scratch bytes canon_conv1d_bwd needs for these sizes and strides (the
  * pointers in *p are not read); negative if the arguments are rejected. */
@@ -223,6 +253,10 @@ int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
 const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p);
 const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p);
 const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p);   /* "bwd_blc_vec" | "bwd_bcl_vec" | "bwd_generic" */
+/* "blc_vec_parts" / "update_vec_parts" (one launch) or "per_part" (one launch per part) */
+const char *canon_conv1d_fwd_parts_plan(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts);
+const char *canon_conv1d_update_parts_plan(const canon_conv1d_update_params *p, const canon_conv1d_part *parts,
+                                           int32_t nparts);
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@ HEADER = os.path.join(ROOT, "include", "canon_conv1d.h")
 
 import causal_conv1d as cc                      # noqa: E402
 from causal_conv1d import _lib                  # noqa: E402
-from causal_conv1d._lib import BwdParams, FwdParams, UpdateParams  # noqa: E402
+from causal_conv1d._lib import BwdParams, FwdParams, Part, UpdateParams  # noqa: E402
 
 
 def test_library_exports_every_declared_function():
@@ -40,7 +40,7 @@ def test_library_exports_every_declared_function():
 def test_ctypes_structs_match_the_header(tmp_path):
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){']
     structs = (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams),
-               ("canon_conv1d_bwd_params", BwdParams))
+               ("canon_conv1d_bwd_params", BwdParams), ("canon_conv1d_part", Part))
     for cname, cls in structs:
         lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')
         for fname, _ in cls._fields_:
@@ -283,3 +283,62 @@ def test_bwd_plan_and_workspace():
     assert "workspace" in last_error()
     assert L.canon_conv1d_bwd(ctypes.byref(bwd_params(dx=FAKE_X)), None) == _lib.ERR_INVALID_ARGUMENT
     assert "alias" in last_error()
+
+
+def make_parts(dims, B=8, L=1024, layout="blc", elem=2, row=None):
+    """Fake part descriptors: separate (B, L, C_i) allocations, or with ``row`` slices of one (B, L, row) tensor."""
+    arr = (Part * len(dims))()
+    c0 = 0
+    for i, d in enumerate(dims):
+        if row is not None:
+            arr[i].x, arr[i].out = FAKE_X + c0 * elem, FAKE_OUT + c0 * elem
+            strides = (row * L, 1, row)
+        else:
+            arr[i].x, arr[i].out = FAKE_X + i * 0x1000000, FAKE_OUT + i * 0x1000000
+            strides = (d * L, 1, d) if layout == "blc" else (d * L, L, 1)
+        arr[i].x_stride_b, arr[i].x_stride_c, arr[i].x_stride_l = strides
+        arr[i].out_stride_b, arr[i].out_stride_c, arr[i].out_stride_l = strides
+        arr[i].channels = d
+        c0 += d
+    return arr
+
+
+def test_parts_plan_and_validation():
+    L = _lib.lib()
+
+    def fplan(p, arr, n=None):
+        r = L.canon_conv1d_fwd_parts_plan(ctypes.byref(p), arr, len(arr) if n is None else n)
+        return r.decode() if r is not None else None
+
+    def uplan_parts(p, arr):
+        r = L.canon_conv1d_update_parts_plan(ctypes.byref(p), arr, len(arr))
+        return r.decode() if r is not None else None
+
+    # Canon-B (q, k, v) and Canon-D (gate, up), separate tensors and slices of one projection output
+    assert fplan(fwd_params(C=960, layout="blc"), make_parts([640, 160, 160])) == "blc_vec_parts"
+    assert fplan(fwd_params(C=3456, layout="blc"), make_parts([1728, 1728])) == "blc_vec_parts"
+    assert fplan(fwd_params(C=960, layout="blc"), make_parts([640, 160, 160], row=960)) == "blc_vec_parts"
+    assert fplan(fwd_params(C=960, layout="blc", x=None, out=None), make_parts([640, 160, 160])) == "blc_vec_parts"
+    # one launch per part: time-contiguous parts, a single part, other widths, channel counts off the vector size
+    assert fplan(fwd_params(C=960), make_parts([640, 320], layout="bcl")) == "per_part"
+    assert fplan(fwd_params(C=640, layout="blc"), make_parts([640])) == "per_part"
+    assert fplan(fwd_params(C=960, layout="blc", width=3, w_stride_c=3), make_parts([640, 320])) == "per_part"
+    assert fplan(fwd_params(C=100, layout="blc"), make_parts([60, 40])) == "per_part"
+    # rejected
+    assert fplan(fwd_params(C=961, layout="blc"), make_parts([640, 160, 160])) is None
+    assert "960 channels" in last_error() and "961" in last_error()
+    assert fplan(fwd_params(C=960, layout="blc"), make_parts([640, 160, 160]), n=0) is None
+    assert "nparts" in last_error()
+    assert fplan(fwd_params(C=5 * 64, layout="blc"), make_parts([64] * 5)) is None
+    assert L.canon_conv1d_fwd_parts_plan(ctypes.byref(fwd_params()), None, 2) is None
+    assert "parts is NULL" in last_error()
+    bad = make_parts([640, 320])
+    bad[1].x = None
+    assert fplan(fwd_params(C=960, layout="blc"), bad) is None
+    assert "must not be NULL" in last_error()
+
+    assert uplan_parts(update_params(C=960, S=8), make_parts([640, 160, 160], L=1)) == "update_vec_parts"
+    assert uplan_parts(update_params(C=3456, S=3), make_parts([1728, 1728], L=1)) == "update_vec_parts"
+    assert uplan_parts(update_params(C=3456, S=5), make_parts([1728, 1728], L=1)) == "per_part"
+    assert uplan_parts(update_params(C=3456, S=3), make_parts([3456], L=1)) == "per_part"
+    assert uplan_parts(update_params(C=3457, S=3), make_parts([1728, 1728], L=1)) is None

@@ -34,10 +34,14 @@ __version__ = "0.1.0"
 __all__ = [
     "causal_conv1d_fn",
     "causal_conv1d_update",
+    "causal_conv1d_fn_parts",
+    "causal_conv1d_update_parts",
     "short_conv_fused",
     "short_conv_update",
     "kernel_plan_fwd",
     "kernel_plan_update",
+    "kernel_plan_fwd_parts",
+    "kernel_plan_update_parts",
 ]
 
 MIN_WIDTH, MAX_WIDTH = 2, 4   # CANON_CONV1D_MIN_WIDTH / _MAX_WIDTH
@@ -115,7 +119,7 @@ _NARROW_MIN_ELEMENTS = 1 << 20
 _narrow_cache = [None, None, None]   # key, the source mask (kept alive so its address stays unique), converted mask
 
 
-def _narrow_mask(mask: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tensor:
     """An integer mask wider than x's element type is converted to x.dtype once.
 
     Every (batch, channel) row re-reads its batch row of the mask, so an int64
@@ -127,7 +131,7 @@ def _narrow_mask(mask: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     Canon call of a forward.  Small problems keep the caller's mask as is.
     """
     if (mask.dtype.is_floating_point or mask.element_size() <= x.element_size()
-            or x.numel() < _NARROW_MIN_ELEMENTS):
+            or numel < _NARROW_MIN_ELEMENTS):
         return mask
     key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, x.dtype, mask.device)
     if _narrow_cache[0] != key:
@@ -167,6 +171,48 @@ def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res
         p.final_stride_b, p.final_stride_c, p.final_stride_s = final_states.stride()
         p.final_len = final_states.shape[2]
     return p
+
+
+def _check_fwd_args(x, shape, weight, bias, attention_mask, initial_states, return_final_states, final_states_out):
+    """Checks shared by the single-tensor and the multi-part prefill; ``x`` is (one of) the input tensor(s),
+    ``shape`` the logical (batch, dim, seqlen).  Returns (bias, attention_mask, final_states) as launched."""
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"Unsupported input dtype {x.dtype}; expected float32, bfloat16 or float16")
+    batch, dim, seqlen = shape
+    _check_shapes(dim, weight, bias)
+    _require_gpu(x, "Input tensor")
+    _check_devices(weight, bias, x.device)
+    bias = _prep_bias(weight, bias)
+
+    if attention_mask is not None:
+        if attention_mask.dim() != 2:
+            raise ValueError(f"Expected 2D attention mask, got {attention_mask.dim()}D")
+        if tuple(attention_mask.shape) != (batch, seqlen):
+            raise ValueError(
+                f"Attention mask shape {tuple(attention_mask.shape)} does not match input shape ({batch}, {seqlen})")
+        if attention_mask.dtype not in _lib.MASK_CODE:
+            raise ValueError(f"Unsupported attention mask dtype {attention_mask.dtype}")
+        if attention_mask.device != x.device:
+            raise ValueError("Attention mask must be on the same device as x")
+        attention_mask = _narrow_mask(attention_mask, x, batch * dim * seqlen)
+    width = weight.shape[1]
+    if initial_states is not None:
+        if initial_states.dim() != 3 or tuple(initial_states.shape[:2]) != (batch, dim):
+            raise ValueError(f"initial_states shape {tuple(initial_states.shape)} does not match (batch, dim, >=width-1)")
+        if initial_states.dtype != x.dtype or initial_states.device != x.device:
+            raise ValueError("initial_states must have the dtype and device of x")
+    final_states = None
+    if return_final_states or final_states_out is not None:
+        if final_states_out is not None:
+            if final_states_out.dim() != 3 or tuple(final_states_out.shape[:2]) != (batch, dim):
+                raise ValueError(
+                    f"final_states_out shape {tuple(final_states_out.shape)} does not match (batch, dim, state_len)")
+            if final_states_out.dtype != x.dtype or final_states_out.device != x.device:
+                raise ValueError("final_states_out must have the dtype and device of x")
+            final_states = final_states_out
+        else:
+            final_states = torch.empty(batch, dim, width - 1, dtype=x.dtype, device=x.device)
+    return bias, attention_mask, final_states
 
 
 def causal_conv1d_fn(
@@ -213,42 +259,8 @@ def causal_conv1d_fn(
         raise NotImplementedError("seq_idx (packed variable-length batches) is not supported")
     if x.dim() != 3:
         raise ValueError(f"Expected 3D input tensor (batch, dim, seqlen), got {x.dim()}D")
-    if x.dtype not in _lib.DTYPE_CODE:
-        raise ValueError(f"Unsupported input dtype {x.dtype}; expected float32, bfloat16 or float16")
-    batch, dim, seqlen = x.shape
-    _check_shapes(dim, weight, bias)
-    _require_gpu(x, "Input tensor")
-    _check_devices(weight, bias, x.device)
-    bias = _prep_bias(weight, bias)
-
-    if attention_mask is not None:
-        if attention_mask.dim() != 2:
-            raise ValueError(f"Expected 2D attention mask, got {attention_mask.dim()}D")
-        if tuple(attention_mask.shape) != (batch, seqlen):
-            raise ValueError(
-                f"Attention mask shape {tuple(attention_mask.shape)} does not match input shape ({batch}, {seqlen})")
-        if attention_mask.dtype not in _lib.MASK_CODE:
-            raise ValueError(f"Unsupported attention mask dtype {attention_mask.dtype}")
-        if attention_mask.device != x.device:
-            raise ValueError("Attention mask must be on the same device as x")
-        attention_mask = _narrow_mask(attention_mask, x)
-    width = weight.shape[1]
-    if initial_states is not None:
-        if initial_states.dim() != 3 or tuple(initial_states.shape[:2]) != (batch, dim):
-            raise ValueError(f"initial_states shape {tuple(initial_states.shape)} does not match (batch, dim, >=width-1)")
-        if initial_states.dtype != x.dtype or initial_states.device != x.device:
-            raise ValueError("initial_states must have the dtype and device of x")
-    final_states = None
-    if return_final_states or final_states_out is not None:
-        if final_states_out is not None:
-            if final_states_out.dim() != 3 or tuple(final_states_out.shape[:2]) != (batch, dim):
-                raise ValueError(
-                    f"final_states_out shape {tuple(final_states_out.shape)} does not match (batch, dim, state_len)")
-            if final_states_out.dtype != x.dtype or final_states_out.device != x.device:
-                raise ValueError("final_states_out must have the dtype and device of x")
-            final_states = final_states_out
-        else:
-            final_states = torch.empty(batch, dim, width - 1, dtype=x.dtype, device=x.device)
+    bias, attention_mask, final_states = _check_fwd_args(
+        x, tuple(x.shape), weight, bias, attention_mask, initial_states, return_final_states, final_states_out)
 
     if x.stride(2) != 1 and x.stride(1) != 1:
         x = x.contiguous()
@@ -447,6 +459,150 @@ def causal_conv1d_update(
 
 
 # ---------------------------------------------------------------------------
+# Channel ranges given as separate tensors (Canon-B: q, k, v; Canon-D: gate, up)
+# ---------------------------------------------------------------------------
+def _part_array(xs, outs):
+    arr = (_lib.Part * len(xs))()
+    for i, (x, o) in enumerate(zip(xs, outs)):
+        arr[i].x = x.data_ptr()
+        arr[i].out = o.data_ptr()
+        arr[i].channels = x.shape[1]
+        if x.dim() == 3:
+            arr[i].x_stride_b, arr[i].x_stride_c, arr[i].x_stride_l = x.stride()
+            arr[i].out_stride_b, arr[i].out_stride_c, arr[i].out_stride_l = o.stride()
+        else:
+            arr[i].x_stride_b, arr[i].x_stride_c = x.stride()
+            arr[i].out_stride_b, arr[i].out_stride_c = o.stride()
+    return arr
+
+
+def _check_parts(xs, ndim: int, what: str):
+    xs = list(xs)
+    if not 1 <= len(xs) <= _lib.MAX_PARTS:
+        raise ValueError(f"{what}: expected 1..{_lib.MAX_PARTS} parts, got {len(xs)}")
+    first = xs[0]
+    for x in xs:
+        if x.dim() != ndim:
+            raise ValueError(f"{what}: expected {ndim}D parts, got {x.dim()}D")
+        if x.dtype != first.dtype or x.device != first.device:
+            raise ValueError(f"{what}: all parts must have one dtype and device")
+        if x.shape[0] != first.shape[0] or tuple(x.shape[2:]) != tuple(first.shape[2:]):
+            raise ValueError(f"{what}: parts differ in batch or seqlen: {tuple(x.shape)} vs {tuple(first.shape)}")
+    return xs
+
+
+def causal_conv1d_fn_parts(
+    xs,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    *,
+    initial_states: Optional[torch.Tensor] = None,
+    return_final_states: bool = False,
+    final_states_out: Optional[torch.Tensor] = None,
+    activation: Optional[str] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+    residual: Union[bool, str] = False,
+    rounding: str = "fused",
+):
+    """``causal_conv1d_fn`` on ``torch.cat(xs, dim=1)`` without making the cat.
+
+    ``xs``: 1..4 tensors (batch, dim_i, seqlen); ``weight`` (sum dim_i, W), ``bias`` and the
+    states cover all channels in the order of the parts.  Returns the tuple of outputs, one per
+    part with that part's strides (and the final states when asked for).  This is what Canon-B /
+    Canon-D need (``model/model.py:772-789, 962-971`` concatenate q/k/v and gate/up only to call
+    the conv once); results equal the call on the concatenation bit for bit.  When a gradient is
+    required the parts are concatenated and the differentiable single-tensor call is used.
+    """
+    act = _activation_flag(activation)
+    res = _residual_mode(residual)
+    rnd = _round_mode(rounding)
+    xs = _check_parts(xs, 3, "causal_conv1d_fn_parts")
+    batch, seqlen = xs[0].shape[0], xs[0].shape[2]
+    dims = [x.shape[1] for x in xs]
+    dim = sum(dims)
+    bias, attention_mask, final_states = _check_fwd_args(
+        xs[0], (batch, dim, seqlen), weight, bias, attention_mask, initial_states, return_final_states,
+        final_states_out)
+    if batch * dim * seqlen == 0 and final_states is not None and final_states.numel():
+        raise ValueError("cannot produce final states from an empty input")
+
+    if _wants_grad(*xs, weight, bias):
+        result = causal_conv1d_fn(
+            torch.cat(xs, dim=1), weight, bias, initial_states=initial_states, final_states_out=final_states,
+            activation=activation, attention_mask=attention_mask, residual=residual, rounding=rounding)
+        y = result[0] if final_states is not None else result
+        outs = tuple(y.split(dims, dim=1))
+        return (outs, final_states) if final_states is not None else outs
+
+    xs = [x if (x.stride(2) == 1 or x.stride(1) == 1) else x.contiguous() for x in xs]
+    outs = tuple(torch.empty_like(x) for x in xs)
+    if batch * dim * seqlen:
+        p = _fill_fwd(xs[0], outs[0], weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+        p.channels = dim
+        p.x = p.out = None
+        arr = _part_array(xs, outs)
+        with torch.cuda.device(xs[0].device):
+            rc = _lib.lib().canon_conv1d_fwd_parts(ctypes.byref(p), arr, len(xs), _stream(xs[0].device))
+        _lib.check(rc, "causal_conv1d_fn_parts")
+    return (outs, final_states) if final_states is not None else outs
+
+
+def causal_conv1d_update_parts(
+    xs,
+    conv_state: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    activation: Optional[str] = None,
+    *,
+    token_mask: Optional[torch.Tensor] = None,
+    residual: Union[bool, str] = False,
+    rounding: str = "fused",
+):
+    """``causal_conv1d_update`` on ``torch.cat(xs, dim=1)`` without making the cat: ``xs`` are 1..4
+    tokens (batch, dim_i); ``conv_state`` (batch, sum dim_i, state_len) is the one state of the layer,
+    updated in place.  Returns the tuple of outputs."""
+    act = _activation_flag(activation)
+    res = _residual_mode(residual)
+    rnd = _round_mode(rounding)
+    xs = _check_parts(xs, 2, "causal_conv1d_update_parts")
+    x0 = xs[0]
+    if x0.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"Unsupported input dtype {x0.dtype}; expected float32, bfloat16 or float16")
+    batch = x0.shape[0]
+    dims = [x.shape[1] for x in xs]
+    dim = sum(dims)
+    if conv_state.dim() != 3:
+        raise ValueError(f"Expected 3D conv_state tensor (batch, dim, state_len), got {conv_state.dim()}D")
+    if tuple(conv_state.shape[:2]) != (batch, dim):
+        raise ValueError(
+            f"Input shape {(batch, dim)} doesn't match conv_state batch/dim {tuple(conv_state.shape[:2])}")
+    if conv_state.dtype != x0.dtype or conv_state.device != x0.device:
+        raise ValueError("conv_state must have the dtype and device of x")
+    _check_shapes(dim, weight, bias)
+    _require_gpu(x0, "Input tensor")
+    _check_devices(weight, bias, x0.device)
+    if conv_state.shape[2] < weight.shape[1] - 1:
+        raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
+    _no_grad_needed(*xs, weight, bias, conv_state)
+    bias = _prep_bias(weight, bias)
+    if token_mask is not None:
+        if token_mask.dim() != 1 or token_mask.shape[0] != batch:
+            raise ValueError(f"token_mask shape {tuple(token_mask.shape)} does not match (batch,) = ({batch},)")
+        if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x0.device:
+            raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
+    outs = tuple(torch.empty_like(x, memory_format=torch.contiguous_format) for x in xs)
+    if batch * dim:
+        p = _fill_update(xs[0], outs[0], conv_state, weight, bias, token_mask, act, res, rnd)
+        p.channels = dim
+        p.x = p.out = None
+        arr = _part_array(xs, outs)
+        with torch.cuda.device(x0.device):
+            rc = _lib.lib().canon_conv1d_update_parts(ctypes.byref(p), arr, len(xs), _stream(x0.device))
+        _lib.check(rc, "causal_conv1d_update_parts")
+    return outs
+
+
+# ---------------------------------------------------------------------------
 # The reference's fused (batch, seqlen, dim) API, same argument meaning.
 # ---------------------------------------------------------------------------
 def short_conv_fused(
@@ -519,4 +675,30 @@ def kernel_plan_update(x, conv_state, weight, bias=None, activation=None, residu
     name = _lib.lib().canon_conv1d_update_plan(ctypes.byref(p))
     if name is None:
         _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_update")
+    return name.decode()
+
+
+def kernel_plan_fwd_parts(xs, weight, bias=None, activation=None, attention_mask=None, residual=False) -> str:
+    """'blc_vec_parts' if ``causal_conv1d_fn_parts`` would run these parts as one launch, else 'per_part'."""
+    xs = list(xs)
+    outs = [torch.empty_like(x) for x in xs]
+    p = _fill_fwd(xs[0], outs[0], weight, _prep_bias(weight, bias), attention_mask, None, None,
+                  _activation_flag(activation), _residual_mode(residual), 0)
+    p.channels = sum(x.shape[1] for x in xs)
+    name = _lib.lib().canon_conv1d_fwd_parts_plan(ctypes.byref(p), _part_array(xs, outs), len(xs))
+    if name is None:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_fwd_parts")
+    return name.decode()
+
+
+def kernel_plan_update_parts(xs, conv_state, weight, bias=None, activation=None, residual=False) -> str:
+    """'update_vec_parts' if ``causal_conv1d_update_parts`` would run as one launch, else 'per_part'."""
+    xs = list(xs)
+    outs = [torch.empty_like(x) for x in xs]
+    p = _fill_update(xs[0], outs[0], conv_state, weight, _prep_bias(weight, bias), None,
+                     _activation_flag(activation), _residual_mode(residual), 0)
+    p.channels = sum(x.shape[1] for x in xs)
+    name = _lib.lib().canon_conv1d_update_parts_plan(ctypes.byref(p), _part_array(xs, outs), len(xs))
+    if name is None:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_update_parts")
     return name.decode()

@@ -78,6 +78,16 @@ class BwdParams(ctypes.Structure):
     ]
 
 
+class Part(ctypes.Structure):
+    _fields_ = [
+        ("x", _vp), ("x_stride_b", _i64), ("x_stride_c", _i64), ("x_stride_l", _i64),
+        ("out", _vp), ("out_stride_b", _i64), ("out_stride_c", _i64), ("out_stride_l", _i64),
+        ("channels", _i64),
+    ]
+
+
+MAX_PARTS = 4
+
 EXPORTS = (
     "canon_conv1d_abi_version",
     "canon_conv1d_last_error",
@@ -88,6 +98,10 @@ EXPORTS = (
     "canon_conv1d_bwd",
     "canon_conv1d_bwd_workspace_bytes",
     "canon_conv1d_bwd_plan",
+    "canon_conv1d_fwd_parts",
+    "canon_conv1d_update_parts",
+    "canon_conv1d_fwd_parts_plan",
+    "canon_conv1d_update_parts_plan",
 )
 
 _lib = None
@@ -120,6 +134,14 @@ def lib() -> ctypes.CDLL:
         L.canon_conv1d_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdParams)]
         L.canon_conv1d_bwd_plan.restype = ctypes.c_char_p
         L.canon_conv1d_bwd_plan.argtypes = [ctypes.POINTER(BwdParams)]
+        L.canon_conv1d_fwd_parts.restype = ctypes.c_int
+        L.canon_conv1d_fwd_parts.argtypes = [ctypes.POINTER(FwdParams), ctypes.POINTER(Part), _i32, _vp]
+        L.canon_conv1d_update_parts.restype = ctypes.c_int
+        L.canon_conv1d_update_parts.argtypes = [ctypes.POINTER(UpdateParams), ctypes.POINTER(Part), _i32, _vp]
+        L.canon_conv1d_fwd_parts_plan.restype = ctypes.c_char_p
+        L.canon_conv1d_fwd_parts_plan.argtypes = [ctypes.POINTER(FwdParams), ctypes.POINTER(Part), _i32]
+        L.canon_conv1d_update_parts_plan.restype = ctypes.c_char_p
+        L.canon_conv1d_update_parts_plan.argtypes = [ctypes.POINTER(UpdateParams), ctypes.POINTER(Part), _i32]
         got = L.canon_conv1d_abi_version()
         if got != ABI_VERSION:
             raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}")

@@ -26,6 +26,11 @@ package is installed and the one the parity vectors come from:
 ``rounding='eager'`` reproduces that branch's intermediate bf16/fp16 roundings
 bit for bit; the default ``'fused'`` rounds once.
 
+``forward_parts`` takes the channel ranges as separate tensors (q, k, v for
+Canon-B, gate and up for Canon-D) and returns one output per part, so the
+``torch.cat`` / ``split`` around the layer (``model/model.py:772-789, 962-971``)
+is not needed; the state on the cache is the same single tensor either way.
+
 Training: a block call without a cache is differentiable (fused backward
 kernel); the cached paths (prefill with state capture continues to work, the
 single-token step does not) are inference paths: run them under
@@ -39,7 +44,7 @@ from typing import Optional
 import torch
 from torch import nn
 
-from . import causal_conv1d_fn, causal_conv1d_update
+from . import causal_conv1d_fn, causal_conv1d_fn_parts, causal_conv1d_update, causal_conv1d_update_parts
 
 STATE_LEN_MIN = 8  # model/model.py:286, :626
 
@@ -76,6 +81,16 @@ class CanonLayer(nn.Module):
     def _state_len(self) -> int:
         return max(STATE_LEN_MIN, self.kernel_size)
 
+    @staticmethod
+    def _block_mask(attention_mask, B: int, T: int):
+        # the mask columns of the T tokens of this call (model/model.py:589-600)
+        if attention_mask is not None and attention_mask.dim() == 2:
+            if tuple(attention_mask.shape) == (B, T):
+                return attention_mask
+            if attention_mask.size(0) == B and attention_mask.size(1) >= T:
+                return attention_mask[:, -T:]
+        return None
+
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 cache=None, layer_idx: Optional[int] = None) -> torch.Tensor:
         B, T, D = x.shape
@@ -95,12 +110,7 @@ class CanonLayer(nn.Module):
             self._slot(cache)[layer_idx] = state
             return y.unsqueeze(1)
 
-        mask = None
-        if attention_mask is not None and attention_mask.dim() == 2:
-            if tuple(attention_mask.shape) == (B, T):
-                mask = attention_mask
-            elif attention_mask.size(0) == B and attention_mask.size(1) >= T:
-                mask = attention_mask[:, -T:]
+        mask = self._block_mask(attention_mask, B, T)
 
         new_state = None
         if use_cache:
@@ -118,3 +128,46 @@ class CanonLayer(nn.Module):
                 state = new_state
             self._slot(cache)[layer_idx] = state
         return out.transpose(1, 2)
+
+    def forward_parts(self, xs, attention_mask: Optional[torch.Tensor] = None,
+                      cache=None, layer_idx: Optional[int] = None):
+        """``forward(torch.cat(xs, dim=-1)).split(...)`` without the cat: ``xs`` are (B, T, D_i) tensors
+        whose widths add up to ``hidden_size``; returns a tuple of (B, T, D_i) outputs."""
+        xs = tuple(xs)
+        B, T = xs[0].shape[:2]
+        D = sum(x.shape[2] for x in xs)
+        if D != self.hidden_size:
+            raise ValueError(f"the parts hold {D} channels, the layer has {self.hidden_size}")
+        use_cache = cache is not None and layer_idx is not None
+        state = self._slot(cache)[layer_idx] if use_cache else None
+        taps = self.weight.squeeze(1)
+        act = "silu" if self.activation else None
+
+        if use_cache and T == 1:
+            token_mask = None
+            if attention_mask is not None and attention_mask.dim() == 2 and attention_mask.shape[0] == B:
+                token_mask = attention_mask[:, -1]
+            if state is None:
+                state = torch.zeros(B, D, self._state_len(), dtype=xs[0].dtype, device=xs[0].device)
+            ys = causal_conv1d_update_parts([x[:, 0] for x in xs], state, taps, self.bias_param, activation=act,
+                                            token_mask=token_mask, residual="unmasked", rounding=self.rounding)
+            self._slot(cache)[layer_idx] = state
+            return tuple(y.unsqueeze(1) for y in ys)
+
+        mask = self._block_mask(attention_mask, B, T)
+        new_state = None
+        if use_cache:
+            new_state = torch.empty(B, D, state.size(-1) if state is not None else self._state_len(),
+                                    dtype=xs[0].dtype, device=xs[0].device)
+        history = state if (state is not None and self.kernel_size > 1) else None
+        outs = causal_conv1d_fn_parts([x.transpose(1, 2) for x in xs], taps, self.bias_param, activation=act,
+                                      initial_states=history, final_states_out=new_state,
+                                      attention_mask=mask, residual="masked", rounding=self.rounding)
+        if use_cache:
+            outs, new_state = outs
+            if state is not None:
+                state.copy_(new_state)
+            else:
+                state = new_state
+            self._slot(cache)[layer_idx] = state
+        return tuple(o.transpose(1, 2) for o in outs)

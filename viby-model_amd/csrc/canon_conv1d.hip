@@ -790,13 +790,13 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
 constexpr int kBlcWaves = 4;   // waves (time slabs) per block
 
 template <int DT, int W, int R, bool MASK, bool NT>
-__global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
+__device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 {
     constexpr int E = Elem<DT>::per_vec;
     static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
     __shared__ uint4 tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
 
-    const uint32_t blk = blockIdx.x;   // plain memory order (an XCD-contiguous remap measured 3 % slower here)
+    // blocks in plain memory order (an XCD-contiguous remap measured 3 % slower here)
     // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
     const uint32_t bt = fdiv(blk, a.div_nct);
     const uint32_t ct = blk - bt * a.nct;
@@ -922,6 +922,38 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
                 store1<DT>(a.fin, b * a.f_sb + (int64_t)(c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
         }
     }
+}
+
+template <int DT, int W, int R, bool MASK, bool NT>
+__global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
+{
+    blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
+}
+
+// Several channel ranges of one logical [B, C, L] problem that live in separate
+// tensors (q / k / v or gate / up projections), one launch: every block belongs
+// to one part and runs the single-tensor code on that part's argument block.
+constexpr int kMaxParts = CANON_CONV1D_MAX_PARTS;
+
+template <typename Args> struct PartTable {
+    Args part[kMaxParts];
+    uint32_t first_block[kMaxParts];   // first block of each part; 0xFFFFFFFF for unused slots
+};
+
+template <typename Args>
+__device__ __forceinline__ uint32_t part_of_block(const PartTable<Args> &m, uint32_t blk)
+{
+    uint32_t p = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxParts; ++i) p += blk >= m.first_block[i] ? 1u : 0u;
+    return p;
+}
+
+template <int DT, int W, int R, bool MASK, bool NT>
+__global__ __launch_bounds__(256) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
+{
+    const uint32_t p = part_of_block(m, blockIdx.x);
+    blc_block<DT, W, R, MASK, NT>(m.part[p], blockIdx.x - m.first_block[p]);
 }
 
 // ---------------------------------------------------------------------------
@@ -1467,6 +1499,12 @@ __global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
 // dweight[c, k] / dbias[c] = sum over the partial sets, in a fixed order: a block owns 32 adjacent
 // (c, j) columns; its 8 slices each sum every 8th set in set order (fp64), then the slices are added
 // in slice order.  Reads are 128 contiguous bytes per set and slice.
+__global__ __launch_bounds__(256) void canon_zero_kernel(float *p, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
 __global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *partial, float *dweight, float *dbias,
                                                               uint32_t C, uint32_t nsets, int W)
 {
@@ -1530,11 +1568,11 @@ template <int DT> struct StateRun {
 };
 
 template <int DT, int W, int S, int NB>
-__global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
+__device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_t blk)
 {
     constexpr int E = Elem<DT>::per_vec;
     constexpr int BY = Elem<DT>::bytes;
-    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t tid = blk * 256u + threadIdx.x;
     if (tid >= a.nthreads) return;
     const uint32_t bg = fdiv(tid, a.div_nvec);
     const uint32_t cv = tid - bg * a.nvec;
@@ -1633,6 +1671,20 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
             dp[k] = q;
         }
     }
+}
+
+template <int DT, int W, int S, int NB>
+__global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
+{
+    update_vec_block<DT, W, S, NB>(a, blockIdx.x);
+}
+
+// the token of one step given as several channel ranges (separate projections), one launch
+template <int DT, int W, int S, int NB>
+__global__ __launch_bounds__(256) void canon_update_vec_parts_kernel(const PartTable<UpdArgs> m)
+{
+    const uint32_t p = part_of_block(m, blockIdx.x);
+    update_vec_block<DT, W, S, NB>(m.part[p], blockIdx.x - m.first_block[p]);
 }
 
 // decode update, any strides / state length / rounding mode: one thread per (b, c)
@@ -2008,6 +2060,212 @@ template <int DT> void launch_update(const UpdPlan &pl, hipStream_t s)
 }
 
 // ---------------------------------------------------------------------------
+// channel ranges in separate tensors: one derived problem per part
+// ---------------------------------------------------------------------------
+const void *advance(const void *p, int64_t elems, int bytes)
+{
+    return p ? (const void *)((const char *)p + elems * bytes) : nullptr;
+}
+
+int check_parts(const canon_conv1d_part *parts, int32_t nparts, int64_t channels)
+{
+    if (!parts) return fail(CANON_ERR_INVALID_ARGUMENT, "parts is NULL");
+    if (nparts < 1 || nparts > kMaxParts)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "nparts %d outside 1..%d", nparts, kMaxParts);
+    int64_t sum = 0;
+    for (int i = 0; i < nparts; ++i) {
+        if (parts[i].channels < 0 || parts[i].channels >= (1ll << 31))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "part %d has %lld channels", i, (long long)parts[i].channels);
+        sum += parts[i].channels;
+    }
+    if (sum != channels)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "the parts hold %lld channels, params.channels is %lld", (long long)sum,
+                    (long long)channels);
+    return CANON_OK;
+}
+
+struct FwdPartsPlan {
+    int n;
+    bool single;            // one launch over a PartTable
+    uint32_t grid;          // of that launch
+    FwdPlan part[kMaxParts];
+};
+
+int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts, FwdPartsPlan *pp)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_fwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_fwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_fwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    int rc = check_parts(parts, nparts, p->channels);
+    if (rc != CANON_OK) return rc;
+    if (p->batch > 0 && p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    const int xb = elem_bytes(p->x_dtype), wb = elem_bytes(p->w_dtype);
+    pp->n = nparts;
+    int64_t c0 = 0;
+    uint64_t blocks = 0;
+    bool all_blc = true;
+    for (int i = 0; i < nparts; ++i) {
+        canon_conv1d_fwd_params q = *p;
+        q.channels = parts[i].channels;
+        q.x = parts[i].x; q.x_stride_b = parts[i].x_stride_b; q.x_stride_c = parts[i].x_stride_c; q.x_stride_l = parts[i].x_stride_l;
+        q.out = parts[i].out; q.out_stride_b = parts[i].out_stride_b; q.out_stride_c = parts[i].out_stride_c;
+        q.out_stride_l = parts[i].out_stride_l;
+        q.weight = advance(p->weight, c0 * p->w_stride_c, wb);
+        q.bias = advance(p->bias, c0, wb);
+        q.initial_state = advance(p->initial_state, c0 * p->init_stride_c, xb);
+        q.final_state = (void *)advance(p->final_state, c0 * p->final_stride_c, xb);
+        rc = plan_fwd(&q, &pp->part[i]);
+        if (rc != CANON_OK) return rc;
+        if (pp->part[i].grid > 0) {
+            all_blc = all_blc && pp->part[i].kind == FWD_BLC;
+            blocks += pp->part[i].grid;
+        }
+        c0 += parts[i].channels;
+    }
+    // whether to stream past the caches is decided on the whole problem
+    const bool nt = 2ull * (uint64_t)p->batch * (uint64_t)p->channels * (uint64_t)p->seqlen * xb >= kStreamBytes;
+    for (int i = 0; i < nparts; ++i) pp->part[i].args.nt = nt;
+    pp->single = nparts > 1 && all_blc && p->width == 4 && blocks > 0 && blocks < (1ull << 31);
+    pp->grid = (uint32_t)blocks;
+    return CANON_OK;
+}
+
+template <int DT, bool MASK, bool NT>
+void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
+{
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(256), 0, s, m);
+}
+
+template <int DT> void launch_fwd_parts(const FwdPartsPlan &pp, hipStream_t s)
+{
+    if (!pp.single) {
+        for (int i = 0; i < pp.n; ++i)
+            if (pp.part[i].grid > 0) launch_fwd<DT>(pp.part[i], s);
+        return;
+    }
+    PartTable<FwdArgs> m;
+    memset(&m, 0, sizeof(m));
+    uint32_t first = 0;
+    bool mask = false, nt = false;
+    for (int i = 0; i < kMaxParts; ++i) {
+        m.first_block[i] = i < pp.n ? first : 0xFFFFFFFFu;
+        if (i < pp.n) {
+            m.part[i] = pp.part[i].args;
+            first += pp.part[i].grid;
+            mask = pp.part[i].args.mask != nullptr;
+            nt = pp.part[i].args.nt != 0;
+        }
+    }
+    if (mask) {
+        if (nt) launch_blc_parts<DT, true, true>(m, pp.grid, s);
+        else launch_blc_parts<DT, true, false>(m, pp.grid, s);
+    } else {
+        if (nt) launch_blc_parts<DT, false, true>(m, pp.grid, s);
+        else launch_blc_parts<DT, false, false>(m, pp.grid, s);
+    }
+}
+
+struct UpdPartsPlan {
+    int n;
+    bool single;
+    uint32_t grid;
+    UpdPlan part[kMaxParts];
+};
+
+int plan_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts, UpdPartsPlan *pp)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_update_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_update_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_update_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    int rc = check_parts(parts, nparts, p->channels);
+    if (rc != CANON_OK) return rc;
+    if (p->batch > 0 && p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels must be below 2^31");
+    const int xb = elem_bytes(p->x_dtype), wb = elem_bytes(p->w_dtype);
+    pp->n = nparts;
+    int64_t c0 = 0;
+    bool all_vec = true;
+    uint64_t nvec_total = 0;
+    for (int i = 0; i < nparts; ++i) {
+        canon_conv1d_update_params q = *p;
+        q.channels = parts[i].channels;
+        q.x = parts[i].x; q.x_stride_b = parts[i].x_stride_b; q.x_stride_c = parts[i].x_stride_c;
+        q.out = parts[i].out; q.out_stride_b = parts[i].out_stride_b; q.out_stride_c = parts[i].out_stride_c;
+        q.conv_state = (void *)advance(p->conv_state, c0 * p->state_stride_c, xb);
+        q.weight = advance(p->weight, c0 * p->w_stride_c, wb);
+        q.bias = advance(p->bias, c0, wb);
+        rc = plan_update(&q, &pp->part[i]);
+        if (rc != CANON_OK) return rc;
+        if (pp->part[i].grid > 0) {
+            all_vec = all_vec && pp->part[i].kind == UPD_VEC;
+            nvec_total += pp->part[i].args.nvec;
+        }
+        c0 += parts[i].channels;
+    }
+    pp->single = nparts > 1 && all_vec && p->width == 4 && nvec_total > 0;
+    pp->grid = 0;
+    if (pp->single) {
+        // batch rows per lane chosen on the whole token, the same for every part
+        const uint32_t nb = (nvec_total * (uint64_t)p->batch / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        uint64_t blocks = 0;
+        for (int i = 0; i < nparts; ++i) {
+            UpdPlan &u = pp->part[i];
+            if (u.grid == 0) continue;
+            u.args.nb = nb;
+            u.args.bgroups = (u.args.B + nb - 1) / nb;
+            u.args.nthreads = u.args.nvec * u.args.bgroups;
+            u.grid = (u.args.nthreads + 255) / 256;
+            blocks += u.grid;
+        }
+        pp->grid = (uint32_t)blocks;
+    }
+    return CANON_OK;
+}
+
+template <int DT, int NB> void launch_update_parts_nb(const PartTable<UpdArgs> &m, int S, uint32_t grid, hipStream_t s)
+{
+    const dim3 g(grid), b(256);
+    switch (S) {
+    case 3: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 3, NB>), g, b, 0, s, m); break;
+    case 4: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 4, NB>), g, b, 0, s, m); break;
+    default: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 8, NB>), g, b, 0, s, m); break;
+    }
+}
+
+template <int DT> void launch_update_parts(const UpdPartsPlan &pp, hipStream_t s)
+{
+    if (!pp.single) {
+        for (int i = 0; i < pp.n; ++i)
+            if (pp.part[i].grid > 0) launch_update<DT>(pp.part[i], s);
+        return;
+    }
+    PartTable<UpdArgs> m;
+    memset(&m, 0, sizeof(m));
+    uint32_t first = 0, nb = 1;
+    int S = 0;
+    for (int i = 0; i < kMaxParts; ++i) {
+        m.first_block[i] = i < pp.n ? first : 0xFFFFFFFFu;
+        if (i < pp.n) {
+            m.part[i] = pp.part[i].args;
+            first += pp.part[i].grid;
+            if (pp.part[i].grid > 0) {
+                nb = pp.part[i].args.nb;
+                S = pp.part[i].args.S;
+            }
+        }
+    }
+    if (nb == kUpdNB) launch_update_parts_nb<DT, kUpdNB>(m, S, pp.grid, s);
+    else launch_update_parts_nb<DT, 1>(m, S, pp.grid, s);
+}
+
+// ---------------------------------------------------------------------------
 // backward: planning and launch
 // ---------------------------------------------------------------------------
 enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
@@ -2217,11 +2475,12 @@ int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream)
     hipStream_t s = (hipStream_t)stream;
     if (pl.grid == 0) {
         // nothing to sum: the gradients of the parameters are zero
+        // (a fill kernel rather than a memset, so that the call can be captured into a HIP graph)
         if (p->channels > 0) {
-            if (hipMemsetAsync(p->dweight, 0, (size_t)p->channels * p->width * sizeof(float), s) != hipSuccess)
-                return check_launch("canon_conv1d_bwd");
-            if (p->dbias && hipMemsetAsync(p->dbias, 0, (size_t)p->channels * sizeof(float), s) != hipSuccess)
-                return check_launch("canon_conv1d_bwd");
+            const uint32_t nw = (uint32_t)(p->channels * p->width), nc = (uint32_t)p->channels;
+            hipLaunchKernelGGL(canon_zero_kernel, dim3((nw + 255) / 256), dim3(256), 0, s, p->dweight, nw);
+            if (p->dbias) hipLaunchKernelGGL(canon_zero_kernel, dim3((nc + 255) / 256), dim3(256), 0, s, p->dbias, nc);
+            return check_launch("canon_conv1d_bwd");
         }
         return CANON_OK;
     }
@@ -2261,6 +2520,50 @@ const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p)
     UpdPlan pl;
     if (plan_update(p, &pl) != CANON_OK) return nullptr;
     return pl.kind == UPD_VEC ? "update_vec" : "update_generic";
+}
+
+int canon_conv1d_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts, void *stream)
+{
+    FwdPartsPlan pp;
+    const int rc = plan_fwd_parts(p, parts, nparts, &pp);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (p->x_dtype) {
+    case CANON_DTYPE_F32: launch_fwd_parts<CANON_DTYPE_F32>(pp, s); break;
+    case CANON_DTYPE_BF16: launch_fwd_parts<CANON_DTYPE_BF16>(pp, s); break;
+    default: launch_fwd_parts<CANON_DTYPE_F16>(pp, s); break;
+    }
+    return check_launch("canon_conv1d_fwd_parts");
+}
+
+int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts,
+                              void *stream)
+{
+    UpdPartsPlan pp;
+    const int rc = plan_update_parts(p, parts, nparts, &pp);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (p->x_dtype) {
+    case CANON_DTYPE_F32: launch_update_parts<CANON_DTYPE_F32>(pp, s); break;
+    case CANON_DTYPE_BF16: launch_update_parts<CANON_DTYPE_BF16>(pp, s); break;
+    default: launch_update_parts<CANON_DTYPE_F16>(pp, s); break;
+    }
+    return check_launch("canon_conv1d_update_parts");
+}
+
+const char *canon_conv1d_fwd_parts_plan(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts)
+{
+    FwdPartsPlan pp;
+    if (plan_fwd_parts(p, parts, nparts, &pp) != CANON_OK) return nullptr;
+    return pp.single ? "blc_vec_parts" : "per_part";
+}
+
+const char *canon_conv1d_update_parts_plan(const canon_conv1d_update_params *p, const canon_conv1d_part *parts,
+                                           int32_t nparts)
+{
+    UpdPartsPlan pp;
+    if (plan_update_parts(p, parts, nparts, &pp) != CANON_OK) return nullptr;
+    return pp.single ? "update_vec_parts" : "per_part";
 }
 
 }  // extern "C"

@@ -85,6 +85,26 @@ def test_backward_matches_autograd_of_the_eager_formulation(cc, dtype, layout):
                 check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_backward_blocks_that_walk_several_tiles(cc, dtype):
+    """Channel-contiguous tensors large enough that a block walks more than one 32-step tile of its chunk
+    (dz handed from tile to tile), with a ragged end (200 = 6 tiles + 8 steps), SiLU, mask and bias."""
+    g = torch.Generator().manual_seed(29)
+    B, C, L = 16, 2048, 200
+    x = torch.randn(B, C, L, generator=g).to(dtype)
+    w = (torch.randn(C, 4, generator=g) * 0.5).to(dtype)
+    b = (torch.randn(C, generator=g) * 0.2).to(dtype)
+    dout = torch.randn(B, C, L, generator=g).to(dtype)
+    mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+    for act, residual, m in [("silu", "masked", mask), (None, "unmasked", mask), ("silu", False, None)]:
+        dx, dw, db, _ = gpu_grads(cc, x, w, b, dout, "blc", m, act, residual)
+        rdx, rdw, rdb, _ = conv1d_grads(x, w, b, dout, m, act, residual)
+        what = f"{dtype} multi-tile {act} {residual} mask{m is not None}"
+        check(dx, rdx, dtype, what + " dx")
+        check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
+        check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
 def test_backward_finite_differences_like_the_reference_tests(cc):
     """causal-conv1d-mps/test.py:259-272 and :275-291: eps 1e-3, atol 1e-3, rtol 1e-2, loss = out.sum()."""
     torch.manual_seed(0)

@@ -77,6 +77,43 @@ def test_small_model_hip_equals_oracle_bit_for_bit():
             assert torch.equal(bits(got), bits(want)), (site, layer)
 
 
+def test_model_with_concat_free_canon_b_d_is_bit_identical(capsys):
+    """Canon-B / Canon-D fed q, k, v and gate, up as separate tensors: same logits and states as the cat path,
+    at the small size and at the full model's shapes (with the time both take)."""
+    cfg = viby_config(hidden_size=64, num_hidden_layers=3, num_attention_heads=2, num_key_value_heads=1,
+                      head_dim=32, intermediate_size=96, vocab_size=512)
+    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(1)).to(DEV)
+    for rounding in ("fused", "eager"):
+        cat = init_weights(VibyShaped(cfg, hip_factory(cfg, rounding)), 7, torch.bfloat16, DEV)
+        par = init_weights(VibyShaped(cfg, hip_factory(cfg, rounding), parts=True), 7, torch.bfloat16, DEV)
+        toks_c, logits_c, cache_c = cat.generate(ids, 6)
+        toks_p, logits_p, cache_p = par.generate(ids, 6)
+        assert torch.equal(toks_c, toks_p) and torch.equal(logits_c, logits_p)
+        for site in "abcd":
+            for a, b in zip(getattr(cache_c, f"canon_cache_{site}"), getattr(cache_p, f"canon_cache_{site}")):
+                assert torch.equal(bits(a), bits(b)), site
+
+    cfg = viby_config()
+    B, T, steps = 16, 1024, 16
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(5)).to(DEV)
+    times, results = {}, {}
+    for name, parts in (("cat", False), ("parts", True)):
+        m = init_weights(VibyShaped(cfg, hip_factory(cfg, "fused"), parts=parts), 11, torch.bfloat16, DEV)
+        m.generate(ids[:2, :64], 2)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        toks, logits, _ = m.generate(ids, steps, forced=results["cat"][0] if parts else None)
+        torch.cuda.synchronize()
+        times[name] = time.perf_counter() - t0
+        results[name] = (toks, logits)
+        del m
+        torch.cuda.empty_cache()
+    assert torch.equal(results["cat"][1], results["parts"][1])
+    with capsys.disabled():
+        print(f"\n[concat-free Canon-B/D] B{B} x L{T} prefill + {steps} steps: cat path {times['cat']:.3f} s, "
+              f"parts {times['parts']:.3f} s")
+
+
 def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
     cfg = viby_config()
     B, T, steps = 16, 1024, 128
@@ -104,6 +141,21 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
     torch.cuda.synchronize()
     t_ref = time.perf_counter() - t0
 
+    # the same network with the Canon layers switched off: what is left is everything else (projections,
+    # attention, norms, python), so the difference is the share of the 72 Canon calls per forward
+    class NoCanon(torch.nn.Module):
+        def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
+            return x
+    bare = init_weights(VibyShaped(cfg, lambda C, n: NoCanon()), 11, torch.bfloat16, DEV)
+    bare.generate(ids[:2, :64], 2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    bare.generate(ids, steps, forced=toks)
+    torch.cuda.synchronize()
+    t_bare = time.perf_counter() - t0
+    del bare
+    torch.cuda.empty_cache()
+
     # the HIP layers round once where the eager module rounds three times: logits agree to bf16
     # noise accumulated over 18 layers, and the greedy choice agrees wherever it is not a near tie
     diff = (logits - logits_r).abs()
@@ -116,7 +168,8 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
     assert bool(agree[decided].all())
     with capsys.disabled():
         print(f"\n[config 5] B{B} x L{T} prefill + {steps} greedy steps, 18 layers bf16: "
-              f"HIP Canon {t_hip:.2f} s, eager torch Canon {t_ref:.2f} s; "
+              f"HIP Canon {t_hip:.2f} s, eager torch Canon {t_ref:.2f} s, Canon layers off {t_bare:.2f} s "
+              f"(Canon share {100 * (t_hip - t_bare) / t_hip:.0f} % with HIP, {100 * (t_ref - t_bare) / t_ref:.0f} % eager); "
               f"greedy tokens equal at {agree.float().mean().item() * 100:.1f} % of steps "
               f"({decided.float().mean().item() * 100:.1f} % decided beyond rounding noise), "
               f"max |dlogit| {diff.max().item():.4f} of scale {scale:.2f}")

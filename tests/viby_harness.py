@@ -43,8 +43,9 @@ def rotary(x: torch.Tensor, pos: torch.Tensor, theta: float) -> torch.Tensor:
 
 
 class Block(nn.Module):
-    def __init__(self, cfg, make_canon: Callable[[int, str], nn.Module]):
+    def __init__(self, cfg, make_canon: Callable[[int, str], nn.Module], parts: bool = False):
         super().__init__()
+        self.parts = parts
         H, hd = cfg.hidden_size, cfg.head_dim
         self.nq, self.nkv, self.hd, self.theta = cfg.num_attention_heads, cfg.num_key_value_heads, hd, cfg.rope_theta
         self.input_layernorm = nn.RMSNorm(H, eps=cfg.rms_norm_eps)
@@ -64,9 +65,13 @@ class Block(nn.Module):
     def forward(self, h, layer_idx, cache, mask, pos0):
         B, T, _ = h.shape
         x = self.canon_a(self.input_layernorm(h), attention_mask=mask, cache=cache, layer_idx=layer_idx)
-        qkv = torch.cat([self.q_proj(x), self.k_proj(x), self.v_proj(x)], dim=-1)
-        qkv = self.canon_b(qkv, attention_mask=mask, cache=cache, layer_idx=layer_idx)
-        q, k, v = qkv.split([self.nq * self.hd, self.nkv * self.hd, self.nkv * self.hd], dim=-1)
+        if self.parts:      # the projections go to the Canon layer where they are (no cat, no split)
+            q, k, v = self.canon_b.forward_parts((self.q_proj(x), self.k_proj(x), self.v_proj(x)),
+                                                 attention_mask=mask, cache=cache, layer_idx=layer_idx)
+        else:               # model/model.py:772-789
+            qkv = torch.cat([self.q_proj(x), self.k_proj(x), self.v_proj(x)], dim=-1)
+            qkv = self.canon_b(qkv, attention_mask=mask, cache=cache, layer_idx=layer_idx)
+            q, k, v = qkv.split([self.nq * self.hd, self.nkv * self.hd, self.nkv * self.hd], dim=-1)
         q = q.reshape(B, T, self.nq, self.hd).transpose(1, 2)
         k = k.reshape(B, T, self.nkv, self.hd).transpose(1, 2)
         v = v.reshape(B, T, self.nkv, self.hd).transpose(1, 2)
@@ -82,17 +87,20 @@ class Block(nn.Module):
         h = h + self.o_proj(att.transpose(1, 2).reshape(B, T, self.nq * self.hd))
         x = self.canon_c(self.post_attention_layernorm(h), attention_mask=mask, cache=cache, layer_idx=layer_idx)
         gate, up = self.gate_proj(x), self.up_proj(x)
-        gu = self.canon_d(torch.cat([gate, up], dim=-1), attention_mask=mask, cache=cache, layer_idx=layer_idx)
-        gate, up = gu[..., : gate.shape[-1]], gu[..., gate.shape[-1]:]
+        if self.parts:
+            gate, up = self.canon_d.forward_parts((gate, up), attention_mask=mask, cache=cache, layer_idx=layer_idx)
+        else:               # model/model.py:962-971
+            gu = self.canon_d(torch.cat([gate, up], dim=-1), attention_mask=mask, cache=cache, layer_idx=layer_idx)
+            gate, up = gu[..., : gate.shape[-1]], gu[..., gate.shape[-1]:]
         return h + self.down_proj(F.silu(gate) * up)
 
 
 class VibyShaped(nn.Module):
-    def __init__(self, cfg, make_canon):
+    def __init__(self, cfg, make_canon, parts: bool = False):
         super().__init__()
         self.cfg = cfg
         self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size)
-        self.layers = nn.ModuleList(Block(cfg, make_canon) for _ in range(cfg.num_hidden_layers))
+        self.layers = nn.ModuleList(Block(cfg, make_canon, parts) for _ in range(cfg.num_hidden_layers))
         self.norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.rms_norm_eps)
 
     def new_cache(self):

@@ -180,6 +180,14 @@ template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint
     else *(u32x4_t *)p = q;
 }
 
+// (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
+// the value almost always fits 32 bits and one conversion instruction does it
+__device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
+{
+    if ((int32_t)hi == ((int32_t)lo >> 31)) return (float)(int32_t)lo;
+    return (float)(int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 // N mask entries of consecutive time steps t_first .. t_first+N-1 (clamped to
 // [0, L-1]) of one batch row.  The element-type switch sits outside the loops
 // and every case is straight-line code, so all N loads are issued back to back
@@ -205,10 +213,14 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
 #pragma unroll
         for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[idx[j]];
         break;
-    case CANON_MASK_I64:
+    case CANON_MASK_I64: {
+        uint2 q[N];
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const int64_t *)p)[idx[j]];
+        for (int j = 0; j < N; ++j) q[j] = ((const uint2 *)p)[idx[j]];
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = i64_words_to_float(q[j].x, q[j].y);
         break;
+    }
     case CANON_MASK_F32:
 #pragma unroll
         for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[idx[j]];
@@ -222,14 +234,6 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
         for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, idx[j]);
         break;
     }
-}
-
-// (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
-// the value almost always fits 32 bits and one conversion instruction does it
-__device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
-{
-    if ((int32_t)hi == ((int32_t)lo >> 31)) return (float)(int32_t)lo;
-    return (float)(int64_t)(((uint64_t)hi << 32) | lo);
 }
 
 // U runs of N (4 or 8) consecutive mask entries, run u starting at element
@@ -1062,7 +1066,8 @@ struct BwdArgs {
     uint32_t chunk;     // time steps per chunk
     uint32_t nthreads;
     uint32_t nsets;     // partial sets = B * nchunk
-    FastDiv div_nvec, div_nchunk;
+    uint32_t nct;       // blc: channel tiles per row
+    FastDiv div_nvec, div_nchunk, div_nct;
 };
 
 __device__ __forceinline__ float silu_grad(float z)
@@ -1273,6 +1278,383 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 #pragma unroll
         for (int k = 0; k < 4; ++k) pp[e * 5 + k] = k < W ? dw[e][k] : 0.0f;
         pp[e * 5 + 4] = dbs[e];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, channel-contiguous tensors ([B, L, C] viewed as [B, C, L]).
+//
+// A block is four waves; a lane owns the channels of one 8-byte group (4 x
+// 16-bit or 2 x fp32), a wave a slab of kBwdSlab consecutive time steps of a
+// 64-lane channel tile, the four waves four consecutive slabs, and the block
+// walks over the `chunk` time steps of its chunk one such 32-step tile at a
+// time, keeping its dweight / dbias sums in registers.
+//
+// Per tile, all rows of x and dout of the slab are requested before anything
+// is waited for.  The three rows of x before a slab come from the previous
+// wave's slab through LDS (the first wave reads them from memory).  dz of the
+// slab's first three steps is computed first and handed to the previous wave
+// through LDS (that wave's dx needs dz of the three steps after its slab; the
+// last wave recomputes them from three extra rows of x and dout).  The slab is
+// then swept from its last step to its first:
+//   dz[t] = dout[t] * act'(z[t]),  dx[t] = sum_k w[k] * dz[t + (W-1) - k]
+// At the end the four waves' sums are added in a fixed order through LDS and
+// written as one partial set entry per channel.
+// ---------------------------------------------------------------------------
+constexpr int kBwdSlab = 8;    // time steps per wave and tile
+constexpr int kBwdWaves = 4;
+
+template <int DT> __device__ __forceinline__ void unpack_half(const uint2 &v, float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        f[0] = bits_f(v.x);
+        f[1] = bits_f(v.y);
+    } else {
+        unpack2<DT>(v.x, f[0], f[1]);
+        unpack2<DT>(v.y, f[2], f[3]);
+    }
+}
+
+template <int DT> __device__ __forceinline__ uint2 pack_half(const float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) return make_uint2(f_bits(f[0]), f_bits(f[1]));
+    else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
+}
+
+// One raw row -> the bits of xm = x * mask in the storage type (zero when the row does not exist)
+template <int DT, bool MASK>
+__device__ __forceinline__ uint2 bwd_mask_row(const uint2 &raw, float m, bool exists)
+{
+    uint2 v = raw;
+    if constexpr (MASK) {
+        if constexpr (DT == CANON_DTYPE_F32) {
+            v.x = f_bits(bits_f(raw.x) * m);
+            v.y = f_bits(bits_f(raw.y) * m);
+        } else {
+            float f[4];
+            unpack_half<DT>(raw, f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f[e] *= m;
+                if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(f[e]));   // see mul_round
+            }
+            v = pack_half<DT>(f);
+        }
+    }
+    if (!exists) v = make_uint2(0, 0);
+    return v;
+}
+
+// dz of one step from its window of xm rows and dout
+template <int W, int E, bool ACT>
+__device__ __forceinline__ void bwd_dz(const float (*w)[W], const float *bias, const float *x0, const float *x1,
+                                       const float *x2, const float *x3, const float *g, float *dz)
+{
+    if constexpr (ACT) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float z = bias[e];
+            if constexpr (W == 4) z = fmaf(w[e][0], x0[e], z);
+            if constexpr (W >= 3) z = fmaf(w[e][W - 3], x1[e], z);
+            z = fmaf(w[e][W - 2], x2[e], z);
+            z = fmaf(w[e][W - 1], x3[e], z);
+            dz[e] = g[e] * silu_grad(z);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) dz[e] = g[e];
+    }
+}
+
+// The sweep over one slab, last step first.  X / H hold xm in storage bits, dzh the dz of the
+// first three steps (already zero past the end of the sequence), dzf the dz of the three steps
+// after the slab.  FULL: all R steps exist.
+template <int DT, int W, bool MASK, bool ACT, bool FULL, int R, int E>
+__device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W], const float *bias, const uint2 *X,
+                                          const uint2 *H, const uint2 *G, const float *mm, const float (*dzh)[E],
+                                          float (*dzf)[E], float (*dw)[W], float *dbs, char *dxp, int64_t ds, int rows,
+                                          bool active)
+{
+    float xw[4][E];   // xm of rows r-3 .. r
+#pragma unroll
+    for (int k = 0; k < 4; ++k) unpack_half<DT>(X[R - 4 + k], xw[k]);
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) {
+        float g[E], dz[E], o[E];
+        unpack_half<DT>(G[r], g);
+        if (r >= 3) {
+            bwd_dz<W, E, ACT>(w, bias, xw[0], xw[1], xw[2], xw[3], g, dz);
+            if constexpr (!FULL) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = r < rows ? dz[e] : 0.0f;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) dz[e] = dzh[r][e];
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float acc = w[e][W - 1] * dz[e];
+            acc = fmaf(w[e][W - 2], dzf[0][e], acc);
+            if constexpr (W >= 3) acc = fmaf(w[e][W - 3], dzf[1][e], acc);
+            if constexpr (W == 4) acc = fmaf(w[e][0], dzf[2][e], acc);
+            o[e] = acc;
+#pragma unroll
+            for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xw[(4 - W) + k][e], dw[e][k]);
+            dbs[e] += dz[e];
+            dzf[2][e] = dzf[1][e];
+            dzf[1][e] = dzf[0][e];
+            dzf[0][e] = dz[e];
+        }
+        if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += g[e];
+        }
+        if constexpr (MASK) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] *= mm[3 + r];
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += g[e];
+        }
+        if ((FULL || r < rows) && active) *(uint2 *)(dxp + r * ds) = pack_half<DT>(o);
+        if (r > 0) {
+            // slide the window one step back: the new oldest row is r - 4
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                xw[3][e] = xw[2][e];
+                xw[2][e] = xw[1][e];
+                xw[1][e] = xw[0][e];
+            }
+            unpack_half<DT>(r - 4 >= 0 ? X[r - 4 >= 0 ? r - 4 : 0] : H[r - 1 < 3 ? r - 1 : 0], xw[0]);
+        }
+    }
+}
+
+template <int DT, int W, bool MASK, bool ACT>
+__global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
+{
+    constexpr int BY = Elem<DT>::bytes;
+    constexpr int E = 8 / BY;
+    constexpr int R = kBwdSlab, NW = kBwdWaves;
+    __shared__ uint2 tailx[NW][3][64];            // last three xm rows of each wave's slab (storage bits)
+    __shared__ float headdz[NW][3][E][64];        // dz of the first three steps of each wave's slab
+    __shared__ float red[NW - 1][5 * E][64];      // dweight / dbias sums of waves 1..3
+
+    // blockIdx = (b * nchunk + ch) * nct + ct : channel tile fastest, i.e. memory order
+    const uint32_t bc = fdiv(blockIdx.x, a.div_nct);
+    const uint32_t ct = blockIdx.x - bc * a.nct;
+    const uint32_t b = fdiv(bc, a.div_nchunk);
+    const uint32_t ch = bc - b * a.nchunk;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t cv = ct * 64u + lane;
+    const bool active = cv < a.nvec;
+    const uint32_t c0 = (active ? cv : a.nvec - 1u) * E;   // idle lanes shadow the last group: loads need no predicate
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * BY;
+    const char *gb = a.dy + ((int64_t)b * a.g_sb + c0) * BY;
+    char *db_ = a.dx + ((int64_t)b * a.d_sb + c0) * BY;
+    const int64_t xs = a.x_sl * BY, gs = a.g_sl * BY, ds = a.d_sl * BY;
+    const int64_t Lm1 = (int64_t)a.L - 1;
+    const int64_t t_chunk = (int64_t)ch * a.chunk;
+    const int ntiles = (int)(a.chunk / (uint32_t)(R * NW));
+
+    RawTaps<E> rawt;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, rawt);
+    float w[E][W], bias[E];
+
+    // The tiles are walked from the last to the first, so the dz of the three steps after a tile
+    // are the head of the tile done just before (still in headdz[0]).  For the chunk's last tile
+    // the last wave computes them here, from six rows of x and three of dout, and leaves them
+    // in that slot itself.
+    {
+        const int64_t te = t_chunk + (int64_t)a.chunk;   // first step after the chunk (at least 32)
+        uint2 XE[6], GE[3];
+        float me[6];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) {
+            XE[j] = make_uint2(0, 0);
+            me[j] = 1.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) GE[j] = make_uint2(0, 0);
+        if (wv == NW - 1 && te <= Lm1) {
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                const int64_t t = te - 3 + j;
+                XE[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+            }
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = te + j;
+                GE[j] = *(const uint2 *)(gb + (t < Lm1 ? t : Lm1) * gs);
+            }
+            if constexpr (MASK) load_mask_rows<6>(a.mask, (int64_t)b * a.m_sb, te - 3, a.L, a.m_sl, a.mask_dtype, me);
+        }
+        decode_taps<DT, W, E>(rawt, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+        if (wv == NW - 1) {
+            float xt[6][E];
+#pragma unroll
+            for (int j = 0; j < 6; ++j) unpack_half<DT>(bwd_mask_row<DT, MASK>(XE[j], me[j], te - 3 + j <= Lm1), xt[j]);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float g[E], d[E];
+                unpack_half<DT>(GE[j], g);
+                bwd_dz<W, E, ACT>(w, bias, xt[j], xt[j + 1], xt[j + 2], xt[j + 3], g, d);
+                const bool inside = te + j <= Lm1;
+#pragma unroll
+                for (int e = 0; e < E; ++e) headdz[0][j][e][lane] = inside ? d[e] : 0.0f;
+            }
+        }
+    }
+
+    float dw[E][W], dbs[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        dbs[e] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) dw[e][k] = 0.0f;
+    }
+
+    // rows of x and dout, the three rows of x before the slab (first wave) and the mask entries of one tile;
+    // requested one tile ahead, so that they arrive while the tile before is being computed
+    uint2 Xn[R], Gn[R], Hn[3];
+    float mmn[R + 3];   // mask of steps t0-3 .. t0+R-1
+    auto request = [&](int it) {
+        const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
+            Xn[r] = *(const uint2 *)(xb + t * xs);
+            Gn[r] = *(const uint2 *)(gb + t * gs);
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) Hn[j] = make_uint2(0, 0);
+        if (wv == 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = t0 - 3 + j;
+                if (t >= 0) Hn[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < R + 3; ++j) mmn[j] = 1.0f;
+        if constexpr (MASK) load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mmn);
+    };
+    request(ntiles - 1);
+
+    for (int it = ntiles - 1; it >= 0; --it) {
+        const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
+        const int64_t left = (int64_t)a.L - t0;
+        const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
+
+        uint2 X[R], G[R], H[3];
+        float mm[R + 3];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            X[r] = Xn[r];
+            G[r] = Gn[r];
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) H[j] = Hn[j];
+#pragma unroll
+        for (int j = 0; j < R + 3; ++j) mm[j] = mmn[j];
+        if (it > 0) request(it - 1);
+
+        // dz of the three steps after the slab; the last wave's are the previous iteration's head of wave 0
+        float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed
+        if (wv == NW - 1) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[0][j][e][lane];
+        }
+
+        // ---- rows become xm (masked, zero where they do not exist), once ----------------
+        if (MASK || rows < R) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) X[r] = bwd_mask_row<DT, MASK>(X[r], mm[3 + r], r < rows);
+        }
+        if constexpr (MASK) {
+            if (wv == 0) {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) H[j] = bwd_mask_row<DT, MASK>(H[j], mm[j], true);   // zero already when t < 0
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) tailx[wv][j][lane] = X[R - 3 + j];
+        __syncthreads();
+        if (wv > 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) H[j] = tailx[wv - 1][j][lane];
+        }
+
+        // ---- dz of the slab's first three steps, handed to the previous wave ---------
+        float dzh[3][E];
+        {
+            float xq[6][E];   // xm of rows -3 .. 2
+#pragma unroll
+            for (int k = 0; k < 3; ++k) unpack_half<DT>(H[k], xq[k]);
+#pragma unroll
+            for (int k = 0; k < 3; ++k) unpack_half<DT>(X[k], xq[3 + k]);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float g[E];
+                unpack_half<DT>(G[j], g);
+                bwd_dz<W, E, ACT>(w, bias, xq[j], xq[j + 1], xq[j + 2], xq[j + 3], g, dzh[j]);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    dzh[j][e] = j < rows ? dzh[j][e] : 0.0f;
+                    headdz[wv][j][e][lane] = dzh[j][e];
+                }
+            }
+        }
+        __syncthreads();
+        if (wv < NW - 1) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[wv + 1][j][e][lane];
+        }
+
+        // ---- sweep the slab from its last step to its first --------------------------
+        if (rows == R)
+            bwd_sweep<DT, W, MASK, ACT, true, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+        else
+            bwd_sweep<DT, W, MASK, ACT, false, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+    }
+
+    // ---- the four waves' sums, added in the order 0, 1, 2, 3 -----------------------------
+    if (wv > 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) red[wv - 1][e * 5 + k][lane] = dw[e][k];
+            red[wv - 1][e * 5 + 4][lane] = dbs[e];
+        }
+    }
+    __syncthreads();
+    if (wv == 0 && active) {
+        float *pp = a.partial + (((int64_t)b * a.nchunk + ch) * a.C + c0) * 5;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float v = 0.0f;
+                if (k < W) {
+                    v = dw[e][k < W ? k : 0];
+#pragma unroll
+                    for (int q = 0; q < NW - 1; ++q) v += red[q][e * 5 + k][lane];
+                }
+                pp[e * 5 + k] = v;
+            }
+            float v = dbs[e];
+#pragma unroll
+            for (int q = 0; q < NW - 1; ++q) v += red[q][e * 5 + 4][lane];
+            pp[e * 5 + 4] = v;
+        }
     }
 }
 
@@ -2270,6 +2652,7 @@ template <int DT> void launch_update_parts(const UpdPartsPlan &pp, hipStream_t s
 // ---------------------------------------------------------------------------
 enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
 constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
+constexpr int kBwdHalfBlocksPerCU = 3;   // grid target of the channel-contiguous backward, in half blocks per CU
 
 struct BwdPlan {
     BwdKind kind;
@@ -2364,11 +2747,40 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
             return CANON_OK;
         }
     }
-    const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E == 0 && a.x_sl != 1 &&
-                     a.x_sb % E == 0 && a.x_sl % E == 0 && a.g_sb % E == 0 && a.g_sl % E == 0 &&
-                     a.d_sb % E == 0 && a.d_sl % E == 0 && ptrs16;
-    plan->kind = vec ? BWD_BLC_VEC : BWD_GENERIC;
-    a.nvec = vec ? a.C / E : a.C;
+    // channel-contiguous tensors: 8-byte groups of channels per lane
+    const int E8 = 8 / elem_bytes(p->x_dtype);
+    const bool ptrs8 = !check_pointers || ((((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0);
+    const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
+                     a.x_sb % E8 == 0 && a.x_sl % E8 == 0 && a.g_sb % E8 == 0 && a.g_sl % E8 == 0 &&
+                     a.d_sb % E8 == 0 && a.d_sl % E8 == 0 && ptrs8;
+    if (vec) {
+        const uint32_t tile = kBwdSlab * kBwdWaves;
+        const uint32_t nvec = a.C / E8;
+        const uint32_t nct = (nvec + 63) / 64;
+        // time steps per block: as long as possible (few partial sets to write and to add up, taps and
+        // chunk-end work amortised) while the grid still has one and a half blocks per CU
+        uint32_t chunk = tile;
+        for (uint32_t cand = 2 * tile; cand <= 32 * tile; cand *= 2) {
+            const uint64_t blocks = (uint64_t)a.B * ((a.L + cand - 1) / cand) * nct;
+            if (2 * blocks >= 256ull * kBwdHalfBlocksPerCU) chunk = cand;
+        }
+        const uint32_t nchunk = (a.L + chunk - 1) / chunk;
+        const uint64_t blocks = (uint64_t)a.B * nchunk * nct;
+        if (blocks < (1ull << 31)) {
+            plan->kind = BWD_BLC_VEC;
+            a.nvec = nvec; a.nct = nct; a.chunk = chunk; a.nchunk = nchunk;
+            a.nsets = a.B * nchunk;
+            a.div_nct = make_fastdiv(nct); a.div_nchunk = make_fastdiv(nchunk);
+            plan->grid = (uint32_t)blocks;
+            plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+            if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
+                return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                            (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+            return CANON_OK;
+        }
+    }
+    plan->kind = BWD_GENERIC;
+    a.nvec = a.C;
     // time steps per lane: about 8 waves per CU, a multiple of the look-ahead, and few enough
     // partial sets that the scratch stays below ~16 MB
     const uint64_t lanes_per_step = (uint64_t)a.B * a.nvec;
@@ -2407,7 +2819,10 @@ template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStre
         default: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 1, MASK>), g, b, 0, s, pl.args); break;
         }
     } else if (pl.kind == BWD_BLC_VEC)
-        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, Elem<DT>::per_vec, true, MASK, kBwdRows>), g, b, 0, s, pl.args);
+    {
+        if (pl.args.act) hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, true>), g, b, 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, false>), g, b, 0, s, pl.args);
+    }
     else
         hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, 1, false, MASK, kBwdRows>), g, b, 0, s, pl.args);
 }

@@ -12,7 +12,8 @@ structs; time is taken with HIP events on the launch stream.
 
 The one JSON line also carries: the decode update (B=256, C=3456, state 3,
 64 carried steps) in microseconds per step, the same prefill in the
-channel-contiguous layout, the roofline fraction, and a CPU baseline (the
+channel-contiguous layout (one tensor, and gate / up as two tensors through the
+multi-part call), its backward, the roofline fraction, and a CPU baseline (the
 eager PyTorch formulation of the reference on this box's host cores).
 """
 import argparse
@@ -86,6 +87,40 @@ def bench_prefill(layout, steps, warmup, nbuf):
         rc = fwd(refs[i % nbuf], stream)
         if rc:
             _lib.check(rc, "canon_conv1d_fwd")
+
+    ms = time_region(step, steps, warmup)
+    return ms, plan
+
+
+def bench_prefill_parts(steps, warmup, nbuf):
+    """Canon-D as the model produces it: gate and up projections as two (B, L, C/2) tensors, convolved
+    by one multi-part launch (no torch.cat, outputs stay split)."""
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(3)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    keep, calls = [], []
+    for _ in range(nbuf):
+        xs = [torch.randn(B, L, C // 2, generator=g, device=dev).bfloat16().transpose(1, 2) for _ in range(2)]
+        outs = [torch.empty_like(x) for x in xs]
+        p = cc._fill_fwd(xs[0], outs[0], w, bias, None, None, None, 0, 1, 0)
+        p.channels = C
+        p.x = p.out = None
+        arr = cc._part_array(xs, outs)
+        keep.append((xs, outs, p, arr))
+        calls.append((ctypes.byref(p), arr))
+    L_ = _lib.lib()
+    plan = L_.canon_conv1d_fwd_parts_plan(calls[0][0], calls[0][1], 2).decode()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step(i):
+        ref, arr = calls[i % nbuf]
+        rc = L_.canon_conv1d_fwd_parts(ref, arr, 2, stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_fwd_parts")
 
     ms = time_region(step, steps, warmup)
     return ms, plan
@@ -233,6 +268,7 @@ def main():
     nbuf = 6  # 6 x 113 MB = 680 MB of distinct traffic between reuses
     ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
+    ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
     dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
@@ -249,6 +285,9 @@ def main():
         "tokens_per_s": round(B * L / (ms * 1e-3)),
         "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
                                  "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1)},
+        "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",
+                                       "kernel": plan_parts, "ms_per_step": round(ms_parts, 6),
+                                       "GB/s": round(nbytes / (ms_parts * 1e-3) / 1e9, 1)},
         "decode": {"workload": f"configs[3]: bf16 state[{DEC_B},{C},{DEC_S}], {DEC_STEPS} carried steps",
                    "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
                    "us_per_step_hipgraph": round(dec_graph_us, 3),

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 1
+#define CANON_CONV1D_ABI_VERSION 2
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -80,7 +80,8 @@ enum {
  *   xm[b,c,t]  = mask ? round(x[b,c,t] * mask[b,t]) : x[b,c,t]
  *   y[b,c,t]   = act(bias[c] + sum_{k<W} weight[c,k] * xm[b,c,t-(W-1)+k])
  *   out        = y (+ xm | + x)
- * with xm == 0 for t < 0, or the last W-1 entries of initial_state when given.
+ * with xm == 0 for t < 0, or the last W-1 entries of initial_state when given
+ * (with seq_idx: also 0 for every position of another packed sequence).
  * final_state (optional) receives the last final_len entries of
  * initial_state ++ xm, zero filled on the left.
  *
@@ -115,6 +116,12 @@ typedef struct canon_conv1d_fwd_params {
     int32_t final_len;              /* >= 1 when final_state != NULL */
     void *final_state;              /* [batch, channels, final_len], or NULL */
     int64_t final_stride_b, final_stride_c, final_stride_s;
+    const int32_t *seq_idx;         /* [batch, seqlen] or NULL: the `seq_idx` argument of causal_conv1d_fn
+                                       (model/model.py:465 passes None).  Positions of one batch row that
+                                       carry different values belong to different packed sequences: an input
+                                       contributes only to outputs with its own value.  Excludes
+                                       initial_state / final_state. */
+    int64_t seq_stride_b, seq_stride_l;
 } canon_conv1d_fwd_params;
 
 /*
@@ -246,7 +253,7 @@ int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
 
 /*
  * Name of the kernel family the call above would launch for these arguments
- * ("bcl_vec", "blc_vec", "generic", "update_vec", "update_generic"), or NULL
+ * ("bcl_vec", "blc_vec", "blc_vec_seq", "generic", "update_vec", "update_generic"), or NULL
  * if the arguments are rejected.  Launches nothing.  Lets a caller or a test
  * assert that a layout takes the fast path.
  */

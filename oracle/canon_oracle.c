@@ -196,6 +196,50 @@ int canon_oracle_fwd(const void *x, const void *weight, const void *bias, const 
 }
 
 /*
+ * Prefill over packed variable-length sequences: seq_idx [B, L] (int32) names
+ * the sequence every position belongs to, and an input only contributes to
+ * outputs of its own sequence (the `seq_idx` slot of causal_conv1d_fn; the
+ * reference passes None, model/model.py:465, and its MPS backend rejects it,
+ * causal_conv1d_mps/autograd.py:64-65, so this follows the published
+ * behaviour of the upstream package: a tap whose input position carries
+ * another index adds weight * 0).  No initial / final state in this mode.
+ * PARITY UNPINNED against upstream (absent from the reference tree); pinned by
+ * the defining property that a packed row equals its sequences run one by one.
+ */
+int canon_oracle_fwd_seq(const void *x, const void *weight, const void *bias, const float *mask,
+                         const int32_t *seq_idx, void *out, int64_t B, int64_t C, int64_t L, int W,
+                         int dtype, int w_dtype, int use_silu, int residual_mode)
+{
+    if (W < 1 || W > 8 || B < 0 || C < 0 || L < 0 || !seq_idx) return -1;
+    for (int64_t b = 0; b < B; ++b) {
+        for (int64_t c = 0; c < C; ++c) {
+            float w[8];
+            for (int k = 0; k < W; ++k) w[k] = round_to(load_elem(weight, c * W + k, w_dtype), dtype);
+            const float bv = bias ? round_to(load_elem(bias, c, w_dtype), dtype) : 0.0f;
+            const int64_t row = (b * C + c) * L;
+            for (int64_t t = 0; t < L; ++t) {
+                const float xr = load_elem(x, row + t, dtype);
+                const float xm_t = mask ? round_to(xr * mask[b * L + t], dtype) : xr;
+                float acc = bv;
+                for (int k = 0; k < W; ++k) {
+                    const int64_t src = t - (W - 1) + k;
+                    float v = 0.0f;
+                    if (src >= 0 && seq_idx[b * L + src] == seq_idx[b * L + t]) {
+                        v = load_elem(x, row + src, dtype);
+                        if (mask) v = round_to(v * mask[b * L + src], dtype);
+                    }
+                    acc = fmaf(w[k], v, acc);
+                }
+                if (use_silu) acc = silu(acc);
+                if (residual_mode) acc += (residual_mode == 1) ? xm_t : xr;
+                store_elem(out, row + t, dtype, acc);
+            }
+        }
+    }
+    return 0;
+}
+
+/*
  * Decode update, one token.  x, out [B, C]; conv_state [B, C, S] is updated
  * in place: shifted left by one with x appended (pure copies, so bit exact).
  *   out = act(bias + sum_{k<W-1} w[k] * state[S-(W-1)+k] + w[W-1] * x) (+ x)

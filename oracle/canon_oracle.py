@@ -40,6 +40,8 @@ def lib() -> ctypes.CDLL:
         L.canon_oracle_fwd.restype = i32
         L.canon_oracle_fwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64,
                                        i32, i32, i32, i32, i32, i32, i32, i32]
+        L.canon_oracle_fwd_seq.restype = i32
+        L.canon_oracle_fwd_seq.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, i32, i32, i32, i32]
         L.canon_oracle_update.restype = i32
         L.canon_oracle_update.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32,
                                           i32, i32, i32, i32, i32]
@@ -121,6 +123,32 @@ def conv1d_fwd(
     if rc != 0:
         raise ValueError("canon_oracle_fwd rejected its arguments")
     return out if fs is None else (out, fs)
+
+
+def conv1d_fwd_seq(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    seq_idx: torch.Tensor,
+    mask: Optional[torch.Tensor] = None,
+    activation=None,
+    residual=0,
+) -> torch.Tensor:
+    """Prefill oracle over packed sequences (``seq_idx`` [B, L] int32); see ``canon_oracle_fwd_seq``."""
+    assert x.dim() == 3 and weight.dim() == 2 and x.device.type == "cpu"
+    B, C, L = x.shape
+    assert weight.shape[0] == C and tuple(seq_idx.shape) == (B, L)
+    xc, wc = x.contiguous(), weight.contiguous()
+    bc = bias.to(weight.dtype).contiguous() if bias is not None else None
+    mc = mask.to(torch.float32).contiguous() if mask is not None else None
+    sc = seq_idx.to(torch.int32).contiguous()
+    out = torch.empty_like(xc)
+    rc = lib().canon_oracle_fwd_seq(
+        _ptr(xc), _ptr(wc), _ptr(bc), _ptr(mc), _ptr(sc), _ptr(out), B, C, L, weight.shape[1],
+        _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype], _act(activation), _res_mode(residual))
+    if rc != 0:
+        raise ValueError("canon_oracle_fwd_seq rejected its arguments")
+    return out
 
 
 def conv1d_update(

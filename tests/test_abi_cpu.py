@@ -190,8 +190,10 @@ def test_wrapper_errors_match_reference_conventions():
         cc.causal_conv1d_fn(x, torch.randn(4, 4), torch.randn(3))
     with pytest.raises(NotImplementedError, match="activation must be None, silu, or swish"):
         cc.causal_conv1d_fn(x, torch.randn(4, 4), activation="relu")
-    with pytest.raises(NotImplementedError, match="seq_idx"):
-        cc.causal_conv1d_fn(x, torch.randn(4, 4), seq_idx=torch.zeros(2, 8, dtype=torch.int32))
+    with pytest.raises(ValueError, match="seq_idx shape"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), seq_idx=torch.zeros(2, 9, dtype=torch.int32))
+    with pytest.raises(ValueError, match="cannot be combined with seq_idx"):
+        cc.causal_conv1d_fn(x, torch.randn(4, 4), seq_idx=torch.zeros(2, 8, dtype=torch.int32), return_final_states=True)
     with pytest.raises(NotImplementedError, match="width 5"):
         cc.causal_conv1d_fn(x, torch.randn(4, 5))
     with pytest.raises(ValueError, match="Unsupported input dtype"):
@@ -342,3 +344,13 @@ def test_parts_plan_and_validation():
     assert uplan_parts(update_params(C=3456, S=5), make_parts([1728, 1728], L=1)) == "per_part"
     assert uplan_parts(update_params(C=3456, S=3), make_parts([3456], L=1)) == "per_part"
     assert uplan_parts(update_params(C=3457, S=3), make_parts([1728, 1728], L=1)) is None
+
+
+def test_seq_idx_plan_and_validation():
+    FAKE_SEQ = 0x50000000
+    assert plan(fwd_params(layout="blc", seq_idx=FAKE_SEQ, seq_stride_b=1024, seq_stride_l=1)) == "blc_vec_seq"
+    assert plan(fwd_params(layout="bcl", seq_idx=FAKE_SEQ, seq_stride_b=1024, seq_stride_l=1)) == "generic"
+    assert plan(fwd_params(layout="blc", seq_idx=FAKE_SEQ + 2, seq_stride_b=1024, seq_stride_l=1)) is None
+    assert "4-byte aligned" in last_error()
+    assert plan(fwd_params(layout="blc", seq_idx=FAKE_SEQ, final_state=FAKE_STATE, final_len=3)) is None
+    assert "seq_idx excludes" in last_error()

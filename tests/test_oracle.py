@@ -380,3 +380,39 @@ def test_eager_step_mode_reproduces_eager_module(dtype):
             else:
                 d = ulp_diff(got, want)
                 assert d.max().item() <= 1 and (d > 0).float().mean().item() < 0.02
+
+
+# ---- packed sequences (seq_idx): pinned by brute force and by the defining property ------------
+def test_seq_idx_oracle_brute_force_and_separate_sequences():
+    g = torch.Generator().manual_seed(81)
+    for W, L in itertools.product([2, 3, 4], [1, 2, 5, 9, 17]):
+        B, C = 2, 3
+        x = torch.randn(B, C, L, generator=g)
+        w = torch.randn(C, W, generator=g)
+        b = torch.randn(C, generator=g)
+        seq = torch.randint(0, 3, (B, L), generator=g).sort(dim=1).values.to(torch.int32)
+        got = co.conv1d_fwd_seq(x, w, b, seq)
+        # index by index, every tap spelled out
+        for bi, c, t in itertools.product(range(B), range(C), range(L)):
+            acc = np.float32(b[c])
+            for k in range(W):
+                src = t - (W - 1) + k
+                v = np.float32(x[bi, c, src]) if src >= 0 and seq[bi, src] == seq[bi, t] else np.float32(0)
+                # the product of two floats is exact in float64, so this is the fused multiply-add up to double rounding
+                acc = np.float32(np.float64(np.float32(w[c, k])) * np.float64(v) + np.float64(acc))
+            assert abs(float(got[bi, c, t]) - float(acc)) <= 1e-6 * max(1.0, abs(float(acc))), (W, L, bi, c, t)
+        # a packed row equals its sequences run one by one, bit for bit
+        for bi in range(B):
+            bounds = [0] + [t for t in range(1, L) if seq[bi, t] != seq[bi, t - 1]] + [L]
+            for lo, hi in zip(bounds[:-1], bounds[1:]):
+                alone = co.conv1d_fwd(x[bi:bi + 1, :, lo:hi].contiguous(), w, b)
+                assert torch.equal(got[bi:bi + 1, :, lo:hi], alone), (W, L, bi, lo, hi)
+    # one sequence per row is the plain conv; SiLU, mask and residual ride along unchanged
+    x = torch.randn(2, 4, 33, generator=g).bfloat16()
+    w = torch.randn(4, 4, generator=g).bfloat16()
+    mask = (torch.rand(2, 33, generator=g) > 0.3).to(torch.int64)
+    same = torch.zeros(2, 33, dtype=torch.int32)
+    for act, res in [(None, 0), ("silu", 1), ("silu", 2)]:
+        a = co.conv1d_fwd_seq(x, w, None, same, mask=mask, activation=act, residual=res)
+        b_ = co.conv1d_fwd(x, w, None, mask=mask, activation=act, residual=res)
+        assert torch.equal(a.view(torch.int16), b_.view(torch.int16))

@@ -365,8 +365,10 @@ def test_errors_surface(cc):
         cc.causal_conv1d_fn(x, torch.randn(5, 4, device=DEV))
     with pytest.raises(NotImplementedError, match="width"):
         cc.causal_conv1d_fn(x, torch.randn(8, 5, device=DEV))
-    with pytest.raises(NotImplementedError):
-        cc.causal_conv1d_fn(x, w, seq_idx=torch.zeros(2, 16, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError, match="int32"):
+        cc.causal_conv1d_fn(x, w, seq_idx=torch.zeros(2, 16, dtype=torch.int64, device=DEV))
+    with pytest.raises(NotImplementedError, match="seq_idx"):
+        cc.causal_conv1d_fn(x.clone().requires_grad_(), w, seq_idx=torch.zeros(2, 16, dtype=torch.int32, device=DEV))
     with pytest.raises(ValueError, match="shorter than width-1"):
         cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 2, device=DEV), w)
     with pytest.raises(NotImplementedError, match="backward"):
@@ -396,3 +398,55 @@ def test_integer_mask_narrowing_is_never_stale(cc):
     sliced = torch.cat([m2, m1], dim=1).to(DEV)[:, -L:]      # a view, as CanonLayer slices it
     got = cc.causal_conv1d_fn(xg, wg, attention_mask=sliced, residual=True)
     assert_parity(got, co.conv1d_fwd(x, w, None, mask=m1, residual=1), exact=True, what="narrowed mask view")
+
+
+# ---- packed variable-length sequences (seq_idx) --------------------------------
+def packed_seq_idx(B, L, gen, max_seqs=6):
+    """Per batch row: L positions cut into 1..max_seqs consecutive sequences (some of length 1..3)."""
+    seq = torch.zeros(B, L, dtype=torch.int32)
+    for b in range(B):
+        n = int(torch.randint(1, max_seqs + 1, (1,), generator=gen))
+        cuts = sorted(set(torch.randint(1, max(L, 2), (n - 1,), generator=gen).tolist())) if L > 1 else []
+        for i, c in enumerate(cuts):
+            seq[b, c:] = i + 1
+    return seq
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_seq_idx_matches_oracle_and_separate_calls(cc, dtype):
+    g = torch.Generator().manual_seed(71)
+    for (B, C, L), W in itertools.product([(3, 64, 100), (2, 520, 37), (1, 8, 5), (4, 24, 257)], [2, 3, 4]):
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, W, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        seq = packed_seq_idx(B, L, g)
+        seq[0, :] = seq[0, :] * 7 + 3                    # the values only matter through equality
+        mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+        for act, res, m in [(None, False, None), ("silu", "masked", mask), (None, "unmasked", mask)]:
+            want = co.conv1d_fwd_seq(x, w, b, seq, mask=m, activation=act, residual=res)
+            for name, xg in layouts(x):
+                plan = cc.kernel_plan_fwd(xg, w.to(DEV), seq_idx=seq.to(DEV))
+                assert plan == ("blc_vec_seq" if name == "blc" and C % (16 // x.element_size()) == 0 else "generic")
+                got = cc.causal_conv1d_fn(xg, w.to(DEV), b.to(DEV), seq_idx=seq.to(DEV), activation=act,
+                                          attention_mask=None if m is None else m.to(DEV), residual=res)
+                xm = x if m is None else (x.float() * m[:, None, :].float()).to(dtype)
+                assert_parity(got, want, exact=act is None, what=f"seq/{dtype}/{B}x{C}x{L}/W{W}/{act}/{res}/{name}",
+                              res=xm if res else None)
+        # the defining property: a packed row equals its sequences convolved one by one
+        xg = x.to(DEV).transpose(1, 2).contiguous().transpose(1, 2)
+        packed = cc.causal_conv1d_fn(xg, w.to(DEV), b.to(DEV), seq_idx=seq.to(DEV), activation="silu")
+        for bi in range(B):
+            bounds = [0] + [t for t in range(1, L) if seq[bi, t] != seq[bi, t - 1]] + [L]
+            for lo, hi in zip(bounds[:-1], bounds[1:]):
+                alone = cc.causal_conv1d_fn(xg[bi:bi + 1, :, lo:hi], w.to(DEV), b.to(DEV), activation="silu")
+                assert torch.equal(bits(packed[bi:bi + 1, :, lo:hi]), bits(alone)), (bi, lo, hi)
+
+
+def test_seq_idx_constant_is_no_seq_idx(cc):
+    g = torch.Generator().manual_seed(72)
+    x = torch.randn(8, 3456, 256, generator=g).bfloat16().to(DEV).transpose(1, 2).contiguous().transpose(1, 2)
+    w = (torch.randn(3456, 4, generator=g) * 0.02).bfloat16().to(DEV)
+    seq = torch.full((8, 256), 5, dtype=torch.int32, device=DEV)
+    a = cc.causal_conv1d_fn(x, w, seq_idx=seq, residual=True)
+    b = cc.causal_conv1d_fn(x, w, residual=True)
+    assert torch.equal(bits(a), bits(b))

@@ -143,7 +143,7 @@ def _stream(dev: torch.device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
 
-def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd) -> FwdParams:
+def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx=None) -> FwdParams:
     p = FwdParams()
     p.struct_size = ctypes.sizeof(FwdParams)
     p.x_dtype = _lib.DTYPE_CODE[x.dtype]
@@ -170,6 +170,9 @@ def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res
         p.final_state = final_states.data_ptr()
         p.final_stride_b, p.final_stride_c, p.final_stride_s = final_states.stride()
         p.final_len = final_states.shape[2]
+    if seq_idx is not None:
+        p.seq_idx = seq_idx.data_ptr()
+        p.seq_stride_b, p.seq_stride_l = seq_idx.stride()
     return p
 
 
@@ -236,6 +239,10 @@ def causal_conv1d_fn(
     contiguous or channel contiguous (a transposed (batch, seqlen, dim) tensor,
     which is what ``model/model.py:459`` passes); the output has x's strides.
 
+    seq_idx          (batch, seqlen) int32: packed variable-length sequences; positions
+                     with different values do not see each other (the slot the
+                     reference leaves at None, ``model/model.py:465``).  Inference
+                     only, without initial / final states.
     initial_states   (batch, dim, >= W-1): history before t = 0 instead of zeros.
     return_final_states / final_states_out (batch, dim, S): receives the last S
                      inputs (S = W-1 when allocated here; any S >= 1 when
@@ -255,10 +262,18 @@ def causal_conv1d_fn(
     act = _activation_flag(activation)
     res = _residual_mode(residual)
     rnd = _round_mode(rounding)
-    if seq_idx is not None:
-        raise NotImplementedError("seq_idx (packed variable-length batches) is not supported")
     if x.dim() != 3:
         raise ValueError(f"Expected 3D input tensor (batch, dim, seqlen), got {x.dim()}D")
+    if seq_idx is not None:
+        if initial_states is not None or return_final_states or final_states_out is not None:
+            raise ValueError("initial_states / final states cannot be combined with seq_idx")
+        if seq_idx.dim() != 2 or tuple(seq_idx.shape) != (x.shape[0], x.shape[2]):
+            raise ValueError(f"seq_idx shape {tuple(seq_idx.shape)} does not match (batch, seqlen) = "
+                             f"({x.shape[0]}, {x.shape[2]})")
+        if seq_idx.dtype != torch.int32 or seq_idx.device != x.device:
+            raise ValueError("seq_idx must be an int32 tensor on the device of x")
+        if _wants_grad(x, weight, bias):
+            raise NotImplementedError("gradients of a call with seq_idx are not implemented")
     bias, attention_mask, final_states = _check_fwd_args(
         x, tuple(x.shape), weight, bias, attention_mask, initial_states, return_final_states, final_states_out)
 
@@ -272,17 +287,17 @@ def causal_conv1d_fn(
             raise NotImplementedError("gradients through a call with initial_states are not implemented")
         result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd)
     else:
-        result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+        result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd, seq_idx)
         if final_states is not None:
             result = (result, final_states)
     return result
 
 
-def _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd) -> torch.Tensor:
+def _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx=None) -> torch.Tensor:
     out = torch.empty_like(x)
     if x.numel() == 0:
         return out
-    p = _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd)
+    p = _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx)
     with torch.cuda.device(x.device):
         rc = _lib.lib().canon_conv1d_fwd(ctypes.byref(p), _stream(x.device))
     _lib.check(rc, "causal_conv1d_fn")
@@ -656,11 +671,11 @@ def short_conv_update(
 # introspection (lets callers and tests assert that a layout takes a fast path)
 # ---------------------------------------------------------------------------
 def kernel_plan_fwd(x, weight, bias=None, activation=None, attention_mask=None, residual=False,
-                    rounding="fused", initial_states=None, final_states_out=None) -> str:
-    """Kernel family ``causal_conv1d_fn`` would launch: 'bcl_vec', 'blc_vec' or 'generic'."""
+                    rounding="fused", initial_states=None, final_states_out=None, seq_idx=None) -> str:
+    """Kernel family ``causal_conv1d_fn`` would launch: 'bcl_vec', 'blc_vec', 'blc_vec_seq' or 'generic'."""
     out = torch.empty_like(x)
     p = _fill_fwd(x, out, weight, _prep_bias(weight, bias), attention_mask, initial_states, final_states_out,
-                  _activation_flag(activation), _residual_mode(residual), _round_mode(rounding))
+                  _activation_flag(activation), _residual_mode(residual), _round_mode(rounding), seq_idx)
     name = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(p))
     if name is None:
         _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_fwd")

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -41,6 +41,7 @@ class FwdParams(ctypes.Structure):
         ("initial_state", _vp), ("init_stride_b", _i64), ("init_stride_c", _i64), ("init_stride_s", _i64),
         ("initial_len", _i32), ("final_len", _i32),
         ("final_state", _vp), ("final_stride_b", _i64), ("final_stride_c", _i64), ("final_stride_s", _i64),
+        ("seq_idx", _vp), ("seq_stride_b", _i64), ("seq_stride_l", _i64),
     ]
 
 

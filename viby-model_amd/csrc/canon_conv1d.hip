@@ -236,6 +236,19 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
     }
 }
 
+// N sequence indices of consecutive time steps t_first .. t_first+N-1 (clamped to [0, L-1]) of one batch row
+template <int N>
+__device__ __forceinline__ void load_seq_rows(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
+                                              int32_t *q)
+{
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        int64_t t = t_first + j;
+        t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+        q[j] = p[row_base + t * stride];
+    }
+}
+
 // U runs of N (4 or 8) consecutive mask entries, run u starting at element
 // base[u].  The element-type switch sits outside the loops and every case is
 // straight-line code, so all loads are issued back to back and waited for
@@ -410,6 +423,8 @@ struct FwdArgs {
     const void *mask;
     const void *init;
     void *fin;
+    const int32_t *seq;
+    int64_t q_sb, q_sl;
     int64_t x_sb, x_sc, x_sl;
     int64_t o_sb, o_sc, o_sl;
     int64_t w_sc, w_sk;
@@ -753,9 +768,12 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 // wave of a block reads its halo from memory.  All loads (slab, halo, taps)
 // are issued before the first wait.
 // ---------------------------------------------------------------------------
+// keep0..2 (wave uniform): whether the rows t-3, t-2, t-1 belong to the packed sequence of row t
+// (always true without seq_idx); a row of another sequence enters as zeros.
 template <int DT, int W, bool MASK, bool NT>
 __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias, float (*hist)[Elem<DT>::per_vec],
-                                        const uint4 &X, float m, char *optr, bool active)
+                                        const uint4 &X, float m, char *optr, bool active, bool keep0 = true,
+                                        bool keep1 = true, bool keep2 = true)
 {
     constexpr int E = Elem<DT>::per_vec;
     float xr[E], xm_store[MASK ? E : 1], o[E];
@@ -768,9 +786,9 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         float acc = bias[e];
-        if constexpr (W == 4) acc = fmaf(w[e][0], hist[0][e], acc);
-        if constexpr (W >= 3) acc = fmaf(w[e][W - 3], hist[1][e], acc);
-        acc = fmaf(w[e][W - 2], hist[2][e], acc);
+        if constexpr (W == 4) acc = fmaf(w[e][0], keep0 ? hist[0][e] : 0.0f, acc);
+        if constexpr (W >= 3) acc = fmaf(w[e][W - 3], keep1 ? hist[1][e] : 0.0f, acc);
+        acc = fmaf(w[e][W - 2], keep2 ? hist[2][e] : 0.0f, acc);
         acc = fmaf(w[e][W - 1], xm[e], acc);
         o[e] = acc;
         hist[0][e] = hist[1][e];
@@ -793,7 +811,7 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
 
 constexpr int kBlcWaves = 4;   // waves (time slabs) per block
 
-template <int DT, int W, int R, bool MASK, bool NT>
+template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false>
 __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 {
     constexpr int E = Elem<DT>::per_vec;
@@ -824,12 +842,15 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     // Rows past the end of the sequence are clamped to the last row (loaded, never used).
     uint4 X[R], H[3];
     float m[R], mh[3];
+    int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         X[r] = make_uint4(0, 0, 0, 0);
         m[r] = 0.0f;
     }
+#pragma unroll
+    for (int j = 0; j < (SEQ ? R + 3 : 1); ++j) sq[j] = 0;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
         H[j] = make_uint4(0, 0, 0, 0);
@@ -850,6 +871,7 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
         }
         // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
         fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+        if constexpr (SEQ) load_seq_rows<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, sq);
         if constexpr (MASK) {
             // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
             float mm[R + 3];
@@ -894,7 +916,18 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 
-    if (rows == R) {
+    if constexpr (SEQ) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= rows) continue;
+            // rows t-3, t-2, t-1 count only if they carry the index of row t; sequence boundaries are rare,
+            // so the all-kept case takes the plain code
+            const int32_t cur = sq[3 + r];
+            const bool k0 = sq[r] == cur, k1 = sq[r + 1] == cur, k2 = sq[r + 2] == cur;
+            if (k0 && k1 && k2) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+            else blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active, k0, k1, k2);
+        }
+    } else if (rows == R) {
 #pragma unroll
         for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
     } else {
@@ -932,6 +965,13 @@ template <int DT, int W, int R, bool MASK, bool NT>
 __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
 {
     blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
+}
+
+// the same over packed variable-length sequences (seq_idx)
+template <int DT, int W, int R, bool MASK>
+__global__ __launch_bounds__(256) void canon_fwd_blc_seq_kernel(const FwdArgs a)
+{
+    blc_block<DT, W, R, MASK, false, true>(a, blockIdx.x);
 }
 
 // Several channel ranges of one logical [B, C, L] problem that live in separate
@@ -995,12 +1035,15 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
     const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
 
     float h[3] = {0, 0, 0};
+    int32_t qh[3] = {0, 0, 0};   // with seq_idx: the sequence each history position belongs to
+    const int32_t *seq = a.seq ? a.seq + (int64_t)b * a.q_sb : nullptr;
     for (int j = 4 - W; j < 3; ++j) {
         const int64_t t = t_begin - 3 + j;
         if (t >= 0) {
             float v = load1<DT>(a.x, xo + t * a.x_sl);
             if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
             h[j] = v;
+            if (seq) qh[j] = seq[t * a.q_sl];
         } else if (a.init && a.S_in + t >= 0) {
             h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
         }
@@ -1010,10 +1053,22 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
         float xm = xr;
         if (a.mask) xm = mul_round<DT>(xr, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
         float acc = bv;
-        if (W == 4) acc = fmaf(w[0], h[0], acc);
-        if (W >= 3) acc = fmaf(w[1], h[1], acc);
-        acc = fmaf(w[2], h[2], acc);
-        acc = fmaf(w[3], xm, acc);
+        if (seq) {
+            // inputs of another packed sequence enter as zeros
+            const int32_t qt = seq[t * a.q_sl];
+            if (W == 4) acc = fmaf(w[0], qh[0] == qt ? h[0] : 0.0f, acc);
+            if (W >= 3) acc = fmaf(w[1], qh[1] == qt ? h[1] : 0.0f, acc);
+            acc = fmaf(w[2], qh[2] == qt ? h[2] : 0.0f, acc);
+            acc = fmaf(w[3], xm, acc);
+            qh[0] = qh[1];
+            qh[1] = qh[2];
+            qh[2] = qt;
+        } else {
+            if (W == 4) acc = fmaf(w[0], h[0], acc);
+            if (W >= 3) acc = fmaf(w[1], h[1], acc);
+            acc = fmaf(w[2], h[2], acc);
+            acc = fmaf(w[3], xm, acc);
+        }
         if (a.eager) {
             acc = round_through<DT>(acc);
             if (a.act) acc = round_through<DT>(silu_precise(acc));
@@ -2210,12 +2265,17 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
         return fail(CANON_ERR_INVALID_ARGUMENT, "final_len %d must be at least 1", p->final_len);
     if (p->final_state && p->final_len > 64)
         return fail(CANON_ERR_UNSUPPORTED, "final_len %d above 64 is not supported", p->final_len);
+    if (p->seq_idx && (p->initial_state || p->final_state))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx excludes initial_state and final_state");
+    if (p->seq_idx && ((uintptr_t)p->seq_idx & 3u))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx must be 4-byte aligned");
 
     FwdArgs &a = plan->args;
     memset(&a, 0, sizeof(a));
     a.x = (const char *)p->x; a.out = (char *)p->out;
     a.weight = p->weight; a.bias = p->bias; a.mask = p->mask;
     a.init = p->initial_state; a.fin = p->final_state;
+    a.seq = p->seq_idx; a.q_sb = p->seq_stride_b; a.q_sl = p->seq_stride_l;
     a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.x_sl = p->x_stride_l;
     a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c; a.o_sl = p->out_stride_l;
     a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
@@ -2241,7 +2301,9 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.nt = 2 * rows * a.L * elem_bytes(p->x_dtype) >= kStreamBytes;
     const bool fused = p->round_mode == CANON_ROUND_FUSED;
     const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
-    const bool bcl_ok = fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
+    // packed sequences: the channel-contiguous kernel has a variant (the index is uniform per time row);
+    // time-contiguous rows take the strided kernel
+    const bool bcl_ok = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
                         a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0 &&
                         a.L / E >= 16;
     const bool blc_ok = fused && ptr_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 &&
@@ -2315,6 +2377,11 @@ template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 {
     const bool mask = pl.args.mask != nullptr;
+    if (pl.args.seq) {   // only the channel-contiguous kernel is planned with seq_idx
+        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        return;
+    }
     // the streaming (non-temporal) variants exist for width 4 only
     if (W == 4 && pl.args.nt) {
         if (mask) launch_fwd_vec<DT, W, true, W == 4>(pl, s);
@@ -2511,7 +2578,7 @@ int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *pa
     // whether to stream past the caches is decided on the whole problem
     const bool nt = 2ull * (uint64_t)p->batch * (uint64_t)p->channels * (uint64_t)p->seqlen * xb >= kStreamBytes;
     for (int i = 0; i < nparts; ++i) pp->part[i].args.nt = nt;
-    pp->single = nparts > 1 && all_blc && p->width == 4 && blocks > 0 && blocks < (1ull << 31);
+    pp->single = nparts > 1 && all_blc && p->width == 4 && !p->seq_idx && blocks > 0 && blocks < (1ull << 31);
     pp->grid = (uint32_t)blocks;
     return CANON_OK;
 }
@@ -2927,6 +2994,7 @@ const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)
 {
     FwdPlan pl;
     if (plan_fwd(p, &pl) != CANON_OK) return nullptr;
+    if (pl.kind == FWD_BLC && pl.args.seq) return "blc_vec_seq";
     return pl.kind == FWD_BCL ? "bcl_vec" : pl.kind == FWD_BLC ? "blc_vec" : "generic";
 }
 

@@ -325,7 +325,8 @@ def test_parts_plan_and_validation():
     assert fplan(fwd_params(C=960), make_parts([640, 320], layout="bcl")) == "per_part"
     assert fplan(fwd_params(C=640, layout="blc"), make_parts([640])) == "per_part"
     assert fplan(fwd_params(C=960, layout="blc", width=3, w_stride_c=3), make_parts([640, 320])) == "per_part"
-    assert fplan(fwd_params(C=100, layout="blc"), make_parts([60, 40])) == "per_part"
+    assert fplan(fwd_params(C=100, layout="blc"), make_parts([60, 40])) == "blc_vec_parts"     # 8-byte channel groups
+    assert fplan(fwd_params(C=102, layout="blc"), make_parts([62, 40])) == "per_part"
     # rejected
     assert fplan(fwd_params(C=961, layout="blc"), make_parts([640, 160, 160])) is None
     assert "960 channels" in last_error() and "961" in last_error()

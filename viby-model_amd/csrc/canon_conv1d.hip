@@ -236,6 +236,53 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
     }
 }
 
+// A lane's access unit in the channel-contiguous kernels: 16 bytes, or 8 bytes (half the registers
+// per lane, twice the waves in flight)
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+template <int VB> struct VecIO;
+template <> struct VecIO<16> {
+    using type = uint4;
+    static __device__ __forceinline__ type zero() { return make_uint4(0, 0, 0, 0); }
+    template <bool NT> static __device__ __forceinline__ type load(const void *p) { return load_vec<NT>(p); }
+    template <bool NT> static __device__ __forceinline__ void store(void *p, const type &v) { store_vec<NT>(p, v); }
+    template <int DT> static __device__ __forceinline__ void unpack(const type &v, float *f) { unpack_vec<DT>(v, f); }
+    template <int DT> static __device__ __forceinline__ type pack(const float *f) { return pack_vec<DT>(f); }
+};
+template <> struct VecIO<8> {
+    using type = uint2;
+    static __device__ __forceinline__ type zero() { return make_uint2(0, 0); }
+    template <bool NT> static __device__ __forceinline__ type load(const void *p)
+    {
+        const u32x2_t *q = (const u32x2_t *)p;
+        u32x2_t v;
+        if constexpr (NT) v = __builtin_nontemporal_load(q);
+        else v = *q;
+        return make_uint2(v.x, v.y);
+    }
+    template <bool NT> static __device__ __forceinline__ void store(void *p, const type &v)
+    {
+        const u32x2_t q = {v.x, v.y};
+        if constexpr (NT) __builtin_nontemporal_store(q, (u32x2_t *)p);
+        else *(u32x2_t *)p = q;
+    }
+    template <int DT> static __device__ __forceinline__ void unpack(const type &v, float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) {
+            f[0] = bits_f(v.x);
+            f[1] = bits_f(v.y);
+        } else {
+            unpack2<DT>(v.x, f[0], f[1]);
+            unpack2<DT>(v.y, f[2], f[3]);
+        }
+    }
+    template <int DT> static __device__ __forceinline__ type pack(const float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return make_uint2(f_bits(f[0]), f_bits(f[1]));
+        else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
+    }
+};
+
 // N sequence indices of consecutive time steps t_first .. t_first+N-1 (clamped to [0, L-1]) of one batch row
 template <int N>
 __device__ __forceinline__ void load_seq_rows(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
@@ -757,12 +804,13 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 // prefill, channel-contiguous rows ([B, L, C] memory, x_stride_c == 1): the
 // layout CanonLayer hands over (a transposed view of [B, T, D]).
 //
-// One lane owns E adjacent channels (16 bytes of every row) and R consecutive
-// time steps; the four waves of a block own four consecutive R-row slabs of
-// the same 64-lane channel tile, so a block streams a [4R rows] x [1 KB] tile
-// and consecutive blocks sweep memory in address order (short-lived waves over
-// a compact window: measured to be what HBM wants; long per-lane time runs
-// lose 10-20 %).  The three rows a wave needs from before its slab are the
+// One lane owns E adjacent channels (VB = 8 bytes of every row: 4 x 16-bit or
+// 2 x fp32; 16-byte lanes need 142 registers and measured 4-9 % slower) and R
+// consecutive time steps; the four waves of a block own four consecutive
+// R-row slabs of the same 64-lane channel tile, so a block streams a
+// [4R rows] x [512 B] tile and consecutive blocks sweep memory in address
+// order (short-lived waves over a compact window: measured to be what HBM
+// wants; long per-lane time runs lose 10-20 %).  The three rows a wave needs from before its slab are the
 // last three rows of the previous wave: each wave publishes the raw tail of
 // its slab in LDS, one barrier, the next wave picks it up -- only the first
 // wave of a block reads its halo from memory.  All loads (slab, halo, taps)
@@ -770,15 +818,15 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 // ---------------------------------------------------------------------------
 // keep0..2 (wave uniform): whether the rows t-3, t-2, t-1 belong to the packed sequence of row t
 // (always true without seq_idx); a row of another sequence enters as zeros.
-template <int DT, int W, bool MASK, bool NT>
-__device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias, float (*hist)[Elem<DT>::per_vec],
-                                        const uint4 &X, float m, char *optr, bool active, bool keep0 = true,
-                                        bool keep1 = true, bool keep2 = true)
+template <int DT, int W, bool MASK, bool NT, int VB>
+__device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias,
+                                        float (*hist)[VB / Elem<DT>::bytes], const typename VecIO<VB>::type &X, float m,
+                                        char *optr, bool active, bool keep0 = true, bool keep1 = true, bool keep2 = true)
 {
-    constexpr int E = Elem<DT>::per_vec;
+    constexpr int E = VB / Elem<DT>::bytes;
     float xr[E], xm_store[MASK ? E : 1], o[E];
     float *xm = MASK ? xm_store : xr;
-    unpack_vec<DT>(X, xr);
+    VecIO<VB>::template unpack<DT>(X, xr);
     if constexpr (MASK) {
 #pragma unroll
         for (int e = 0; e < E; ++e) xm[e] = mul_round<DT>(xr[e], m);
@@ -806,17 +854,20 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] += xm[e];
     }
-    if (active) store_vec<NT>(optr, pack_vec<DT>(o));
+    if (active) VecIO<VB>::template store<NT>(optr, VecIO<VB>::template pack<DT>(o));
 }
 
 constexpr int kBlcWaves = 4;   // waves (time slabs) per block
+constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 % faster than 16 (half the registers, twice the waves)
 
-template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false>
+template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
 __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 {
-    constexpr int E = Elem<DT>::per_vec;
+    constexpr int E = VB / Elem<DT>::bytes;
+    using V = VecIO<VB>;
+    using vec_t = typename V::type;
     static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
-    __shared__ uint4 tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
+    __shared__ vec_t tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
 
     // blocks in plain memory order (an XCD-contiguous remap measured 3 % slower here)
     // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
@@ -840,37 +891,37 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 
     // slab rows, then (first wave only) the three rows before the block, then the taps.
     // Rows past the end of the sequence are clamped to the last row (loaded, never used).
-    uint4 X[R], H[3];
+    vec_t X[R], H[3];
     float m[R], mh[3];
     int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        X[r] = make_uint4(0, 0, 0, 0);
+        X[r] = V::zero();
         m[r] = 0.0f;
     }
 #pragma unroll
     for (int j = 0; j < (SEQ ? R + 3 : 1); ++j) sq[j] = 0;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-        H[j] = make_uint4(0, 0, 0, 0);
+        H[j] = V::zero();
         mh[j] = 0.0f;
     }
     if (rows > 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t t = t0 + r < t_last ? t0 + r : t_last;
-            X[r] = load_vec<NT>(xb + t * xs);
+            X[r] = V::template load<NT>(xb + t * xs);
         }
         if (wv == 0) {
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
                 const int64_t t = t0 - 3 + j;
-                if (j >= 3 - (W - 1) && t >= 0) H[j] = load_vec<false>(xb + t * xs);
+                if (j >= 3 - (W - 1) && t >= 0) H[j] = V::template load<false>(xb + t * xs);
             }
         }
         // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
-        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
         if constexpr (SEQ) load_seq_rows<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, sq);
         if constexpr (MASK) {
             // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
@@ -898,7 +949,7 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     float hist[3][E];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-        unpack_vec<DT>(H[j], hist[j]);
+        V::template unpack<DT>(H[j], hist[j]);
         if constexpr (MASK) {
 #pragma unroll
             for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mh[j]);
@@ -924,16 +975,16 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
             // so the all-kept case takes the plain code
             const int32_t cur = sq[3 + r];
             const bool k0 = sq[r] == cur, k1 = sq[r + 1] == cur, k2 = sq[r + 2] == cur;
-            if (k0 && k1 && k2) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
-            else blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active, k0, k1, k2);
+            if (k0 && k1 && k2) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+            else blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active, k0, k1, k2);
         }
     } else if (rows == R) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (r < rows) blc_row<DT, W, MASK, NT>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+            if (r < rows) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
     }
 
     if (a.fin && active && t0 + rows == (int64_t)a.L) {
@@ -943,7 +994,7 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 #pragma unroll
             for (int e = 0; e < E; ++e) v[e] = 0.0f;
             if (t >= 0) {
-                unpack_vec<DT>(load_vec<false>(xb + t * xs), v);
+                V::template unpack<DT>(V::template load<false>(xb + t * xs), v);
                 if constexpr (MASK) {
                     const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
 #pragma unroll
@@ -971,7 +1022,7 @@ __global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
 template <int DT, int W, int R, bool MASK>
 __global__ __launch_bounds__(256) void canon_fwd_blc_seq_kernel(const FwdArgs a)
 {
-    blc_block<DT, W, R, MASK, false, true>(a, blockIdx.x);
+    blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
 // Several channel ranges of one logical [B, C, L] problem that live in separate
@@ -2306,8 +2357,10 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const bool bcl_ok = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
                         a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0 &&
                         a.L / E >= 16;
-    const bool blc_ok = fused && ptr_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 &&
-                        a.x_sb % E == 0 && a.x_sl % E == 0 && a.o_sb % E == 0 && a.o_sl % E == 0 &&
+    const uint32_t EB = kBlcVecBytes / elem_bytes(p->x_dtype);   // channels per lane of the channel-contiguous kernel
+    const bool ptr8_ok = (((uintptr_t)p->x | (uintptr_t)p->out) & (kBlcVecBytes - 1)) == 0;
+    const bool blc_ok = fused && ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
+                        a.x_sb % EB == 0 && a.x_sl % EB == 0 && a.o_sb % EB == 0 && a.o_sl % EB == 0 &&
                         a.x_sl != 1;
 
     if (bcl_ok) {
@@ -2331,7 +2384,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
         }
     }
     if (blc_ok) {
-        const uint32_t nvec = a.C / E;
+        const uint32_t nvec = a.C / EB;
         const uint32_t nct = (nvec + 63) / 64;                                   // channel tiles per row
         const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
         const uint64_t nblocks = (uint64_t)a.B * ntt * nct;

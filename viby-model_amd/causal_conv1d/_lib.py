@@ -114,7 +114,7 @@ def lib() -> ctypes.CDLL:
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError(
-                f"{LIB_PATH} not found: build it with `make -C viby-model_amd/csrc` "
+                f"{LIB_PATH} not found: build it with `make -j4 -C viby-model_amd/csrc` "
                 "(hipcc, --offload-arch=gfx950). There is no fallback implementation.")
         L = ctypes.CDLL(LIB_PATH)
         L.canon_conv1d_abi_version.restype = ctypes.c_int

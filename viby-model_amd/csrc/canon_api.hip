@@ -1,0 +1,653 @@
+// libcanon_conv1d.so, host side: argument validation, choice of kernel family
+// and launch geometry (the plan), and the extern "C" entry points declared in
+// include/canon_conv1d.h.  No device code in this file.
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "canon_plan.h"
+
+using namespace canon;
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// host side: validation, planning, launch
+// ---------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool valid_dtype(int d) { return d == CANON_DTYPE_F32 || d == CANON_DTYPE_BF16 || d == CANON_DTYPE_F16; }
+bool valid_mask_dtype(int d) { return d >= CANON_MASK_U8 && d <= CANON_MASK_F16; }
+int elem_bytes(int d) { return d == CANON_DTYPE_F32 ? 4 : 2; }
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+FastDiv make_fastdiv(uint32_t d)
+{
+    // floor(n / d) for 0 <= n < 2^32 (Granlund-Montgomery round-up method)
+    FastDiv f;
+    f.d = d ? d : 1;
+    uint32_t l = 0;
+    while ((1ull << l) < f.d) ++l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << l) - f.d)) / f.d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 0 ? l - 1 : 0;
+    return f;
+}
+
+// a run of E consecutive mask entries (E = elements of x per 16 bytes) starting
+// at a multiple of E is contiguous and aligned to its own size
+bool mask_run_aligned(const void *mask, int mask_dtype, int64_t stride_b, int64_t stride_l, int x_dtype)
+{
+    if (!mask || stride_l != 1) return false;
+    static const int msize[] = {1, 4, 8, 4, 2, 2};
+    const int E = 16 / elem_bytes(x_dtype);
+    const int64_t run = (int64_t)E * msize[mask_dtype];
+    const int64_t align = run < 16 ? run : 16;
+    return ((uintptr_t)mask % align) == 0 && (stride_b * msize[mask_dtype]) % align == 0;
+}
+
+int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_fwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_fwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_fwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->round_mode != CANON_ROUND_FUSED && p->round_mode != CANON_ROUND_EAGER)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
+    if (p->batch < 0 || p->channels < 0 || p->seqlen < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld, seqlen %lld)",
+                    (long long)p->batch, (long long)p->channels, (long long)p->seqlen);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->seqlen >= (1ll << 31) ||
+        p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
+    if (!empty) {
+        if (!p->x || !p->out || !p->weight) return fail(CANON_ERR_INVALID_ARGUMENT, "x, out and weight must not be NULL");
+        if (p->x == p->out) return fail(CANON_ERR_INVALID_ARGUMENT, "out must not alias x");
+    }
+    if (p->mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    if (p->initial_state && p->initial_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "initial_len %d is shorter than width-1 = %d", p->initial_len, p->width - 1);
+    if (p->final_state && p->final_len < 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "final_len %d must be at least 1", p->final_len);
+    if (p->final_state && p->final_len > 64)
+        return fail(CANON_ERR_UNSUPPORTED, "final_len %d above 64 is not supported", p->final_len);
+    if (p->seq_idx && (p->initial_state || p->final_state))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx excludes initial_state and final_state");
+    if (p->seq_idx && ((uintptr_t)p->seq_idx & 3u))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx must be 4-byte aligned");
+
+    FwdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.out = (char *)p->out;
+    a.weight = p->weight; a.bias = p->bias; a.mask = p->mask;
+    a.init = p->initial_state; a.fin = p->final_state;
+    a.seq = p->seq_idx; a.q_sb = p->seq_stride_b; a.q_sl = p->seq_stride_l;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.x_sl = p->x_stride_l;
+    a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c; a.o_sl = p->out_stride_l;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
+    a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
+    a.i_sb = p->init_stride_b; a.i_sc = p->init_stride_c; a.i_ss = p->init_stride_s;
+    a.f_sb = p->final_stride_b; a.f_sc = p->final_stride_c; a.f_ss = p->final_stride_s;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
+    a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
+    a.S_in = p->initial_state ? p->initial_len : 0;
+    a.S_out = p->final_state ? p->final_len : 0;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
+    a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
+    a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
+    plan->U = 1;
+    plan->grid = 0;
+    plan->kind = FWD_GENERIC;
+    if (empty) return CANON_OK;
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const uint64_t rows = (uint64_t)a.B * a.C;
+    a.nt = 2 * rows * a.L * elem_bytes(p->x_dtype) >= kStreamBytes;
+    const bool fused = p->round_mode == CANON_ROUND_FUSED;
+    const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
+    // packed sequences: the channel-contiguous kernel has a variant (the index is uniform per time row);
+    // time-contiguous rows take the strided kernel
+    const bool bcl_ok = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
+                        a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0 &&
+                        a.L / E >= 16;
+    const uint32_t EB = kBlcVecBytes / elem_bytes(p->x_dtype);   // channels per lane of the channel-contiguous kernel
+    const bool ptr8_ok = (((uintptr_t)p->x | (uintptr_t)p->out) & (kBlcVecBytes - 1)) == 0;
+    const bool blc_ok = fused && ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
+                        a.x_sb % EB == 0 && a.x_sl % EB == 0 && a.o_sb % EB == 0 && a.o_sl % EB == 0 &&
+                        a.x_sl != 1;
+
+    if (bcl_ok) {
+        const uint32_t nvec = a.L / E;
+        // vectors per lane: as many as keep >= 2048 waves in flight, at most 4
+        int U = 1;
+        for (int cand = 2; cand <= 4; cand *= 2) {
+            const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
+            if (nvec >= 64u * cand && rows * nseg >= 2048) U = cand;
+        }
+        const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
+        const uint64_t ntasks = rows * nseg;
+        if (ntasks < (1ull << 31)) {
+            plan->kind = FWD_BCL;
+            plan->U = U;
+            a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
+            a.div_nseg = make_fastdiv(a.nseg); a.div_C = make_fastdiv(a.C);
+            a.nblocks = (uint32_t)((ntasks + 3) / 4);
+            plan->grid = a.nblocks;
+            return CANON_OK;
+        }
+    }
+    if (blc_ok) {
+        const uint32_t nvec = a.C / EB;
+        const uint32_t nct = (nvec + 63) / 64;                                   // channel tiles per row
+        const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
+        const uint64_t nblocks = (uint64_t)a.B * ntt * nct;
+        if (nblocks < (1ull << 31) - 8) {
+            plan->kind = FWD_BLC;
+            a.nvec = nvec; a.nct = nct; a.ntt = ntt; a.ntasks = (uint32_t)nblocks;
+            a.div_nct = make_fastdiv(nct); a.div_ntt = make_fastdiv(ntt);
+            a.nblocks = (uint32_t)nblocks;
+            plan->grid = a.nblocks;
+            return CANON_OK;
+        }
+    }
+    {
+        const uint32_t nseg = (a.L + kGenericChunk - 1) / kGenericChunk;
+        const uint64_t nthreads = rows * nseg;
+        if (nthreads >= (1ull << 32))
+            return fail(CANON_ERR_UNSUPPORTED, "problem too large for the strided kernel (%llu threads)",
+                        (unsigned long long)nthreads);
+        plan->kind = FWD_GENERIC;
+        a.nseg = nseg; a.chunk = kGenericChunk; a.ntasks = (uint32_t)nthreads;
+        a.nblocks = (uint32_t)((nthreads + 255) / 256);
+        plan->grid = a.nblocks;
+    }
+    return CANON_OK;
+}
+
+int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_update_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_update_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_update_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->round_mode != CANON_ROUND_FUSED && p->round_mode != CANON_ROUND_EAGER)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
+    if (p->cache_seqlens) return fail(CANON_ERR_UNSUPPORTED, "cache_seqlens (circular conv_state) is not supported");
+    if (p->conv_state_indices) return fail(CANON_ERR_UNSUPPORTED, "conv_state_indices is not supported");
+    if (p->batch < 0 || p->channels < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld)", (long long)p->batch, (long long)p->channels);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels must be below 2^31");
+    if (p->state_len < 1 || p->state_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_len %d is shorter than width-1 = %d", p->state_len, p->width - 1);
+    const bool empty = p->batch == 0 || p->channels == 0;
+    if (!empty && (!p->x || !p->out || !p->conv_state || !p->weight))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "x, out, conv_state and weight must not be NULL");
+    if (p->token_mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+
+    UpdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.out = (char *)p->out; a.state = (char *)p->conv_state;
+    a.weight = p->weight; a.bias = p->bias; a.tmask = p->token_mask;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c;
+    a.s_sb = p->state_stride_b; a.s_sc = p->state_stride_c; a.s_ss = p->state_stride_s;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k; a.m_sb = p->mask_stride_b;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels;
+    a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
+    plan->kind = UPD_GENERIC;
+    plan->grid = 0;
+    if (empty) return CANON_OK;
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    const int S = p->state_len;
+    const bool vec_ok = p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
+                        aligned16(p->x) && aligned16(p->out) && aligned16(p->conv_state) &&
+                        a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb % E == 0 && a.o_sb % E == 0 &&
+                        a.s_ss == 1 && a.s_sc == S && a.s_sb % E == 0;
+    if (vec_ok) {
+        plan->kind = UPD_VEC;
+        a.nvec = a.C / E;
+        // two batch rows per lane halve the tap loads; with little work, more waves matter more
+        a.nb = ((uint64_t)a.nvec * a.B / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        a.bgroups = (a.B + a.nb - 1) / a.nb;
+        a.nthreads = a.nvec * a.bgroups;
+        a.div_nvec = make_fastdiv(a.nvec);
+        plan->grid = (a.nthreads + 255) / 256;
+    } else {
+        a.nthreads = a.B * a.C;
+        plan->grid = (a.nthreads + 255) / 256;
+    }
+    return CANON_OK;
+}
+
+// ---------------------------------------------------------------------------
+// channel ranges in separate tensors: one derived problem per part
+// ---------------------------------------------------------------------------
+const void *advance(const void *p, int64_t elems, int bytes)
+{
+    return p ? (const void *)((const char *)p + elems * bytes) : nullptr;
+}
+
+int check_parts(const canon_conv1d_part *parts, int32_t nparts, int64_t channels)
+{
+    if (!parts) return fail(CANON_ERR_INVALID_ARGUMENT, "parts is NULL");
+    if (nparts < 1 || nparts > kMaxParts)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "nparts %d outside 1..%d", nparts, kMaxParts);
+    int64_t sum = 0;
+    for (int i = 0; i < nparts; ++i) {
+        if (parts[i].channels < 0 || parts[i].channels >= (1ll << 31))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "part %d has %lld channels", i, (long long)parts[i].channels);
+        sum += parts[i].channels;
+    }
+    if (sum != channels)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "the parts hold %lld channels, params.channels is %lld", (long long)sum,
+                    (long long)channels);
+    return CANON_OK;
+}
+
+int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts, FwdPartsPlan *pp)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_fwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_fwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_fwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    int rc = check_parts(parts, nparts, p->channels);
+    if (rc != CANON_OK) return rc;
+    if (p->batch > 0 && p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    const int xb = elem_bytes(p->x_dtype), wb = elem_bytes(p->w_dtype);
+    pp->n = nparts;
+    int64_t c0 = 0;
+    uint64_t blocks = 0;
+    bool all_blc = true;
+    for (int i = 0; i < nparts; ++i) {
+        canon_conv1d_fwd_params q = *p;
+        q.channels = parts[i].channels;
+        q.x = parts[i].x; q.x_stride_b = parts[i].x_stride_b; q.x_stride_c = parts[i].x_stride_c; q.x_stride_l = parts[i].x_stride_l;
+        q.out = parts[i].out; q.out_stride_b = parts[i].out_stride_b; q.out_stride_c = parts[i].out_stride_c;
+        q.out_stride_l = parts[i].out_stride_l;
+        q.weight = advance(p->weight, c0 * p->w_stride_c, wb);
+        q.bias = advance(p->bias, c0, wb);
+        q.initial_state = advance(p->initial_state, c0 * p->init_stride_c, xb);
+        q.final_state = (void *)advance(p->final_state, c0 * p->final_stride_c, xb);
+        rc = plan_fwd(&q, &pp->part[i]);
+        if (rc != CANON_OK) return rc;
+        if (pp->part[i].grid > 0) {
+            all_blc = all_blc && pp->part[i].kind == FWD_BLC;
+            blocks += pp->part[i].grid;
+        }
+        c0 += parts[i].channels;
+    }
+    // whether to stream past the caches is decided on the whole problem
+    const bool nt = 2ull * (uint64_t)p->batch * (uint64_t)p->channels * (uint64_t)p->seqlen * xb >= kStreamBytes;
+    for (int i = 0; i < nparts; ++i) pp->part[i].args.nt = nt;
+    pp->single = nparts > 1 && all_blc && p->width == 4 && !p->seq_idx && blocks > 0 && blocks < (1ull << 31);
+    pp->grid = (uint32_t)blocks;
+    return CANON_OK;
+}
+
+int plan_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts, UpdPartsPlan *pp)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_update_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_update_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_update_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    int rc = check_parts(parts, nparts, p->channels);
+    if (rc != CANON_OK) return rc;
+    if (p->batch > 0 && p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels must be below 2^31");
+    const int xb = elem_bytes(p->x_dtype), wb = elem_bytes(p->w_dtype);
+    pp->n = nparts;
+    int64_t c0 = 0;
+    bool all_vec = true;
+    uint64_t nvec_total = 0;
+    for (int i = 0; i < nparts; ++i) {
+        canon_conv1d_update_params q = *p;
+        q.channels = parts[i].channels;
+        q.x = parts[i].x; q.x_stride_b = parts[i].x_stride_b; q.x_stride_c = parts[i].x_stride_c;
+        q.out = parts[i].out; q.out_stride_b = parts[i].out_stride_b; q.out_stride_c = parts[i].out_stride_c;
+        q.conv_state = (void *)advance(p->conv_state, c0 * p->state_stride_c, xb);
+        q.weight = advance(p->weight, c0 * p->w_stride_c, wb);
+        q.bias = advance(p->bias, c0, wb);
+        rc = plan_update(&q, &pp->part[i]);
+        if (rc != CANON_OK) return rc;
+        if (pp->part[i].grid > 0) {
+            all_vec = all_vec && pp->part[i].kind == UPD_VEC;
+            nvec_total += pp->part[i].args.nvec;
+        }
+        c0 += parts[i].channels;
+    }
+    pp->single = nparts > 1 && all_vec && p->width == 4 && nvec_total > 0;
+    pp->grid = 0;
+    if (pp->single) {
+        // batch rows per lane chosen on the whole token, the same for every part
+        const uint32_t nb = (nvec_total * (uint64_t)p->batch / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        uint64_t blocks = 0;
+        for (int i = 0; i < nparts; ++i) {
+            UpdPlan &u = pp->part[i];
+            if (u.grid == 0) continue;
+            u.args.nb = nb;
+            u.args.bgroups = (u.args.B + nb - 1) / nb;
+            u.args.nthreads = u.args.nvec * u.args.bgroups;
+            u.grid = (u.args.nthreads + 255) / 256;
+            blocks += u.grid;
+        }
+        pp->grid = (uint32_t)blocks;
+    }
+    return CANON_OK;
+}
+
+// ---------------------------------------------------------------------------
+// backward: planning and launch
+// ---------------------------------------------------------------------------
+int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointers)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_bwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_bwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_bwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->batch < 0 || p->channels < 0 || p->seqlen < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld, seqlen %lld)",
+                    (long long)p->batch, (long long)p->channels, (long long)p->seqlen);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->seqlen >= (1ll << 31) ||
+        p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
+    if (p->mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
+    if (check_pointers) {
+        if (p->channels > 0 && (!p->weight || !p->dweight))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "weight and dweight must not be NULL");
+        if (!empty && (!p->x || !p->dout || !p->dx))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "x, dout and dx must not be NULL");
+        if (!empty && (p->dx == p->x || p->dx == p->dout))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "dx must not alias x or dout");
+    }
+
+    BwdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.dy = (const char *)p->dout; a.dx = (char *)p->dx;
+    a.weight = p->weight; a.bias = p->bias; a.mask = p->mask;
+    a.partial = (float *)p->workspace; a.dweight = p->dweight; a.dbias = p->dbias;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.x_sl = p->x_stride_l;
+    a.g_sb = p->dout_stride_b; a.g_sc = p->dout_stride_c; a.g_sl = p->dout_stride_l;
+    a.d_sb = p->dx_stride_b; a.d_sc = p->dx_stride_c; a.d_sl = p->dx_stride_l;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
+    a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
+    a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode;
+    a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
+    a.b_vec = p->bias && aligned16(p->bias);
+    plan->kind = BWD_GENERIC;
+    plan->U = 1;
+    plan->grid = 0;
+    plan->workspace_bytes = 0;
+    if (empty) return CANON_OK;   // the caller's dweight/dbias are zero filled by canon_conv1d_bwd
+
+    const int E = 16 / elem_bytes(p->x_dtype);
+    a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
+    a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
+    const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
+    const bool rows = ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
+                      a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
+                      a.d_sb % E == 0 && a.d_sc % E == 0;
+    if (rows) {
+        const uint32_t nvec = a.L / E;
+        const uint64_t nrows = (uint64_t)a.B * a.C;
+        int U = 1;
+        for (int cand = 2; cand <= 4; cand *= 2) {
+            const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
+            if (nvec >= 64u * cand && nrows * nseg >= 2048) U = cand;
+        }
+        const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
+        const uint64_t ntasks = nrows * nseg;
+        if (ntasks < (1ull << 31)) {
+            plan->kind = BWD_BCL_VEC;
+            plan->U = U;
+            // field use in this kernel family: nthreads = wave tasks, nchunk = segments per row
+            a.nvec = nvec; a.nchunk = (uint32_t)nseg; a.nthreads = (uint32_t)ntasks;
+            a.nsets = a.B * a.nchunk;
+            a.div_nchunk = make_fastdiv(a.nchunk); a.div_nvec = make_fastdiv(a.C);
+            plan->grid = (uint32_t)((ntasks + 3) / 4);
+            plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+            if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
+                return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                            (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+            return CANON_OK;
+        }
+    }
+    // channel-contiguous tensors: 8-byte groups of channels per lane
+    const int E8 = 8 / elem_bytes(p->x_dtype);
+    const bool ptrs8 = !check_pointers || ((((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0);
+    const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
+                     a.x_sb % E8 == 0 && a.x_sl % E8 == 0 && a.g_sb % E8 == 0 && a.g_sl % E8 == 0 &&
+                     a.d_sb % E8 == 0 && a.d_sl % E8 == 0 && ptrs8;
+    if (vec) {
+        const uint32_t tile = kBwdSlab * kBwdWaves;
+        const uint32_t nvec = a.C / E8;
+        const uint32_t nct = (nvec + 63) / 64;
+        // time steps per block: as long as possible (few partial sets to write and to add up, taps and
+        // chunk-end work amortised) while the grid still has one and a half blocks per CU
+        uint32_t chunk = tile;
+        for (uint32_t cand = 2 * tile; cand <= 32 * tile; cand *= 2) {
+            const uint64_t blocks = (uint64_t)a.B * ((a.L + cand - 1) / cand) * nct;
+            if (2 * blocks >= 256ull * kBwdHalfBlocksPerCU) chunk = cand;
+        }
+        const uint32_t nchunk = (a.L + chunk - 1) / chunk;
+        const uint64_t blocks = (uint64_t)a.B * nchunk * nct;
+        if (blocks < (1ull << 31)) {
+            plan->kind = BWD_BLC_VEC;
+            a.nvec = nvec; a.nct = nct; a.chunk = chunk; a.nchunk = nchunk;
+            a.nsets = a.B * nchunk;
+            a.div_nct = make_fastdiv(nct); a.div_nchunk = make_fastdiv(nchunk);
+            plan->grid = (uint32_t)blocks;
+            plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+            if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
+                return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                            (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+            return CANON_OK;
+        }
+    }
+    plan->kind = BWD_GENERIC;
+    a.nvec = a.C;
+    // time steps per lane: about 8 waves per CU, a multiple of the look-ahead, and few enough
+    // partial sets that the scratch stays below ~16 MB
+    const uint64_t lanes_per_step = (uint64_t)a.B * a.nvec;
+    uint64_t want_chunks = (256ull * 8 * 64 + lanes_per_step - 1) / lanes_per_step;
+    const uint64_t max_sets = (16ull << 20) / ((uint64_t)a.C * 20) + 1;
+    if ((uint64_t)a.B * want_chunks > max_sets) want_chunks = max_sets / a.B;
+    if (want_chunks < 1) want_chunks = 1;
+    uint32_t chunk = (uint32_t)((a.L + want_chunks - 1) / want_chunks);
+    chunk = ((chunk + kBwdRows - 1) / kBwdRows) * kBwdRows;
+    if (chunk < 4 * kBwdRows) chunk = 4 * kBwdRows;
+    a.chunk = chunk;
+    a.nchunk = (a.L + chunk - 1) / chunk;
+    const uint64_t nthreads = lanes_per_step * a.nchunk;
+    if (nthreads >= (1ull << 32)) return fail(CANON_ERR_UNSUPPORTED, "problem too large for the backward kernel");
+    a.nthreads = (uint32_t)nthreads;
+    a.nsets = a.B * a.nchunk;
+    a.div_nvec = make_fastdiv(a.nvec);
+    a.div_nchunk = make_fastdiv(a.nchunk);
+    plan->grid = (uint32_t)((nthreads + 255) / 256);
+    plan->workspace_bytes = (int64_t)a.nsets * a.C * 5 * (int64_t)sizeof(float);
+    if (check_pointers) {
+        if (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes)
+            return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                        (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+    }
+    return CANON_OK;
+}
+
+int check_launch(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return CANON_OK;
+}
+
+}  // namespace
+
+#define CANON_API __attribute__((visibility("default")))
+
+extern "C" {
+
+CANON_API int canon_conv1d_abi_version(void) { return CANON_CONV1D_ABI_VERSION; }
+
+CANON_API const char *canon_conv1d_last_error(void) { return g_err; }
+
+CANON_API int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream)
+{
+    FwdPlan pl;
+    const int rc = plan_fwd(p, &pl);
+    if (rc != CANON_OK) return rc;
+    if (pl.grid == 0) return CANON_OK;
+    hipStream_t s = (hipStream_t)stream;
+    launch_fwd(pl, p->x_dtype, s);
+    return check_launch("canon_conv1d_fwd");
+}
+
+CANON_API int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream)
+{
+    UpdPlan pl;
+    const int rc = plan_update(p, &pl);
+    if (rc != CANON_OK) return rc;
+    if (pl.grid == 0) return CANON_OK;
+    hipStream_t s = (hipStream_t)stream;
+    launch_update(pl, p->x_dtype, s);
+    return check_launch("canon_conv1d_update");
+}
+
+CANON_API int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream)
+{
+    BwdPlan pl;
+    const int rc = plan_bwd(p, &pl, true);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (pl.grid == 0) {
+        // nothing to sum: the gradients of the parameters are zero
+        // (a fill kernel rather than a memset, so that the call can be captured into a HIP graph)
+        if (p->channels > 0) {
+            launch_zero(p->dweight, (uint32_t)(p->channels * p->width), s);
+            if (p->dbias) launch_zero(p->dbias, (uint32_t)p->channels, s);
+            return check_launch("canon_conv1d_bwd");
+        }
+        return CANON_OK;
+    }
+    launch_bwd(pl, p->x_dtype, s);
+    return check_launch("canon_conv1d_bwd");
+}
+
+CANON_API int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p)
+{
+    BwdPlan pl;
+    if (plan_bwd(p, &pl, false) != CANON_OK) return -1;
+    return pl.workspace_bytes;
+}
+
+CANON_API const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p)
+{
+    BwdPlan pl;
+    if (plan_bwd(p, &pl, false) != CANON_OK) return nullptr;
+    return pl.kind == BWD_BLC_VEC ? "bwd_blc_vec" : pl.kind == BWD_BCL_VEC ? "bwd_bcl_vec" : "bwd_generic";
+}
+
+CANON_API const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)
+{
+    FwdPlan pl;
+    if (plan_fwd(p, &pl) != CANON_OK) return nullptr;
+    if (pl.kind == FWD_BLC && pl.args.seq) return "blc_vec_seq";
+    return pl.kind == FWD_BCL ? "bcl_vec" : pl.kind == FWD_BLC ? "blc_vec" : "generic";
+}
+
+CANON_API const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p)
+{
+    UpdPlan pl;
+    if (plan_update(p, &pl) != CANON_OK) return nullptr;
+    return pl.kind == UPD_VEC ? "update_vec" : "update_generic";
+}
+
+CANON_API int canon_conv1d_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts, void *stream)
+{
+    FwdPartsPlan pp;
+    const int rc = plan_fwd_parts(p, parts, nparts, &pp);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    launch_fwd_parts(pp, p->x_dtype, s);
+    return check_launch("canon_conv1d_fwd_parts");
+}
+
+CANON_API int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts,
+                              void *stream)
+{
+    UpdPartsPlan pp;
+    const int rc = plan_update_parts(p, parts, nparts, &pp);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    launch_update_parts(pp, p->x_dtype, s);
+    return check_launch("canon_conv1d_update_parts");
+}
+
+CANON_API const char *canon_conv1d_fwd_parts_plan(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts)
+{
+    FwdPartsPlan pp;
+    if (plan_fwd_parts(p, parts, nparts, &pp) != CANON_OK) return nullptr;
+    return pp.single ? "blc_vec_parts" : "per_part";
+}
+
+CANON_API const char *canon_conv1d_update_parts_plan(const canon_conv1d_update_params *p, const canon_conv1d_part *parts,
+                                           int32_t nparts)
+{
+    UpdPartsPlan pp;
+    if (plan_update_parts(p, parts, nparts, &pp) != CANON_OK) return nullptr;
+    return pp.single ? "update_vec_parts" : "per_part";
+}
+
+}  // extern "C"

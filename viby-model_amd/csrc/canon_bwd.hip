@@ -1,0 +1,909 @@
+// Canon causal depthwise conv1d for MI355X (gfx950): backward of the prefill
+// (dx, and dweight / dbias through partial sets and a fixed-order reduction).
+#include "canon_device.h"
+
+namespace canon {
+
+// ---------------------------------------------------------------------------
+// backward of the prefill: dx, and per-chunk partial sums of dweight / dbias
+//
+// One lane owns E channels and walks a chunk of time steps from its END to its
+// start: dx[t] needs dz[t .. t+W-1] (the three later steps are carried in
+// registers), z[t] needs xm[t-3 .. t] (a sliding window refilled with one row
+// per step, fetched R rows ahead).  The three dz values just past the chunk are
+// recomputed from memory.  dweight / dbias accumulate in registers over the
+// chunk and go to partial[(b * nchunk + chunk) * C + c][5] (w0..w3, bias);
+// canon_bwd_reduce_kernel sums the partial sets in a fixed order.
+//   VEC:  channel-contiguous tensors, E = elements per 16 bytes, vector access
+//   !VEC: E = 1, any strides (the fallback for every other layout)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float silu_grad(float z)
+{
+    const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+    return s * (1.0f + z * (1.0f - s));
+}
+
+template <int DT, int E, bool VEC>
+__device__ __forceinline__ void bwd_load_row(const char *base, int64_t row_off, int64_t sc, float *f)
+{
+    // E values of one time step; VEC: 16 contiguous bytes at base + row_off (bytes)
+    if constexpr (VEC) {
+        unpack_vec<DT>(load_vec<false>(base + row_off), f);
+    } else {
+        f[0] = load1<DT>(base + row_off, 0);
+    }
+}
+
+template <int DT, int W, int E, bool VEC, bool MASK, int R>
+__global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
+{
+    constexpr int BY = Elem<DT>::bytes;
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.nthreads) return;
+    const uint32_t bc = fdiv(tid, a.div_nvec);
+    const uint32_t cv = tid - bc * a.nvec;
+    const uint32_t b = fdiv(bc, a.div_nchunk);
+    const uint32_t ch = bc - b * a.nchunk;
+    const uint32_t c0 = cv * E;
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + (int64_t)c0 * a.x_sc) * BY;
+    const char *gb = a.dy + ((int64_t)b * a.g_sb + (int64_t)c0 * a.g_sc) * BY;
+    char *db_ = a.dx + ((int64_t)b * a.d_sb + (int64_t)c0 * a.d_sc) * BY;
+    const int64_t xs = a.x_sl * BY, gs = a.g_sl * BY, ds = a.d_sl * BY;
+    const int64_t t_begin = (int64_t)ch * a.chunk;
+    const int64_t t_stop = t_begin + (int64_t)a.chunk;
+    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+    const int64_t Lm1 = (int64_t)a.L - 1;
+
+    RawTaps<E> raw;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, VEC && a.w_vec != 0, VEC && a.b_vec != 0, c0, raw);
+
+    // rows t_end-4 .. t_end+2 of xm (window for the last step + the three steps past the chunk)
+    float xr7[7][E], m7[7];
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+        const int64_t t = t_end - 4 + j;
+        const int64_t tc = t < 0 ? 0 : (t > Lm1 ? Lm1 : t);
+        bwd_load_row<DT, E, VEC>(xb, tc * xs, a.x_sc, xr7[j]);
+        m7[j] = 1.0f;
+    }
+    float g3[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int64_t t = t_end + j;
+        bwd_load_row<DT, E, VEC>(gb, (t > Lm1 ? Lm1 : t) * gs, a.g_sc, g3[j]);
+    }
+    if constexpr (MASK) load_mask_rows<7>(a.mask, (int64_t)b * a.m_sb, t_end - 4, a.L, a.m_sl, a.mask_dtype, m7);
+
+    float w[E][W], bias[E];
+    decode_taps<DT, W, E>(raw, a.w_dtype, VEC && a.w_vec != 0, a.bias != nullptr, w, bias);
+
+#pragma unroll
+    for (int j = 0; j < 7; ++j) {
+        const int64_t t = t_end - 4 + j;
+        const bool inside = t >= 0 && t <= Lm1;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float v = MASK ? mul_round<DT>(xr7[j][e], m7[j]) : xr7[j][e];
+            xr7[j][e] = inside ? v : 0.0f;
+        }
+    }
+    // dzf[j] = dz[t_end + j]
+    float dzf[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const bool inside = t_end + j <= Lm1;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float z = bias[e];
+#pragma unroll
+            for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xr7[j + 1 + (4 - W) + k][e], z);   // xm[t_end+j-(W-1)+k]
+            const float d = a.act ? g3[j][e] * silu_grad(z) : g3[j][e];
+            dzf[j][e] = inside ? d : 0.0f;
+        }
+    }
+    // xw[k] = xm[t-3+k] for the step being processed, starting with t = t_end - 1
+    float xw[4][E];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) xw[k][e] = xr7[k][e];
+
+    float dw[E][W], dbs[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        dbs[e] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) dw[e][k] = 0.0f;
+    }
+
+    for (int64_t t_hi = t_end - 1; t_hi >= t_begin; t_hi -= R) {
+        // this batch: steps t_hi, t_hi-1, .., t_hi-R+1; needs dout of those steps and x rows t-4.
+        // Rows are kept as loaded (raw) until their step, to keep the register count down.
+        typename std::conditional<VEC, uint4, float>::type G[R], XN[R];
+        float mk[R], mn[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t_hi - r;
+            const int64_t tg = t < 0 ? 0 : t;
+            const int64_t tn = t - 4 < 0 ? 0 : t - 4;
+            if constexpr (VEC) {
+                G[r] = load_vec<false>(gb + tg * gs);
+                XN[r] = load_vec<false>(xb + tn * xs);
+            } else {
+                G[r] = load1<DT>(gb + tg * gs, 0);
+                XN[r] = load1<DT>(xb + tn * xs, 0);
+            }
+            mk[r] = 1.0f;
+            mn[r] = 1.0f;
+        }
+        if constexpr (MASK) {
+            // masks of steps t_hi-R+1 .. t_hi (for dx) and of rows t_hi-R-3 .. t_hi-4 (for the window)
+            float mm[R + 4];
+            load_mask_rows<R + 4>(a.mask, (int64_t)b * a.m_sb, t_hi - R - 3, a.L, a.m_sl, a.mask_dtype, mm);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                mk[r] = mm[R + 3 - r];      // step t_hi - r
+                mn[r] = mm[R - 1 - r];      // row  t_hi - r - 4
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t_hi - r;
+            if (t < t_begin) break;
+            float g[E], xn[E], dz[E], o[E];
+            if constexpr (VEC) {
+                unpack_vec<DT>(G[r], g);
+                unpack_vec<DT>(XN[r], xn);
+            } else {
+                g[0] = G[r];
+                xn[0] = XN[r];
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float z = bias[e];
+#pragma unroll
+                for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xw[(4 - W) + k][e], z);
+                dz[e] = z;
+            }
+            if (a.act) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = g[e] * silu_grad(dz[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = g[e];
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                // dxm[t] = sum_k w[k] * dz[t + (W-1) - k]
+                float acc = w[e][W - 1] * dz[e];
+                acc = fmaf(w[e][W - 2], dzf[0][e], acc);
+                if constexpr (W >= 3) acc = fmaf(w[e][W - 3], dzf[1][e], acc);
+                if constexpr (W == 4) acc = fmaf(w[e][0], dzf[2][e], acc);
+                o[e] = acc;
+#pragma unroll
+                for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xw[(4 - W) + k][e], dw[e][k]);
+                dbs[e] += dz[e];
+                dzf[2][e] = dzf[1][e];
+                dzf[1][e] = dzf[0][e];
+                dzf[0][e] = dz[e];
+            }
+            if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] += g[e];
+            }
+            if constexpr (MASK) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] *= mk[r];
+            }
+            if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) o[e] += g[e];
+            }
+            // slide the window one step back: the new oldest row is t - 4
+            const bool has_row = t - 4 >= 0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float v = xn[e];
+                if constexpr (MASK) v = mul_round<DT>(v, mn[r]);
+                xw[3][e] = xw[2][e];
+                xw[2][e] = xw[1][e];
+                xw[1][e] = xw[0][e];
+                xw[0][e] = has_row ? v : 0.0f;
+            }
+            if constexpr (VEC) {
+                store_vec<false>(db_ + t * ds, pack_vec<DT>(o));
+            } else {
+                store1<DT>(db_ + t * ds, 0, o[0]);
+            }
+        }
+    }
+
+    float *pp = a.partial + (((int64_t)b * a.nchunk + ch) * a.C + c0) * 5;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) pp[e * 5 + k] = k < W ? dw[e][k] : 0.0f;
+        pp[e * 5 + 4] = dbs[e];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, channel-contiguous tensors ([B, L, C] viewed as [B, C, L]).
+//
+// A block is four waves; a lane owns the channels of one 8-byte group (4 x
+// 16-bit or 2 x fp32), a wave a slab of kBwdSlab consecutive time steps of a
+// 64-lane channel tile, the four waves four consecutive slabs, and the block
+// walks over the `chunk` time steps of its chunk one such 32-step tile at a
+// time, keeping its dweight / dbias sums in registers.
+//
+// Per tile, all rows of x and dout of the slab are requested before anything
+// is waited for.  The three rows of x before a slab come from the previous
+// wave's slab through LDS (the first wave reads them from memory).  dz of the
+// slab's first three steps is computed first and handed to the previous wave
+// through LDS (that wave's dx needs dz of the three steps after its slab; the
+// last wave recomputes them from three extra rows of x and dout).  The slab is
+// then swept from its last step to its first:
+//   dz[t] = dout[t] * act'(z[t]),  dx[t] = sum_k w[k] * dz[t + (W-1) - k]
+// At the end the four waves' sums are added in a fixed order through LDS and
+// written as one partial set entry per channel.
+// ---------------------------------------------------------------------------
+template <int DT> __device__ __forceinline__ void unpack_half(const uint2 &v, float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        f[0] = bits_f(v.x);
+        f[1] = bits_f(v.y);
+    } else {
+        unpack2<DT>(v.x, f[0], f[1]);
+        unpack2<DT>(v.y, f[2], f[3]);
+    }
+}
+
+template <int DT> __device__ __forceinline__ uint2 pack_half(const float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) return make_uint2(f_bits(f[0]), f_bits(f[1]));
+    else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
+}
+
+// One raw row -> the bits of xm = x * mask in the storage type (zero when the row does not exist)
+template <int DT, bool MASK>
+__device__ __forceinline__ uint2 bwd_mask_row(const uint2 &raw, float m, bool exists)
+{
+    uint2 v = raw;
+    if constexpr (MASK) {
+        if constexpr (DT == CANON_DTYPE_F32) {
+            v.x = f_bits(bits_f(raw.x) * m);
+            v.y = f_bits(bits_f(raw.y) * m);
+        } else {
+            float f[4];
+            unpack_half<DT>(raw, f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f[e] *= m;
+                if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(f[e]));   // see mul_round
+            }
+            v = pack_half<DT>(f);
+        }
+    }
+    if (!exists) v = make_uint2(0, 0);
+    return v;
+}
+
+// dz of one step from its window of xm rows and dout
+template <int W, int E, bool ACT>
+__device__ __forceinline__ void bwd_dz(const float (*w)[W], const float *bias, const float *x0, const float *x1,
+                                       const float *x2, const float *x3, const float *g, float *dz)
+{
+    if constexpr (ACT) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float z = bias[e];
+            if constexpr (W == 4) z = fmaf(w[e][0], x0[e], z);
+            if constexpr (W >= 3) z = fmaf(w[e][W - 3], x1[e], z);
+            z = fmaf(w[e][W - 2], x2[e], z);
+            z = fmaf(w[e][W - 1], x3[e], z);
+            dz[e] = g[e] * silu_grad(z);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) dz[e] = g[e];
+    }
+}
+
+// The sweep over one slab, last step first.  X / H hold xm in storage bits, dzh the dz of the
+// first three steps (already zero past the end of the sequence), dzf the dz of the three steps
+// after the slab.  FULL: all R steps exist.
+template <int DT, int W, bool MASK, bool ACT, bool FULL, int R, int E>
+__device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W], const float *bias, const uint2 *X,
+                                          const uint2 *H, const uint2 *G, const float *mm, const float (*dzh)[E],
+                                          float (*dzf)[E], float (*dw)[W], float *dbs, char *dxp, int64_t ds, int rows,
+                                          bool active)
+{
+    float xw[4][E];   // xm of rows r-3 .. r
+#pragma unroll
+    for (int k = 0; k < 4; ++k) unpack_half<DT>(X[R - 4 + k], xw[k]);
+#pragma unroll
+    for (int r = R - 1; r >= 0; --r) {
+        float g[E], dz[E], o[E];
+        unpack_half<DT>(G[r], g);
+        if (r >= 3) {
+            bwd_dz<W, E, ACT>(w, bias, xw[0], xw[1], xw[2], xw[3], g, dz);
+            if constexpr (!FULL) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dz[e] = r < rows ? dz[e] : 0.0f;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) dz[e] = dzh[r][e];
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float acc = w[e][W - 1] * dz[e];
+            acc = fmaf(w[e][W - 2], dzf[0][e], acc);
+            if constexpr (W >= 3) acc = fmaf(w[e][W - 3], dzf[1][e], acc);
+            if constexpr (W == 4) acc = fmaf(w[e][0], dzf[2][e], acc);
+            o[e] = acc;
+#pragma unroll
+            for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xw[(4 - W) + k][e], dw[e][k]);
+            dbs[e] += dz[e];
+            dzf[2][e] = dzf[1][e];
+            dzf[1][e] = dzf[0][e];
+            dzf[0][e] = dz[e];
+        }
+        if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += g[e];
+        }
+        if constexpr (MASK) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] *= mm[3 + r];
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += g[e];
+        }
+        if ((FULL || r < rows) && active) *(uint2 *)(dxp + r * ds) = pack_half<DT>(o);
+        if (r > 0) {
+            // slide the window one step back: the new oldest row is r - 4
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                xw[3][e] = xw[2][e];
+                xw[2][e] = xw[1][e];
+                xw[1][e] = xw[0][e];
+            }
+            unpack_half<DT>(r - 4 >= 0 ? X[r - 4 >= 0 ? r - 4 : 0] : H[r - 1 < 3 ? r - 1 : 0], xw[0]);
+        }
+    }
+}
+
+template <int DT, int W, bool MASK, bool ACT>
+__global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
+{
+    constexpr int BY = Elem<DT>::bytes;
+    constexpr int E = 8 / BY;
+    constexpr int R = kBwdSlab, NW = kBwdWaves;
+    __shared__ uint2 tailx[NW][3][64];            // last three xm rows of each wave's slab (storage bits)
+    __shared__ float headdz[NW][3][E][64];        // dz of the first three steps of each wave's slab
+    __shared__ float red[NW - 1][5 * E][64];      // dweight / dbias sums of waves 1..3
+
+    // blockIdx = (b * nchunk + ch) * nct + ct : channel tile fastest, i.e. memory order
+    const uint32_t bc = fdiv(blockIdx.x, a.div_nct);
+    const uint32_t ct = blockIdx.x - bc * a.nct;
+    const uint32_t b = fdiv(bc, a.div_nchunk);
+    const uint32_t ch = bc - b * a.nchunk;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t cv = ct * 64u + lane;
+    const bool active = cv < a.nvec;
+    const uint32_t c0 = (active ? cv : a.nvec - 1u) * E;   // idle lanes shadow the last group: loads need no predicate
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * BY;
+    const char *gb = a.dy + ((int64_t)b * a.g_sb + c0) * BY;
+    char *db_ = a.dx + ((int64_t)b * a.d_sb + c0) * BY;
+    const int64_t xs = a.x_sl * BY, gs = a.g_sl * BY, ds = a.d_sl * BY;
+    const int64_t Lm1 = (int64_t)a.L - 1;
+    const int64_t t_chunk = (int64_t)ch * a.chunk;
+    const int ntiles = (int)(a.chunk / (uint32_t)(R * NW));
+
+    RawTaps<E> rawt;
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, rawt);
+    float w[E][W], bias[E];
+
+    // The tiles are walked from the last to the first, so the dz of the three steps after a tile
+    // are the head of the tile done just before (still in headdz[0]).  For the chunk's last tile
+    // the last wave computes them here, from six rows of x and three of dout, and leaves them
+    // in that slot itself.
+    {
+        const int64_t te = t_chunk + (int64_t)a.chunk;   // first step after the chunk (at least 32)
+        uint2 XE[6], GE[3];
+        float me[6];
+#pragma unroll
+        for (int j = 0; j < 6; ++j) {
+            XE[j] = make_uint2(0, 0);
+            me[j] = 1.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) GE[j] = make_uint2(0, 0);
+        if (wv == NW - 1 && te <= Lm1) {
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                const int64_t t = te - 3 + j;
+                XE[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+            }
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = te + j;
+                GE[j] = *(const uint2 *)(gb + (t < Lm1 ? t : Lm1) * gs);
+            }
+            if constexpr (MASK) load_mask_rows<6>(a.mask, (int64_t)b * a.m_sb, te - 3, a.L, a.m_sl, a.mask_dtype, me);
+        }
+        decode_taps<DT, W, E>(rawt, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+        if (wv == NW - 1) {
+            float xt[6][E];
+#pragma unroll
+            for (int j = 0; j < 6; ++j) unpack_half<DT>(bwd_mask_row<DT, MASK>(XE[j], me[j], te - 3 + j <= Lm1), xt[j]);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float g[E], d[E];
+                unpack_half<DT>(GE[j], g);
+                bwd_dz<W, E, ACT>(w, bias, xt[j], xt[j + 1], xt[j + 2], xt[j + 3], g, d);
+                const bool inside = te + j <= Lm1;
+#pragma unroll
+                for (int e = 0; e < E; ++e) headdz[0][j][e][lane] = inside ? d[e] : 0.0f;
+            }
+        }
+    }
+
+    float dw[E][W], dbs[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        dbs[e] = 0.0f;
+#pragma unroll
+        for (int k = 0; k < W; ++k) dw[e][k] = 0.0f;
+    }
+
+    // rows of x and dout, the three rows of x before the slab (first wave) and the mask entries of one tile;
+    // requested one tile ahead, so that they arrive while the tile before is being computed
+    uint2 Xn[R], Gn[R], Hn[3];
+    float mmn[R + 3];   // mask of steps t0-3 .. t0+R-1
+    auto request = [&](int it) {
+        const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
+            Xn[r] = *(const uint2 *)(xb + t * xs);
+            Gn[r] = *(const uint2 *)(gb + t * gs);
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) Hn[j] = make_uint2(0, 0);
+        if (wv == 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = t0 - 3 + j;
+                if (t >= 0) Hn[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < R + 3; ++j) mmn[j] = 1.0f;
+        if constexpr (MASK) load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mmn);
+    };
+    request(ntiles - 1);
+
+    for (int it = ntiles - 1; it >= 0; --it) {
+        const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
+        const int64_t left = (int64_t)a.L - t0;
+        const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
+
+        uint2 X[R], G[R], H[3];
+        float mm[R + 3];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            X[r] = Xn[r];
+            G[r] = Gn[r];
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) H[j] = Hn[j];
+#pragma unroll
+        for (int j = 0; j < R + 3; ++j) mm[j] = mmn[j];
+        if (it > 0) request(it - 1);
+
+        // dz of the three steps after the slab; the last wave's are the previous iteration's head of wave 0
+        float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed
+        if (wv == NW - 1) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[0][j][e][lane];
+        }
+
+        // ---- rows become xm (masked, zero where they do not exist), once ----------------
+        if (MASK || rows < R) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) X[r] = bwd_mask_row<DT, MASK>(X[r], mm[3 + r], r < rows);
+        }
+        if constexpr (MASK) {
+            if (wv == 0) {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) H[j] = bwd_mask_row<DT, MASK>(H[j], mm[j], true);   // zero already when t < 0
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) tailx[wv][j][lane] = X[R - 3 + j];
+        __syncthreads();
+        if (wv > 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) H[j] = tailx[wv - 1][j][lane];
+        }
+
+        // ---- dz of the slab's first three steps, handed to the previous wave ---------
+        float dzh[3][E];
+        {
+            float xq[6][E];   // xm of rows -3 .. 2
+#pragma unroll
+            for (int k = 0; k < 3; ++k) unpack_half<DT>(H[k], xq[k]);
+#pragma unroll
+            for (int k = 0; k < 3; ++k) unpack_half<DT>(X[k], xq[3 + k]);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float g[E];
+                unpack_half<DT>(G[j], g);
+                bwd_dz<W, E, ACT>(w, bias, xq[j], xq[j + 1], xq[j + 2], xq[j + 3], g, dzh[j]);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    dzh[j][e] = j < rows ? dzh[j][e] : 0.0f;
+                    headdz[wv][j][e][lane] = dzh[j][e];
+                }
+            }
+        }
+        __syncthreads();
+        if (wv < NW - 1) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+#pragma unroll
+                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[wv + 1][j][e][lane];
+        }
+
+        // ---- sweep the slab from its last step to its first --------------------------
+        if (rows == R)
+            bwd_sweep<DT, W, MASK, ACT, true, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+        else
+            bwd_sweep<DT, W, MASK, ACT, false, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+    }
+
+    // ---- the four waves' sums, added in the order 0, 1, 2, 3 -----------------------------
+    if (wv > 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) red[wv - 1][e * 5 + k][lane] = dw[e][k];
+            red[wv - 1][e * 5 + 4][lane] = dbs[e];
+        }
+    }
+    __syncthreads();
+    if (wv == 0 && active) {
+        float *pp = a.partial + (((int64_t)b * a.nchunk + ch) * a.C + c0) * 5;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float v = 0.0f;
+                if (k < W) {
+                    v = dw[e][k < W ? k : 0];
+#pragma unroll
+                    for (int q = 0; q < NW - 1; ++q) v += red[q][e * 5 + k][lane];
+                }
+                pp[e * 5 + k] = v;
+            }
+            float v = dbs[e];
+#pragma unroll
+            for (int q = 0; q < NW - 1; ++q) v += red[q][e * 5 + 4][lane];
+            pp[e * 5 + 4] = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward, time-contiguous rows ([B, C, L]): one wave owns one segment of one
+// (b, c) row, U vectors of E time steps per lane, exactly as the forward
+// kernel.  Pass 1 recomputes z and dz = dout * act'(z) for the lane's own
+// steps (history from lane l-1 by wave shift) and accumulates the lane's share
+// of dweight / dbias; pass 2 forms dx[t] = sum_k w[k] * dz[t+(W-1)-k] with the
+// three later dz values taken from lane l+1 (wave shift the other way), from
+// the next vector's lane 0, or -- for the last lane of a segment that is not
+// the end of the row -- recomputed from memory.  The wave's dweight / dbias
+// are reduced across lanes in a fixed butterfly order and written as one
+// partial set entry; canon_bwd_reduce_kernel sums the sets.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_shift_down(float v, float last)
+{
+    // lane i <- lane i+1 across the whole wave; lane 63 <- `last`
+    return bits_f((uint32_t)__builtin_amdgcn_update_dpp((int)f_bits(last), (int)f_bits(v),
+                                                        0x130 /* wave_shl:1 */, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float read_lane0(float v)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_readfirstlane((int)f_bits(v)));
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+    // fixed-order butterfly: every lane ends with the same total
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <int DT, int W, int U, bool MASK>
+__global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    constexpr int BY = Elem<DT>::bytes;
+    const int lane = threadIdx.x & 63;
+    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    if (task >= a.nthreads) return;          // nthreads = wave tasks in this kernel
+    uint32_t row = task, seg = 0;
+    if (a.nchunk > 1) {                      // nchunk = segments per row
+        row = fdiv(task, a.div_nchunk);
+        seg = task - row * a.nchunk;
+    }
+    const uint32_t b = fdiv(row, a.div_nvec);   // div_nvec divides by C here
+    const uint32_t c = row - b * a.C;
+
+    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * BY;
+    const char *grow = a.dy + ((int64_t)b * a.g_sb + (int64_t)c * a.g_sc) * BY;
+    char *drow = a.dx + ((int64_t)b * a.d_sb + (int64_t)c * a.d_sc) * BY;
+    const uint32_t nvec = a.L / E;
+    const uint32_t v0 = seg * (64u * U) + lane;
+
+    uint4 X[U], G[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        const uint32_t vc = v < nvec ? v : nvec - 1u;
+        X[u] = load_vec<false>(xrow + (int64_t)vc * 16);
+        G[u] = load_vec<false>(grow + (int64_t)vc * 16);
+    }
+    RawTaps<1> raw;
+    fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
+    float M[MASK ? U : 1][E];
+    if constexpr (MASK) {
+        int64_t mbase[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t v = v0 + u * 64u;
+            mbase[u] = b * a.m_sb + (int64_t)(v < nvec ? v : nvec - 1u) * E * a.m_sl;
+        }
+        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+    }
+    float w[1][W], bvv[1];
+    decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
+    const float bv = bvv[0];
+
+    // left history of the segment's first vector (lane 0 only), right dz of its last vector (lane 63 only)
+    float carry[3] = {0.0f, 0.0f, 0.0f};
+    float edge[3] = {0.0f, 0.0f, 0.0f};
+    const int64_t t_seg0 = (int64_t)seg * (64 * U) * E;
+    const int64_t t_seg1 = t_seg0 + (int64_t)(64 * U) * E;      // first step after the segment
+    if (lane == 0 && seg > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            float v = load1<DT>(xrow, t_seg0 - 3 + j);
+            if constexpr (MASK) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + (t_seg0 - 3 + j) * a.m_sl, a.mask_dtype));
+            carry[j] = v;
+        }
+    }
+    if (lane == 63 && t_seg1 < (int64_t)a.L) {
+        // dz[t_seg1 + j], j = 0..2, from x[t_seg1-3 .. t_seg1+2] and dout[t_seg1 .. t_seg1+2]
+        float xs6[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            const int64_t t = t_seg1 - 3 + i;
+            float v = 0.0f;
+            if (t < (int64_t)a.L) {
+                v = load1<DT>(xrow, t);
+                if constexpr (MASK) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            }
+            xs6[i] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int64_t t = t_seg1 + j;
+            if (t < (int64_t)a.L) {
+                float z = bv;
+#pragma unroll
+                for (int k = 0; k < W; ++k) z = fmaf(w[0][k], xs6[j + (4 - W) + k], z);
+                const float g = load1<DT>(grow, t);
+                edge[j] = a.act ? g * silu_grad(z) : g;
+            }
+        }
+    }
+
+    // pass 1: dz of the lane's own steps, and its share of dweight / dbias
+    float dz[U][E], gg[U][E];
+    float dwl[W], dbl = 0.0f;
+#pragma unroll
+    for (int k = 0; k < W; ++k) dwl[k] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const bool valid = v0 + u * 64u < nvec;
+        float xr[E], xm_store[MASK ? E : 1];
+        float *xm = MASK ? xm_store : xr;
+        unpack_vec<DT>(X[u], xr);
+        unpack_vec<DT>(G[u], gg[u]);
+        if constexpr (MASK) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
+        }
+        float seq[E + 3];
+        seq[0] = wave_shift_up(xm[E - 3], carry[0]);
+        seq[1] = wave_shift_up(xm[E - 2], carry[1]);
+        seq[2] = wave_shift_up(xm[E - 1], carry[2]);
+        if (u + 1 < U) {
+            carry[0] = read_lane63(xm[E - 3]);
+            carry[1] = read_lane63(xm[E - 2]);
+            carry[2] = read_lane63(xm[E - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) seq[3 + j] = xm[j];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float z = bv;
+#pragma unroll
+            for (int k = 0; k < W; ++k) z = fmaf(w[0][k], seq[j + (4 - W) + k], z);
+            dz[u][j] = z;
+        }
+        if (a.act) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = gg[u][j] * silu_grad(dz[u][j]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = gg[u][j];
+        }
+        if (!valid) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dz[u][j] = 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) dwl[k] = fmaf(dz[u][j], seq[j + (4 - W) + k], dwl[k]);
+            dbl += dz[u][j];
+        }
+    }
+
+    // pass 2: dx
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        // the three dz values after this vector: lane l+1 of the same step, for lane 63 lane 0 of the next
+        float nx[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const float last = (u + 1 < U) ? read_lane0(dz[u + 1 < U ? u + 1 : u][j]) : edge[j];
+            nx[j] = wave_shift_down(dz[u][j], last);
+        }
+        float dq[E + 3];
+#pragma unroll
+        for (int j = 0; j < E; ++j) dq[j] = dz[u][j];
+        dq[E] = nx[0]; dq[E + 1] = nx[1]; dq[E + 2] = nx[2];
+        float o[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float acc = w[0][W - 1] * dq[j];
+#pragma unroll
+            for (int k = W - 2; k >= 0; --k) acc = fmaf(w[0][k], dq[j + (W - 1) - k], acc);
+            o[j] = acc;
+        }
+        if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += gg[u][j];
+        }
+        if constexpr (MASK) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] *= M[u][j];
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += gg[u][j];
+        }
+        if (v < nvec) store_vec<false>(drow + (int64_t)v * 16, pack_vec<DT>(o));
+    }
+
+    // the wave's dweight / dbias -> partial[(b * nseg + seg) * C + c][5]
+    float tot[5];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) tot[k] = k < W ? wave_sum(dwl[k < W ? k : 0]) : 0.0f;
+    tot[4] = wave_sum(dbl);
+    if (lane == 0) {
+        float *pp = a.partial + (((int64_t)b * a.nchunk + seg) * a.C + c) * 5;
+#pragma unroll
+        for (int k = 0; k < 5; ++k) pp[k] = tot[k];
+    }
+}
+
+// dweight[c, k] / dbias[c] = sum over the partial sets, in a fixed order: a block owns 32 adjacent
+// (c, j) columns; its 8 slices each sum every 8th set in set order (fp64), then the slices are added
+// in slice order.  Reads are 128 contiguous bytes per set and slice.
+__global__ __launch_bounds__(256) void canon_zero_kernel(float *p, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+__global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *partial, float *dweight, float *dbias,
+                                                              uint32_t C, uint32_t nsets, int W)
+{
+    __shared__ double part[8][32];
+    const uint32_t col = threadIdx.x & 31u, slice = threadIdx.x >> 5;
+    const uint32_t ncols = C * 5u;
+    const uint32_t i = blockIdx.x * 32u + col;   // (c, j), j in 0..4
+    double acc = 0.0;
+    if (i < ncols)
+        for (uint32_t s = slice; s < nsets; s += 8u) acc += (double)partial[(int64_t)s * ncols + i];
+    part[slice][col] = acc;
+    __syncthreads();
+    if (slice != 0 || i >= ncols) return;
+    double total = part[0][col];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) total += part[k][col];
+    const uint32_t c = i / 5u, j = i - c * 5u;
+    if (j < 4) {
+        if ((int)j < W) dweight[c * W + j] = (float)total;
+    } else if (dbias) {
+        dbias[c] = (float)total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// launch
+// ---------------------------------------------------------------------------
+namespace {
+
+template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStream_t s)
+{
+    const dim3 g(pl.grid), b(256);
+    if (pl.kind == BWD_BCL_VEC) {
+        switch (pl.U) {
+        case 4: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 4, MASK>), g, b, 0, s, pl.args); break;
+        case 2: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 2, MASK>), g, b, 0, s, pl.args); break;
+        default: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 1, MASK>), g, b, 0, s, pl.args); break;
+        }
+    } else if (pl.kind == BWD_BLC_VEC)
+    {
+        if (pl.args.act) hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, true>), g, b, 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, false>), g, b, 0, s, pl.args);
+    }
+    else
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, 1, false, MASK, kBwdRows>), g, b, 0, s, pl.args);
+}
+
+template <int DT> void launch_bwd(const BwdPlan &pl, hipStream_t s)
+{
+    const bool m = pl.args.mask != nullptr;
+    switch (pl.args.W) {
+    case 2: m ? launch_bwd_m<DT, 2, true>(pl, s) : launch_bwd_m<DT, 2, false>(pl, s); break;
+    case 3: m ? launch_bwd_m<DT, 3, true>(pl, s) : launch_bwd_m<DT, 3, false>(pl, s); break;
+    default: m ? launch_bwd_m<DT, 4, true>(pl, s) : launch_bwd_m<DT, 4, false>(pl, s); break;
+    }
+}
+
+}  // namespace
+
+void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s)
+{
+    switch (x_dtype) {
+    case CANON_DTYPE_F32: launch_bwd<CANON_DTYPE_F32>(pl, s); break;
+    case CANON_DTYPE_BF16: launch_bwd<CANON_DTYPE_BF16>(pl, s); break;
+    default: launch_bwd<CANON_DTYPE_F16>(pl, s); break;
+    }
+    hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 31u) / 32u), dim3(256), 0, s,
+                       pl.args.partial, pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.nsets, pl.args.W);
+}
+
+void launch_zero(float *p, uint32_t n, hipStream_t s)
+{
+    if (n) hipLaunchKernelGGL(canon_zero_kernel, dim3((n + 255) / 256), dim3(256), 0, s, p, n);
+}
+
+}  // namespace canon

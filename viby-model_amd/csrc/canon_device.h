@@ -1,0 +1,607 @@
+// Device-side helpers shared by the kernels: storage-type conversions, vector
+// and mask loads, tap fetch / decode, wave shifts.  Everything is
+// __device__ __forceinline__ or a template, so the header may be included by
+// every kernel translation unit.
+#ifndef CANON_DEVICE_H
+#define CANON_DEVICE_H
+
+#include <type_traits>
+
+#include "canon_plan.h"
+
+namespace canon {
+
+// ---------------------------------------------------------------------------
+// storage types
+// ---------------------------------------------------------------------------
+template <int DT> struct Elem;
+template <> struct Elem<CANON_DTYPE_F32> { static constexpr int bytes = 4; static constexpr int per_vec = 4; };
+template <> struct Elem<CANON_DTYPE_BF16> { static constexpr int bytes = 2; static constexpr int per_vec = 8; };
+template <> struct Elem<CANON_DTYPE_F16> { static constexpr int bytes = 2; static constexpr int per_vec = 8; };
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bits_f(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f_bits(float f) { return __float_as_uint(f); }
+
+// two packed 16-bit values -> two floats
+template <int DT> __device__ __forceinline__ void unpack2(uint32_t u, float &lo, float &hi)
+{
+    if constexpr (DT == CANON_DTYPE_BF16) {
+        lo = bits_f(u << 16);
+        hi = bits_f(u & 0xFFFF0000u);
+    } else {
+        f16x2_t h = __builtin_bit_cast(f16x2_t, u);
+        lo = (float)h.x;
+        hi = (float)h.y;
+    }
+}
+
+// two floats -> two packed 16-bit values, round to nearest even
+template <int DT> __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+    float2_t v = {lo, hi};
+    if constexpr (DT == CANON_DTYPE_BF16) {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    } else {
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    }
+}
+
+// value -> storage type -> value
+template <int DT> __device__ __forceinline__ float round_through(float v)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        return v;
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        return (float)(__bf16)v;
+    } else {
+        return (float)(_Float16)v;
+    }
+}
+
+// x * m rounded to the storage type.  For fp16 the product is hidden from the
+// instruction selector: it would otherwise fuse multiply and conversion into
+// v_fma_mixlo_f16 with a +0 addend, which turns a -0 product into +0, and the
+// captured conv state must carry the bits of x * mask exactly.
+template <int DT> __device__ __forceinline__ float mul_round(float x, float m)
+{
+    float p = x * m;
+    if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(p));
+    return round_through<DT>(p);
+}
+
+template <int DT> __device__ __forceinline__ void unpack_vec(const uint4 &v, float *f)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        f[0] = bits_f(v.x); f[1] = bits_f(v.y); f[2] = bits_f(v.z); f[3] = bits_f(v.w);
+    } else {
+        unpack2<DT>(v.x, f[0], f[1]);
+        unpack2<DT>(v.y, f[2], f[3]);
+        unpack2<DT>(v.z, f[4], f[5]);
+        unpack2<DT>(v.w, f[6], f[7]);
+    }
+}
+
+template <int DT> __device__ __forceinline__ uint4 pack_vec(const float *f)
+{
+    uint4 v;
+    if constexpr (DT == CANON_DTYPE_F32) {
+        v.x = f_bits(f[0]); v.y = f_bits(f[1]); v.z = f_bits(f[2]); v.w = f_bits(f[3]);
+    } else {
+        v.x = pack2<DT>(f[0], f[1]);
+        v.y = pack2<DT>(f[2], f[3]);
+        v.z = pack2<DT>(f[4], f[5]);
+        v.w = pack2<DT>(f[6], f[7]);
+    }
+    return v;
+}
+
+template <int DT> __device__ __forceinline__ float load1(const void *p, int64_t i)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        return ((const float *)p)[i];
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        return bits_f((uint32_t)((const uint16_t *)p)[i] << 16);
+    } else {
+        return (float)((const _Float16 *)p)[i];
+    }
+}
+
+template <int DT> __device__ __forceinline__ void store1(void *p, int64_t i, float v)
+{
+    if constexpr (DT == CANON_DTYPE_F32) {
+        ((float *)p)[i] = v;
+    } else if constexpr (DT == CANON_DTYPE_BF16) {
+        ((__bf16 *)p)[i] = (__bf16)v;
+    } else {
+        ((_Float16 *)p)[i] = (_Float16)v;
+    }
+}
+
+// weight / bias element of run-time type
+__device__ __forceinline__ float load_w(const void *p, int64_t i, int dt)
+{
+    if (dt == CANON_DTYPE_F32) return load1<CANON_DTYPE_F32>(p, i);
+    if (dt == CANON_DTYPE_BF16) return load1<CANON_DTYPE_BF16>(p, i);
+    return load1<CANON_DTYPE_F16>(p, i);
+}
+
+__device__ __forceinline__ float load_mask(const void *p, int64_t i, int dt)
+{
+    switch (dt) {
+    case CANON_MASK_U8: return (float)((const uint8_t *)p)[i];
+    case CANON_MASK_I32: return (float)((const int32_t *)p)[i];
+    case CANON_MASK_I64: return (float)((const int64_t *)p)[i];
+    case CANON_MASK_F32: return ((const float *)p)[i];
+    case CANON_MASK_BF16: return load1<CANON_DTYPE_BF16>(p, i);
+    default: return load1<CANON_DTYPE_F16>(p, i);
+    }
+}
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16-byte access; NT marks streaming data that will not be touched again soon
+template <bool NT> __device__ __forceinline__ uint4 load_vec(const void *p)
+{
+    const u32x4_t *q = (const u32x4_t *)p;
+    u32x4_t v;
+    if constexpr (NT) v = __builtin_nontemporal_load(q);
+    else v = *q;
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint4 &v)
+{
+    const u32x4_t q = {v.x, v.y, v.z, v.w};
+    if constexpr (NT) __builtin_nontemporal_store(q, (u32x4_t *)p);
+    else *(u32x4_t *)p = q;
+}
+
+// (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
+// the value almost always fits 32 bits and one conversion instruction does it
+__device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
+{
+    if ((int32_t)hi == ((int32_t)lo >> 31)) return (float)(int32_t)lo;
+    return (float)(int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// N mask entries of consecutive time steps t_first .. t_first+N-1 (clamped to
+// [0, L-1]) of one batch row.  The element-type switch sits outside the loops
+// and every case is straight-line code, so all N loads are issued back to back
+// and waited for once (a per-entry switch puts a wait after every load, which
+// also waits for -- and so serialises -- the row loads issued before it).
+template <int N>
+__device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
+                                               int dt, float *m)
+{
+    int64_t idx[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        int64_t t = t_first + j;
+        t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+        idx[j] = row_base + t * stride;
+    }
+    switch (dt) {
+    case CANON_MASK_U8:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[idx[j]];
+        break;
+    case CANON_MASK_I32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[idx[j]];
+        break;
+    case CANON_MASK_I64: {
+        uint2 q[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) q[j] = ((const uint2 *)p)[idx[j]];
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = i64_words_to_float(q[j].x, q[j].y);
+        break;
+    }
+    case CANON_MASK_F32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[idx[j]];
+        break;
+    case CANON_MASK_BF16:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, idx[j]);
+        break;
+    default:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, idx[j]);
+        break;
+    }
+}
+
+// A lane's access unit in the channel-contiguous kernels: 16 bytes, or 8 bytes (half the registers
+// per lane, twice the waves in flight)
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+template <int VB> struct VecIO;
+template <> struct VecIO<16> {
+    using type = uint4;
+    static __device__ __forceinline__ type zero() { return make_uint4(0, 0, 0, 0); }
+    template <bool NT> static __device__ __forceinline__ type load(const void *p) { return load_vec<NT>(p); }
+    template <bool NT> static __device__ __forceinline__ void store(void *p, const type &v) { store_vec<NT>(p, v); }
+    template <int DT> static __device__ __forceinline__ void unpack(const type &v, float *f) { unpack_vec<DT>(v, f); }
+    template <int DT> static __device__ __forceinline__ type pack(const float *f) { return pack_vec<DT>(f); }
+};
+template <> struct VecIO<8> {
+    using type = uint2;
+    static __device__ __forceinline__ type zero() { return make_uint2(0, 0); }
+    template <bool NT> static __device__ __forceinline__ type load(const void *p)
+    {
+        const u32x2_t *q = (const u32x2_t *)p;
+        u32x2_t v;
+        if constexpr (NT) v = __builtin_nontemporal_load(q);
+        else v = *q;
+        return make_uint2(v.x, v.y);
+    }
+    template <bool NT> static __device__ __forceinline__ void store(void *p, const type &v)
+    {
+        const u32x2_t q = {v.x, v.y};
+        if constexpr (NT) __builtin_nontemporal_store(q, (u32x2_t *)p);
+        else *(u32x2_t *)p = q;
+    }
+    template <int DT> static __device__ __forceinline__ void unpack(const type &v, float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) {
+            f[0] = bits_f(v.x);
+            f[1] = bits_f(v.y);
+        } else {
+            unpack2<DT>(v.x, f[0], f[1]);
+            unpack2<DT>(v.y, f[2], f[3]);
+        }
+    }
+    template <int DT> static __device__ __forceinline__ type pack(const float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return make_uint2(f_bits(f[0]), f_bits(f[1]));
+        else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
+    }
+};
+
+// N sequence indices of consecutive time steps t_first .. t_first+N-1 (clamped to [0, L-1]) of one batch row
+template <int N>
+__device__ __forceinline__ void load_seq_rows(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
+                                              int32_t *q)
+{
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        int64_t t = t_first + j;
+        t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+        q[j] = p[row_base + t * stride];
+    }
+}
+
+// U runs of N (4 or 8) consecutive mask entries, run u starting at element
+// base[u].  The element-type switch sits outside the loops and every case is
+// straight-line code, so all loads are issued back to back and waited for
+// once.  `vec` (decided on the host) says the entries are contiguous and each
+// run is aligned to its own size: it is fetched with a few wide loads instead
+// of N narrow ones.
+template <int N, int U>
+__device__ __forceinline__ void load_mask_vec(const void *p, const int64_t *base, int64_t stride, int dt, bool vec,
+                                              float (*m)[N])
+{
+    if (vec) {
+        switch (dt) {
+        case CANON_MASK_U8: {
+            uint32_t q[U][N / 4];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint32_t *)((const uint8_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < N; ++j) m[u][j] = (float)((q[u][j / 4] >> (8 * (j % 4))) & 0xFFu);
+            return;
+        }
+        case CANON_MASK_I32: {
+            uint4 q[U][N / 4];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint4 *)((const int32_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) {
+                    m[u][4 * i] = (float)(int32_t)q[u][i].x; m[u][4 * i + 1] = (float)(int32_t)q[u][i].y;
+                    m[u][4 * i + 2] = (float)(int32_t)q[u][i].z; m[u][4 * i + 3] = (float)(int32_t)q[u][i].w;
+                }
+            return;
+        }
+        case CANON_MASK_I64: {
+            uint4 q[U][N / 2];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) q[u][i] = ((const uint4 *)((const int64_t *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) {
+                    m[u][2 * i] = i64_words_to_float(q[u][i].x, q[u][i].y);
+                    m[u][2 * i + 1] = i64_words_to_float(q[u][i].z, q[u][i].w);
+                }
+            return;
+        }
+        case CANON_MASK_F32: {
+            uint4 q[U][N / 4];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint4 *)((const float *)p + base[u]))[i];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 4; ++i) {
+                    m[u][4 * i] = bits_f(q[u][i].x); m[u][4 * i + 1] = bits_f(q[u][i].y);
+                    m[u][4 * i + 2] = bits_f(q[u][i].z); m[u][4 * i + 3] = bits_f(q[u][i].w);
+                }
+            return;
+        }
+        default: {   // bf16 / fp16
+            uint32_t q[U][N / 2];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if constexpr (N == 8) {
+                    const uint4 v = *(const uint4 *)((const uint16_t *)p + base[u]);
+                    q[u][0] = v.x; q[u][1] = v.y; q[u][2 % (N / 2)] = v.z; q[u][3 % (N / 2)] = v.w;
+                } else {
+                    const uint2 v = *(const uint2 *)((const uint16_t *)p + base[u]);
+                    q[u][0] = v.x; q[u][1] = v.y;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int i = 0; i < N / 2; ++i) {
+                    if (dt == CANON_MASK_BF16) unpack2<CANON_DTYPE_BF16>(q[u][i], m[u][2 * i], m[u][2 * i + 1]);
+                    else unpack2<CANON_DTYPE_F16>(q[u][i], m[u][2 * i], m[u][2 * i + 1]);
+                }
+            return;
+        }
+        }
+    }
+    switch (dt) {
+    case CANON_MASK_U8:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const uint8_t *)p)[base[u] + j * stride];
+        break;
+    case CANON_MASK_I32:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const int32_t *)p)[base[u] + j * stride];
+        break;
+    case CANON_MASK_I64:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = (float)((const int64_t *)p)[base[u] + j * stride];
+        break;
+    case CANON_MASK_F32:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = ((const float *)p)[base[u] + j * stride];
+        break;
+    case CANON_MASK_BF16:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = load1<CANON_DTYPE_BF16>(p, base[u] + j * stride);
+        break;
+    default:
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int j = 0; j < N; ++j) m[u][j] = load1<CANON_DTYPE_F16>(p, base[u] + j * stride);
+        break;
+    }
+}
+
+__device__ __forceinline__ float silu_fast(float v)
+{
+    // v / (1 + e^-v); v_exp_f32 and v_rcp_f32 are each good to 1 ulp
+    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+}
+
+__device__ __forceinline__ float silu_precise(float v) { return v / (1.0f + expf(-v)); }
+
+// lane i <- lane i-1 across the whole wave; lane 0 <- `first`
+__device__ __forceinline__ float wave_shift_up(float v, float first)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_update_dpp((int)f_bits(first), (int)f_bits(v),
+                                                        0x138 /* wave_shr:1 */, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ float read_lane63(float v)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), 63));
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
+{
+    const uint32_t t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
+// The activated, residual-added output of one element (fused rounding mode).
+__device__ __forceinline__ float finish(float acc, int act, int res_mode, float xm, float xr)
+{
+    if (act) acc = silu_fast(acc);
+    if (res_mode == CANON_RESIDUAL_MASKED) acc += xm;
+    else if (res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
+    return acc;
+}
+
+// Write final_state[b, c, :] for one row from global memory (the row was just
+// streamed by this wave, so these are cache hits).  One lane per slot.
+template <int DT>
+__device__ __forceinline__ void capture_row_state(const FwdArgs &a, uint32_t b, uint32_t c, int slot)
+{
+    if (slot >= a.S_out) return;
+    const int64_t t = (int64_t)a.L - a.S_out + slot;
+    float v = 0.0f;
+    if (t >= 0) {
+        v = load1<DT>(a.x, b * a.x_sb + c * a.x_sc + t * a.x_sl);
+        if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+    } else if (a.init && a.S_in + t >= 0) {
+        v = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+    }
+    store1<DT>(a.fin, b * a.f_sb + c * a.f_sc + slot * a.f_ss, v);
+}
+
+// Taps and bias of NC adjacent channels, in two phases so that the loads can
+// be issued early and nothing waits on them until the values are needed:
+// fetch_taps() only loads raw bits, decode_taps() converts them (rounded to
+// the storage type of x).  `vec` (decided on the host): weight is a
+// contiguous, 16-byte aligned [C, 4].
+template <int NC> struct RawTaps {
+    uint32_t w[NC][4];   // fp32: one tap per word; 16-bit + vec: two taps per word in w[.][0..1];
+                         // 16-bit scalar path: one tap per word, low half
+    uint32_t b[NC];
+};
+
+template <int W, int NC>
+__device__ __forceinline__ void fetch_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
+                                           int w_dtype, bool vec, bool bvec, uint32_t c0, RawTaps<NC> &r)
+{
+    const bool wide = w_dtype == CANON_DTYPE_F32;
+    // bias first: whatever follows the tap loads may wait on them, and nothing must be issued after a wait
+    if (bias) {
+        if (wide) {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
+        } else if (NC == 8 && bvec) {
+            // eight 16-bit biases are one aligned 16-byte run (c0 is a multiple of 8)
+            const uint4 q = *(const uint4 *)((const uint16_t *)bias + c0);
+            r.b[0] = q.x & 0xFFFFu; r.b[1 % NC] = q.x >> 16;
+            r.b[2 % NC] = q.y & 0xFFFFu; r.b[3 % NC] = q.y >> 16;
+            r.b[4 % NC] = q.z & 0xFFFFu; r.b[5 % NC] = q.z >> 16;
+            r.b[6 % NC] = q.w & 0xFFFFu; r.b[7 % NC] = q.w >> 16;
+        } else {
+#pragma unroll
+            for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
+        }
+    }
+    if (W == 4 && vec) {
+        if (wide) {
+            const uint4 *p = (const uint4 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < NC; ++e) {
+                const uint4 q = p[e];
+                r.w[e][0] = q.x; r.w[e][1] = q.y; r.w[e][2] = q.z; r.w[e][3] = q.w;
+            }
+        } else if constexpr (NC % 2 == 0) {
+            const uint4 *p = (const uint4 *)((const uint2 *)weight + c0);   // c0 is a multiple of NC
+#pragma unroll
+            for (int e = 0; e < NC; e += 2) {
+                const uint4 q = p[e / 2];
+                r.w[e][0] = q.x; r.w[e][1] = q.y;
+                r.w[e + 1][0] = q.z; r.w[e + 1][1] = q.w;
+            }
+        } else {
+            const uint2 *p = (const uint2 *)weight + c0;
+#pragma unroll
+            for (int e = 0; e < NC; ++e) {
+                const uint2 q = p[e];
+                r.w[e][0] = q.x; r.w[e][1] = q.y;
+            }
+        }
+    } else if (wide) {
+#pragma unroll
+        for (int e = 0; e < NC; ++e)
+#pragma unroll
+            for (int k = 0; k < W; ++k) r.w[e][k] = ((const uint32_t *)weight)[(int64_t)(c0 + e) * w_sc + k * w_sk];
+    } else {
+#pragma unroll
+        for (int e = 0; e < NC; ++e)
+#pragma unroll
+            for (int k = 0; k < W; ++k) r.w[e][k] = ((const uint16_t *)weight)[(int64_t)(c0 + e) * w_sc + k * w_sk];
+    }
+}
+
+// One channel's taps for a whole wave (c is wave-uniform): shaped so that the
+// common cases become scalar-memory loads.  `pair`: bias may be read as the
+// aligned 32-bit word that contains element c.
+template <int W>
+__device__ __forceinline__ void fetch_taps_uniform(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
+                                                   int w_dtype, bool vec, bool pair, uint32_t c, RawTaps<1> &r)
+{
+    const bool wide = w_dtype == CANON_DTYPE_F32;
+    if (bias && pair) {
+        if (wide) {
+            r.b[0] = ((const uint32_t *)bias)[c];
+        } else {
+            const uint32_t d = ((const uint32_t *)bias)[c >> 1];
+            r.b[0] = (c & 1u) ? (d >> 16) : (d & 0xFFFFu);
+        }
+        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, false, c, r);
+    } else {
+        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, false, c, r);
+    }
+}
+
+template <int WDT> __device__ __forceinline__ float half_bits_f(uint32_t raw)
+{
+    if constexpr (WDT == CANON_DTYPE_BF16) return bits_f(raw << 16);
+    else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+}
+
+template <int DT, int WDT, int W, int NC>
+__device__ __forceinline__ void decode_taps_typed(const RawTaps<NC> &r, bool vec, bool has_bias, float (*w)[W], float *bv)
+{
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        if constexpr (WDT == CANON_DTYPE_F32) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) w[e][k] = round_through<DT>(bits_f(r.w[e][k]));
+            bv[e] = has_bias ? round_through<DT>(bits_f(r.b[e])) : 0.0f;
+        } else {
+            if (W == 4 && vec) {
+                float t0, t1, t2, t3;
+                unpack2<WDT>(r.w[e][0], t0, t1);
+                unpack2<WDT>(r.w[e][1], t2, t3);
+                w[e][0] = round_through<DT>(t0);
+                w[e][1] = round_through<DT>(t1);
+                w[e][W - 2] = round_through<DT>(t2);
+                w[e][W - 1] = round_through<DT>(t3);
+            } else {
+#pragma unroll
+                for (int k = 0; k < W; ++k) w[e][k] = round_through<DT>(half_bits_f<WDT>(r.w[e][k]));
+            }
+            bv[e] = has_bias ? round_through<DT>(half_bits_f<WDT>(r.b[e])) : 0.0f;
+        }
+    }
+}
+
+template <int DT, int W, int NC>
+__device__ __forceinline__ void decode_taps(const RawTaps<NC> &r, int w_dtype, bool vec, bool has_bias, float (*w)[W], float *bv)
+{
+    // weights that already have the storage type of x need no rounding: decode them as if x were fp32
+    if (w_dtype == DT) decode_taps_typed<CANON_DTYPE_F32, DT, W, NC>(r, vec, has_bias, w, bv);
+    else if (w_dtype == CANON_DTYPE_F32) decode_taps_typed<DT, CANON_DTYPE_F32, W, NC>(r, vec, has_bias, w, bv);
+    else if (w_dtype == CANON_DTYPE_BF16) decode_taps_typed<DT, CANON_DTYPE_BF16, W, NC>(r, vec, has_bias, w, bv);
+    else decode_taps_typed<DT, CANON_DTYPE_F16, W, NC>(r, vec, has_bias, w, bv);
+}
+
+template <typename Args>
+__device__ __forceinline__ uint32_t part_of_block(const PartTable<Args> &m, uint32_t blk)
+{
+    uint32_t p = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxParts; ++i) p += blk >= m.first_block[i] ? 1u : 0u;
+    return p;
+}
+
+}  // namespace canon
+#endif  // CANON_DEVICE_H

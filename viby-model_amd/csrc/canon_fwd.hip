@@ -1,0 +1,571 @@
+// Canon causal depthwise conv1d for MI355X (gfx950, wave64): the prefill kernels
+// (time-contiguous, channel-contiguous, strided) and their launchers.
+//
+// The op is a width-<=4 FIR per (batch, channel) row: ~2 flop per byte moved,
+// so every kernel here is organised around HBM traffic, not arithmetic:
+//   * one 16-byte load and one 16-byte store per lane per vector, each element
+//     of x read from HBM once and each element of out written once;
+//   * the (W-1)-element history a vector needs comes from the neighbouring
+//     lane (DPP wave shift) or from the previous vector of the same wave held
+//     in registers; only the first lane of a row segment touches memory for it;
+//   * taps and bias live in registers; bias, SiLU, mask multiply, residual and
+//     the conv-state capture are fused into the same pass.
+//
+// Arithmetic contract (the tests hold a CPU restatement of exactly this):
+//     acc = bias;  for k in 0..W-1: acc = fmaf(w[k], xm[t-(W-1)+k], acc)
+// taps/bias rounded to the storage type of x first; one rounding at the store.
+#include "canon_device.h"
+
+namespace canon {
+
+// ---------------------------------------------------------------------------
+// prefill, time-contiguous rows ([B, C, L], x_stride_l == 1)
+//
+// One wave owns one segment of one (b, c) row: U vectors per lane, lane l of
+// step u holding elements [(seg*U + u)*64 + l] * E .. +E.  All U loads are
+// issued before any arithmetic.  The three elements before a vector come from
+// lane l-1 (wave shift), for lane 0 from lane 63 of the previous step, and for
+// the very first vector of the segment from memory / the initial state / zero.
+// Everything that does not change per element (activation, residual, mask
+// element type) is branched on once per vector, never per element, so the
+// unmasked path is ~130 VALU instructions per 2 KB row and hides under the
+// memory time.
+// ---------------------------------------------------------------------------
+template <int DT, int W, int U, bool MASK, bool NT>
+__global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    const int lane = threadIdx.x & 63;
+    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    if (task >= a.ntasks) return;
+    uint32_t row = task, seg = 0;
+    if (a.nseg > 1) {
+        row = fdiv(task, a.div_nseg);
+        seg = task - row * a.nseg;
+    }
+    const uint32_t b = fdiv(row, a.div_C);
+    const uint32_t c = row - b * a.C;
+
+    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
+    char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
+    const uint32_t v0 = seg * (64u * U) + lane;
+
+    // row data first (the long latency), then the taps (scalar-cache hits)
+    uint4 X[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        X[u] = make_uint4(0, 0, 0, 0);
+        if (v < a.nvec) X[u] = load_vec<NT>(xrow + (int64_t)v * 16);
+    }
+
+    RawTaps<1> raw;
+    fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
+
+    // all mask entries of the segment, requested before anything is consumed
+    float M[MASK ? U : 1][E];
+    if constexpr (MASK) {
+        int64_t mbase[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t v = v0 + u * 64u;
+            mbase[u] = b * a.m_sb + (int64_t)(v < a.nvec ? v : a.nvec - 1u) * E * a.m_sl;   // idle lanes shadow the last vector
+        }
+        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+    }
+
+    float w[1][W], bvv[1];
+    decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
+    const float bv = bvv[0];
+
+    // history of the segment's first vector (only lane 0's copy is consumed)
+    float carry[3] = {0.0f, 0.0f, 0.0f};
+    if (lane == 0) {
+        if (seg > 0) {
+            const int64_t t0 = (int64_t)v0 * E;
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                float v = load1<DT>(xrow, t0 - 3 + j);
+                if constexpr (MASK)
+                    v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + (t0 - 3 + j) * a.m_sl, a.mask_dtype));
+                carry[j] = v;
+            }
+        } else if (a.init) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                if (j >= 3 - (W - 1))
+                    carry[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+        }
+    }
+
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * 64u;
+        float xr[E], xm_store[MASK ? E : 1];
+        float *xm = MASK ? xm_store : xr;
+        unpack_vec<DT>(X[u], xr);
+        if constexpr (MASK) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
+        }
+        // seq[0..2] = the three masked inputs before this vector
+        float seq[E + 3];
+        seq[0] = wave_shift_up(xm[E - 3], carry[0]);
+        seq[1] = wave_shift_up(xm[E - 2], carry[1]);
+        seq[2] = wave_shift_up(xm[E - 1], carry[2]);
+        if (u + 1 < U) {
+            carry[0] = read_lane63(xm[E - 3]);
+            carry[1] = read_lane63(xm[E - 2]);
+            carry[2] = read_lane63(xm[E - 1]);
+        }
+#pragma unroll
+        for (int j = 0; j < E; ++j) seq[3 + j] = xm[j];
+
+        float o[E];
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            float acc = bv;
+#pragma unroll
+            for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
+            o[j] = acc;
+        }
+        if (a.act) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] = silu_fast(o[j]);
+        }
+        if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += xr[j];
+        } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) o[j] += xm[j];
+        }
+        if (v < a.nvec) store_vec<NT>(orow + (int64_t)v * 16, pack_vec<DT>(o));
+    }
+
+    if (a.fin && seg == a.nseg - 1) capture_row_state<DT>(a, b, c, lane);
+}
+
+// ---------------------------------------------------------------------------
+// prefill, channel-contiguous rows ([B, L, C] memory, x_stride_c == 1): the
+// layout CanonLayer hands over (a transposed view of [B, T, D]).
+//
+// One lane owns E adjacent channels (VB = 8 bytes of every row: 4 x 16-bit or
+// 2 x fp32; 16-byte lanes need 142 registers and measured 4-9 % slower) and R
+// consecutive time steps; the four waves of a block own four consecutive
+// R-row slabs of the same 64-lane channel tile, so a block streams a
+// [4R rows] x [512 B] tile and consecutive blocks sweep memory in address
+// order (short-lived waves over a compact window: measured to be what HBM
+// wants; long per-lane time runs lose 10-20 %).  The three rows a wave needs from before its slab are the
+// last three rows of the previous wave: each wave publishes the raw tail of
+// its slab in LDS, one barrier, the next wave picks it up -- only the first
+// wave of a block reads its halo from memory.  All loads (slab, halo, taps)
+// are issued before the first wait.
+// ---------------------------------------------------------------------------
+// keep0..2 (wave uniform): whether the rows t-3, t-2, t-1 belong to the packed sequence of row t
+// (always true without seq_idx); a row of another sequence enters as zeros.
+template <int DT, int W, bool MASK, bool NT, int VB>
+__device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias,
+                                        float (*hist)[VB / Elem<DT>::bytes], const typename VecIO<VB>::type &X, float m,
+                                        char *optr, bool active, bool keep0 = true, bool keep1 = true, bool keep2 = true)
+{
+    constexpr int E = VB / Elem<DT>::bytes;
+    float xr[E], xm_store[MASK ? E : 1], o[E];
+    float *xm = MASK ? xm_store : xr;
+    VecIO<VB>::template unpack<DT>(X, xr);
+    if constexpr (MASK) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) xm[e] = mul_round<DT>(xr[e], m);
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        float acc = bias[e];
+        if constexpr (W == 4) acc = fmaf(w[e][0], keep0 ? hist[0][e] : 0.0f, acc);
+        if constexpr (W >= 3) acc = fmaf(w[e][W - 3], keep1 ? hist[1][e] : 0.0f, acc);
+        acc = fmaf(w[e][W - 2], keep2 ? hist[2][e] : 0.0f, acc);
+        acc = fmaf(w[e][W - 1], xm[e], acc);
+        o[e] = acc;
+        hist[0][e] = hist[1][e];
+        hist[1][e] = hist[2][e];
+        hist[2][e] = xm[e];
+    }
+    if (a.act) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
+    }
+    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] += xr[e];
+    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] += xm[e];
+    }
+    if (active) VecIO<VB>::template store<NT>(optr, VecIO<VB>::template pack<DT>(o));
+}
+
+template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
+__device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
+{
+    constexpr int E = VB / Elem<DT>::bytes;
+    using V = VecIO<VB>;
+    using vec_t = typename V::type;
+    static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
+    __shared__ vec_t tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
+
+    // blocks in plain memory order (an XCD-contiguous remap measured 3 % slower here)
+    // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
+    const uint32_t bt = fdiv(blk, a.div_nct);
+    const uint32_t ct = blk - bt * a.nct;
+    const uint32_t b = fdiv(bt, a.div_ntt);
+    const uint32_t tt = bt - b * a.ntt;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t cv = ct * 64u + lane;
+    const bool active = cv < a.nvec;
+    const uint32_t c0 = (active ? cv : a.nvec - 1u) * E;   // idle lanes shadow the last vector, loads need no predicate
+
+    const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * Elem<DT>::bytes;
+    char *ob = a.out + ((int64_t)b * a.o_sb + c0) * Elem<DT>::bytes;
+    const int64_t xs = a.x_sl * Elem<DT>::bytes, os = a.o_sl * Elem<DT>::bytes;
+    const int64_t t0 = ((int64_t)tt * kBlcWaves + wv) * R;
+    const int64_t left = (int64_t)a.L - t0;
+    const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
+    const int64_t t_last = (int64_t)a.L - 1;
+
+    // slab rows, then (first wave only) the three rows before the block, then the taps.
+    // Rows past the end of the sequence are clamped to the last row (loaded, never used).
+    vec_t X[R], H[3];
+    float m[R], mh[3];
+    int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
+    RawTaps<E> raw;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        X[r] = V::zero();
+        m[r] = 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < (SEQ ? R + 3 : 1); ++j) sq[j] = 0;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        H[j] = V::zero();
+        mh[j] = 0.0f;
+    }
+    if (rows > 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t t = t0 + r < t_last ? t0 + r : t_last;
+            X[r] = V::template load<NT>(xb + t * xs);
+        }
+        if (wv == 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = t0 - 3 + j;
+                if (j >= 3 - (W - 1) && t >= 0) H[j] = V::template load<false>(xb + t * xs);
+            }
+        }
+        // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
+        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
+        if constexpr (SEQ) load_seq_rows<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, sq);
+        if constexpr (MASK) {
+            // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
+            float mm[R + 3];
+            load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mm);
+#pragma unroll
+            for (int j = 0; j < 3; ++j) mh[j] = mm[j];
+#pragma unroll
+            for (int r = 0; r < R; ++r) m[r] = mm[3 + r];
+        }
+    }
+
+    // hand the raw tail of this slab to the next wave
+#pragma unroll
+    for (int j = 0; j < 3; ++j) tail[wv][j][lane] = X[R - 3 + j];
+    __syncthreads();
+    if (wv > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (j >= 3 - (W - 1)) H[j] = tail[wv - 1][j][lane];
+    }
+    if (rows == 0) return;   // after the barrier
+
+    // hist[j] = masked row t0 - 3 + j
+    float hist[3][E];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        V::template unpack<DT>(H[j], hist[j]);
+        if constexpr (MASK) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) hist[j][e] = mul_round<DT>(hist[j][e], mh[j]);
+        }
+    }
+    if (t0 == 0 && a.init && active) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            if (j < 3 - (W - 1)) continue;
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+        }
+    }
+    float w[E][W], bias[E];
+    decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+
+    if constexpr (SEQ) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= rows) continue;
+            // rows t-3, t-2, t-1 count only if they carry the index of row t; sequence boundaries are rare,
+            // so the all-kept case takes the plain code
+            const int32_t cur = sq[3 + r];
+            const bool k0 = sq[r] == cur, k1 = sq[r + 1] == cur, k2 = sq[r + 2] == cur;
+            if (k0 && k1 && k2) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+            else blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active, k0, k1, k2);
+        }
+    } else if (rows == R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (r < rows) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+    }
+
+    if (a.fin && active && t0 + rows == (int64_t)a.L) {
+        for (int slot = 0; slot < a.S_out; ++slot) {
+            const int64_t t = (int64_t)a.L - a.S_out + slot;
+            float v[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = 0.0f;
+            if (t >= 0) {
+                V::template unpack<DT>(V::template load<false>(xb + t * xs), v);
+                if constexpr (MASK) {
+                    const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) v[e] = mul_round<DT>(v[e], mm);
+                }
+            } else if (a.init && a.S_in + t >= 0) {
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    v[e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                store1<DT>(a.fin, b * a.f_sb + (int64_t)(c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
+        }
+    }
+}
+
+template <int DT, int W, int R, bool MASK, bool NT>
+__global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
+{
+    blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
+}
+
+// the same over packed variable-length sequences (seq_idx)
+template <int DT, int W, int R, bool MASK>
+__global__ __launch_bounds__(256) void canon_fwd_blc_seq_kernel(const FwdArgs a)
+{
+    blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
+}
+
+template <int DT, int W, int R, bool MASK, bool NT>
+__global__ __launch_bounds__(256) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
+{
+    const uint32_t p = part_of_block(m, blockIdx.x);
+    blc_block<DT, W, R, MASK, NT>(m.part[p], blockIdx.x - m.first_block[p]);
+}
+
+// ---------------------------------------------------------------------------
+// prefill, any strides / any length / either rounding mode: one thread per
+// (b, c, chunk of time steps), scalar accesses.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.ntasks) return;
+    // fastest-varying index follows the contiguous dimension of x
+    uint32_t b, c, ch;
+    if (a.x_sc == 1 && a.x_sl != 1) {
+        c = tid % a.C;
+        const uint32_t r = tid / a.C;
+        ch = r % a.nseg;
+        b = r / a.nseg;
+    } else {
+        ch = tid % a.nseg;
+        const uint32_t r = tid / a.nseg;
+        c = r % a.C;
+        b = r / a.C;
+    }
+    const int W = a.W;
+    float w[4] = {0, 0, 0, 0};
+    for (int k = 0; k < W; ++k)
+        w[4 - W + k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
+    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+
+    const int64_t xo = (int64_t)b * a.x_sb + (int64_t)c * a.x_sc;
+    const int64_t oo = (int64_t)b * a.o_sb + (int64_t)c * a.o_sc;
+    const int64_t t_begin = (int64_t)ch * a.chunk;
+    const int64_t t_stop = t_begin + (int64_t)a.chunk;
+    const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
+
+    float h[3] = {0, 0, 0};
+    int32_t qh[3] = {0, 0, 0};   // with seq_idx: the sequence each history position belongs to
+    const int32_t *seq = a.seq ? a.seq + (int64_t)b * a.q_sb : nullptr;
+    for (int j = 4 - W; j < 3; ++j) {
+        const int64_t t = t_begin - 3 + j;
+        if (t >= 0) {
+            float v = load1<DT>(a.x, xo + t * a.x_sl);
+            if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            h[j] = v;
+            if (seq) qh[j] = seq[t * a.q_sl];
+        } else if (a.init && a.S_in + t >= 0) {
+            h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+        }
+    }
+    for (int64_t t = t_begin; t < t_end; ++t) {
+        const float xr = load1<DT>(a.x, xo + t * a.x_sl);
+        float xm = xr;
+        if (a.mask) xm = mul_round<DT>(xr, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+        float acc = bv;
+        if (seq) {
+            // inputs of another packed sequence enter as zeros
+            const int32_t qt = seq[t * a.q_sl];
+            if (W == 4) acc = fmaf(w[0], qh[0] == qt ? h[0] : 0.0f, acc);
+            if (W >= 3) acc = fmaf(w[1], qh[1] == qt ? h[1] : 0.0f, acc);
+            acc = fmaf(w[2], qh[2] == qt ? h[2] : 0.0f, acc);
+            acc = fmaf(w[3], xm, acc);
+            qh[0] = qh[1];
+            qh[1] = qh[2];
+            qh[2] = qt;
+        } else {
+            if (W == 4) acc = fmaf(w[0], h[0], acc);
+            if (W >= 3) acc = fmaf(w[1], h[1], acc);
+            acc = fmaf(w[2], h[2], acc);
+            acc = fmaf(w[3], xm, acc);
+        }
+        if (a.eager) {
+            acc = round_through<DT>(acc);
+            if (a.act) acc = round_through<DT>(silu_precise(acc));
+            if (a.res_mode == CANON_RESIDUAL_MASKED) acc += xm;
+            else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
+        } else {
+            acc = finish(acc, a.act, a.res_mode, xm, xr);
+        }
+        store1<DT>(a.out, oo + t * a.o_sl, acc);
+        h[0] = h[1];
+        h[1] = h[2];
+        h[2] = xm;
+    }
+    if (a.fin && ch == a.nseg - 1)
+        for (int slot = 0; slot < a.S_out; ++slot) capture_row_state<DT>(a, b, c, slot);
+}
+
+// ---------------------------------------------------------------------------
+// launch: pick the template instance for a plan
+// ---------------------------------------------------------------------------
+namespace {
+
+template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+{
+    const dim3 g(pl.grid), b(256);
+    switch (pl.U) {
+    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, NT>), g, b, 0, s, pl.args); break;
+    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, NT>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, NT>), g, b, 0, s, pl.args); break;
+    }
+}
+
+template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+}
+
+template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
+{
+    const bool mask = pl.args.mask != nullptr;
+    if (pl.args.seq) {   // only the channel-contiguous kernel is planned with seq_idx
+        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        return;
+    }
+    // the streaming (non-temporal) variants exist for width 4 only
+    if (W == 4 && pl.args.nt) {
+        if (mask) launch_fwd_vec<DT, W, true, W == 4>(pl, s);
+        else launch_fwd_vec<DT, W, false, W == 4>(pl, s);
+    } else {
+        if (mask) launch_fwd_vec<DT, W, true, false>(pl, s);
+        else launch_fwd_vec<DT, W, false, false>(pl, s);
+    }
+}
+
+template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.kind == FWD_GENERIC) {
+        hipLaunchKernelGGL((canon_fwd_generic_kernel<DT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        return;
+    }
+    switch (pl.args.W) {
+    case 2: launch_fwd_w<DT, 2>(pl, s); break;
+    case 3: launch_fwd_w<DT, 3>(pl, s); break;
+    default: launch_fwd_w<DT, 4>(pl, s); break;
+    }
+}
+
+template <int DT, bool MASK, bool NT>
+void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
+{
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(256), 0, s, m);
+}
+
+template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)
+{
+    if (!pp.single) {
+        for (int i = 0; i < pp.n; ++i)
+            if (pp.part[i].grid > 0) launch_fwd<DT>(pp.part[i], s);
+        return;
+    }
+    PartTable<FwdArgs> m;
+    memset(&m, 0, sizeof(m));
+    uint32_t first = 0;
+    bool mask = false, nt = false;
+    for (int i = 0; i < kMaxParts; ++i) {
+        m.first_block[i] = i < pp.n ? first : 0xFFFFFFFFu;
+        if (i < pp.n) {
+            m.part[i] = pp.part[i].args;
+            first += pp.part[i].grid;
+            mask = pp.part[i].args.mask != nullptr;
+            nt = pp.part[i].args.nt != 0;
+        }
+    }
+    if (mask) {
+        if (nt) launch_blc_parts<DT, true, true>(m, pp.grid, s);
+        else launch_blc_parts<DT, true, false>(m, pp.grid, s);
+    } else {
+        if (nt) launch_blc_parts<DT, false, true>(m, pp.grid, s);
+        else launch_blc_parts<DT, false, false>(m, pp.grid, s);
+    }
+}
+
+}  // namespace
+
+void launch_fwd(const FwdPlan &pl, int x_dtype, hipStream_t s)
+{
+    switch (x_dtype) {
+    case CANON_DTYPE_F32: launch_fwd<CANON_DTYPE_F32>(pl, s); break;
+    case CANON_DTYPE_BF16: launch_fwd<CANON_DTYPE_BF16>(pl, s); break;
+    default: launch_fwd<CANON_DTYPE_F16>(pl, s); break;
+    }
+}
+
+void launch_fwd_parts(const FwdPartsPlan &pp, int x_dtype, hipStream_t s)
+{
+    switch (x_dtype) {
+    case CANON_DTYPE_F32: launch_fwd_parts_t<CANON_DTYPE_F32>(pp, s); break;
+    case CANON_DTYPE_BF16: launch_fwd_parts_t<CANON_DTYPE_BF16>(pp, s); break;
+    default: launch_fwd_parts_t<CANON_DTYPE_F16>(pp, s); break;
+    }
+}
+
+}  // namespace canon

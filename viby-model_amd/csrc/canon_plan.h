@@ -1,0 +1,180 @@
+// Kernel argument blocks, launch plans and launcher entry points shared by the
+// translation units of libcanon_conv1d.so: canon_api.hip plans (pure host
+// code), canon_fwd.hip / canon_update.hip / canon_bwd.hip hold the kernels and
+// the functions that pick the template instance and launch it.
+#ifndef CANON_PLAN_H
+#define CANON_PLAN_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "canon_conv1d.h"
+
+// build-time tuning knob of the channel-contiguous prefill kernel
+#ifndef CANON_BLC_ROWS
+#define CANON_BLC_ROWS 8
+#endif
+
+namespace canon {
+
+// Division by a run-time constant as multiply-high and shifts (set up on the host).
+struct FastDiv {
+    uint32_t d, m, s1, s2;
+};
+
+// ---------------------------------------------------------------------------
+// kernel argument blocks (device copies of the validated ABI structs)
+// ---------------------------------------------------------------------------
+struct FwdArgs {
+    const char *x;
+    char *out;
+    const void *weight;
+    const void *bias;
+    const void *mask;
+    const void *init;
+    void *fin;
+    const int32_t *seq;
+    int64_t q_sb, q_sl;
+    int64_t x_sb, x_sc, x_sl;
+    int64_t o_sb, o_sc, o_sl;
+    int64_t w_sc, w_sk;
+    int64_t m_sb, m_sl;
+    int64_t i_sb, i_sc, i_ss;
+    int64_t f_sb, f_sc, f_ss;
+    uint32_t B, C, L;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt;
+    // launch geometry
+    uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
+    uint32_t nseg;      // bcl: segments per row       generic: time chunks per row
+    uint32_t chunk;     // generic: time steps per chunk
+    uint32_t ntasks;    // bcl: wave tasks   blc: blocks   generic: threads
+    uint32_t nblocks;   // blocks to launch
+    FastDiv div_nseg, div_C;
+    // blc: tiles
+    uint32_t nct, ntt;  // channel tiles per row, time tiles per sequence
+    FastDiv div_nct, div_ntt;
+};
+
+struct UpdArgs {
+    const char *x;
+    char *out;
+    char *state;
+    const void *weight;
+    const void *bias;
+    const void *tmask;
+    int64_t x_sb, x_sc, o_sb, o_sc;
+    int64_t s_sb, s_sc, s_ss;
+    int64_t w_sc, w_sk;
+    int64_t m_sb;
+    uint32_t B, C;
+    int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec, b_vec;
+    uint32_t nvec;      // channel vectors per batch row
+    uint32_t bgroups;   // batch groups (each thread walks nb batch rows)
+    uint32_t nb;
+    uint32_t nthreads;
+    FastDiv div_nvec;
+};
+
+struct BwdArgs {
+    const char *x;
+    const char *dy;
+    char *dx;
+    const void *weight;
+    const void *bias;
+    const void *mask;
+    float *partial;
+    float *dweight;
+    float *dbias;
+    int64_t x_sb, x_sc, x_sl;
+    int64_t g_sb, g_sc, g_sl;
+    int64_t d_sb, d_sc, d_sl;
+    int64_t w_sc, w_sk;
+    int64_t m_sb, m_sl;
+    uint32_t B, C, L;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_vec, b_pair, m_vec;
+    uint32_t nvec;      // channel groups per row (C / E)
+    uint32_t nchunk;    // time chunks per sequence
+    uint32_t chunk;     // time steps per chunk
+    uint32_t nthreads;
+    uint32_t nsets;     // partial sets = B * nchunk
+    uint32_t nct;       // blc: channel tiles per row
+    FastDiv div_nvec, div_nchunk, div_nct;
+};
+
+// Several channel ranges of one logical [B, C, L] problem that live in separate
+// tensors (q / k / v or gate / up projections), one launch: every block belongs
+// to one part and runs the single-tensor code on that part's argument block.
+constexpr int kMaxParts = CANON_CONV1D_MAX_PARTS;
+
+template <typename Args> struct PartTable {
+    Args part[kMaxParts];
+    uint32_t first_block[kMaxParts];   // first block of each part; 0xFFFFFFFF for unused slots
+};
+
+// ---------------------------------------------------------------------------
+// kernel geometry (needed by the planner and by the kernels)
+// ---------------------------------------------------------------------------
+constexpr int kBlcWaves = 4;   // waves (time slabs) per block
+constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 % faster than 16 (half the registers, twice the waves)
+constexpr int kBwdSlab = 8;    // time steps per wave and tile
+constexpr int kBwdWaves = 4;
+enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
+enum UpdKind { UPD_VEC, UPD_GENERIC };
+
+constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
+constexpr int kBlcRows = CANON_BLC_ROWS;   // time steps per wave in the channel-contiguous kernel
+constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
+constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work
+enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
+constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
+constexpr int kBwdHalfBlocksPerCU = 3;   // grid target of the channel-contiguous backward, in half blocks per CU
+
+// ---------------------------------------------------------------------------
+// launch plans: what the validated arguments of one call turn into
+// ---------------------------------------------------------------------------
+struct FwdPlan {
+    FwdKind kind;
+    int U;
+    FwdArgs args;
+    uint32_t grid;
+};
+
+struct UpdPlan {
+    UpdKind kind;
+    UpdArgs args;
+    uint32_t grid;
+};
+
+struct FwdPartsPlan {
+    int n;
+    bool single;            // one launch over a PartTable
+    uint32_t grid;          // of that launch
+    FwdPlan part[kMaxParts];
+};
+
+struct UpdPartsPlan {
+    int n;
+    bool single;
+    uint32_t grid;
+    UpdPlan part[kMaxParts];
+};
+
+struct BwdPlan {
+    BwdKind kind;
+    int U;
+    BwdArgs args;
+    uint32_t grid;
+    int64_t workspace_bytes;
+};
+
+// Launchers (x_dtype is a CANON_DTYPE_* code; nothing here synchronises)
+void launch_fwd(const FwdPlan &pl, int x_dtype, hipStream_t s);
+void launch_fwd_parts(const FwdPartsPlan &pp, int x_dtype, hipStream_t s);
+void launch_update(const UpdPlan &pl, int x_dtype, hipStream_t s);
+void launch_update_parts(const UpdPartsPlan &pp, int x_dtype, hipStream_t s);
+void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s);          // dx + partial sets, then the reduction
+void launch_zero(float *p, uint32_t n, hipStream_t s);                    // fill kernel (graph-capture safe)
+
+}  // namespace canon
+#endif  // CANON_PLAN_H

@@ -203,3 +203,31 @@ def test_unsupported_gradients_raise(cc):
         cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
     assert out.requires_grad and not fs.requires_grad
+
+
+def test_backward_more_than_2_31_elements(cc):
+    """Index arithmetic past 32 bits in the backward kernels: dx of a batch row inside a 2.26e9-element
+    call equals dx of that row differentiated alone (dx has no term across batch rows)."""
+    B, C, L = 64, 3456, 10240
+    g = torch.Generator(device=DEV).manual_seed(5)
+    w = (torch.randn(C, 4, generator=g, device=DEV) * 0.3).bfloat16().requires_grad_(True)
+    for layout in ("blc", "bcl"):
+        shape = (B, L, C) if layout == "blc" else (B, C, L)
+        x = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+        dout = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+        for b in range(B):
+            x[b].normal_(generator=g)
+            dout[b].normal_(generator=g)
+        if layout == "blc":
+            x, dout = x.transpose(1, 2), dout.transpose(1, 2)
+        x.requires_grad_(True)
+        cc.causal_conv1d_fn(x, w, activation="silu", residual=True).backward(dout)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(w.grad).all())
+        for b in (0, 40, 63):
+            xb = x[b:b + 1].detach().requires_grad_(True)
+            cc.causal_conv1d_fn(xb, w, activation="silu", residual=True).backward(dout[b:b + 1])
+            assert torch.equal(bits(x.grad[b:b + 1]), bits(xb.grad)), (layout, b)
+        w.grad = None
+        del x, dout
+        torch.cuda.empty_cache()

@@ -450,3 +450,35 @@ def test_seq_idx_constant_is_no_seq_idx(cc):
     a = cc.causal_conv1d_fn(x, w, seq_idx=seq, residual=True)
     b = cc.causal_conv1d_fn(x, w, residual=True)
     assert torch.equal(bits(a), bits(b))
+
+
+def test_more_than_2_31_elements(cc):
+    """Index arithmetic past 32 bits: 2.26e9 elements per tensor (4.5 GB of bf16).  The CPU oracle is
+    run on a few (batch, channel) rows only; the rest is covered by a size-independent property, a batch
+    row convolved alone gives the bits it has inside the big call."""
+    B, C, L = 64, 3456, 10240
+    assert B * C * L > 2 ** 31
+    g = torch.Generator(device=DEV).manual_seed(99)
+    w_cpu = (torch.randn(C, 4, generator=torch.Generator().manual_seed(98)) * 0.3).bfloat16()
+    w = w_cpu.to(DEV)
+    for layout in ("bcl", "blc"):
+        if layout == "bcl":
+            x = torch.empty(B, C, L, dtype=torch.bfloat16, device=DEV)
+        else:
+            x = torch.empty(B, L, C, dtype=torch.bfloat16, device=DEV).transpose(1, 2)
+        for b in range(B):
+            x[b].copy_(torch.randn(C, L, generator=g, device=DEV))
+        assert cc.kernel_plan_fwd(x, w) == f"{layout}_vec"
+        out, state = cc.causal_conv1d_fn(x, w, activation=None, residual=True, return_final_states=True)
+        torch.cuda.synchronize()
+        for b in (0, 31, 63):
+            alone, st = cc.causal_conv1d_fn(x[b:b + 1], w, residual=True, return_final_states=True)
+            assert torch.equal(bits(out[b:b + 1]), bits(alone)), (layout, b)
+            assert torch.equal(bits(state[b:b + 1]), bits(st)), (layout, b)
+        # the last rows in memory against the oracle
+        xs = x[B - 1:, C - 8:, :].contiguous().cpu()
+        want, want_state = co.conv1d_fwd(xs, w_cpu[C - 8:], None, residual=1, final_state_len=3)
+        assert torch.equal(bits(out[B - 1:, C - 8:, :]), bits(want)), layout
+        assert torch.equal(bits(state[B - 1:, C - 8:, :]), bits(want_state)), layout
+        del x, out, state
+        torch.cuda.empty_cache()

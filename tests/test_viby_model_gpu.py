@@ -10,7 +10,7 @@ from torch import nn
 from helpers import bits
 from oracle import canon_oracle as co
 from oracle.canon_eager import EagerCanon
-from viby_harness import VibyShaped, init_weights, viby_config
+from viby_harness import generate_graphed, VibyShaped, init_weights, viby_config
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -173,3 +173,39 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
               f"greedy tokens equal at {agree.float().mean().item() * 100:.1f} % of steps "
               f"({decided.float().mean().item() * 100:.1f} % decided beyond rounding noise), "
               f"max |dlogit| {diff.max().item():.4f} of scale {scale:.2f}")
+
+
+def test_config5_decode_as_one_hip_graph_per_token(capsys):
+    """The whole decode step of the 18-layer model (72 Canon update launches among everything else) captured
+    once and replayed for every generated token: bit-identical to the same step launched eagerly, same tokens
+    and logits as the growing-KV loop up to the attention kernel's rounding (it runs over a fixed-length KV
+    buffer here), and the time it takes."""
+    cfg = viby_config()
+    B, T, steps = 16, 1024, 128
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(5)).to(DEV)
+    model = init_weights(VibyShaped(cfg, hip_factory(cfg, "fused")), 11, torch.bfloat16, DEV)
+    model.generate(ids[:2, :64], 2)
+    generate_graphed(model, ids[:2, :64], 3)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    toks_e, logits_e, _ = model.generate(ids, steps)
+    torch.cuda.synchronize()
+    t_eager = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    toks_g, logits_g = generate_graphed(model, ids, steps)
+    torch.cuda.synchronize()
+    t_graph = time.perf_counter() - t0
+    # the same step function launched kernel by kernel: the replays must reproduce it bit for bit
+    toks_s, logits_s = generate_graphed(model, ids, steps, capture=False)
+    assert torch.equal(toks_s, toks_g) and torch.equal(logits_s, logits_g)
+    assert torch.equal(logits_e[0], logits_g[0])                     # the prefill is the same code
+    # teacher-forced comparison is not possible inside a graph: compare up to the first diverging token
+    same = (toks_e == toks_g).all(dim=0).int().cumprod(0).sum().item()
+    assert same >= 4, same
+    diff = (logits_e[:same + 1] - logits_g[:same + 1]).abs().max().item()
+    scale = logits_e.abs().max().item()
+    assert diff <= 0.05 * scale, (diff, scale)
+    with capsys.disabled():
+        print(f"\n[config 5, graph-captured decode] B{B} x L{T} prefill + {steps} greedy steps: eager loop {t_eager:.2f} s, "
+              f"one HIP graph per token {t_graph:.2f} s; first {same} of {steps} steps identical for every sequence, "
+              f"max |dlogit| {diff:.4f} of scale {scale:.2f} over them")

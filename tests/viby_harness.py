@@ -75,15 +75,28 @@ class Block(nn.Module):
         q = q.reshape(B, T, self.nq, self.hd).transpose(1, 2)
         k = k.reshape(B, T, self.nkv, self.hd).transpose(1, 2)
         v = v.reshape(B, T, self.nkv, self.hd).transpose(1, 2)
-        pos = torch.arange(pos0, pos0 + T, device=h.device)
-        q, k = rotary(q, pos, self.theta), rotary(k, pos, self.theta)
-        if cache.kv[layer_idx] is not None:
-            pk, pv = cache.kv[layer_idx]
-            k, v = torch.cat([pk, k], dim=2), torch.cat([pv, v], dim=2)
-        cache.kv[layer_idx] = (k, v)
         rep = self.nq // self.nkv
-        att = F.scaled_dot_product_attention(q, k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1),
-                                             is_causal=(T > 1))
+        if getattr(cache, "static_kv", None) is not None:
+            # decode step over preallocated K / V (shapes never change, so the step can be captured as a HIP
+            # graph): the position lives in a device tensor, the new row is written in place, and attention
+            # runs over the whole buffer with the rows beyond the position masked out
+            pos = cache.pos_t + torch.arange(T, device=h.device)
+            q, k = rotary(q, pos, self.theta), rotary(k, pos, self.theta)
+            K, V = cache.static_kv[layer_idx]
+            K.index_copy_(2, pos, k)
+            V.index_copy_(2, pos, v)
+            seen = torch.arange(K.shape[2], device=h.device)[None, None, None, :] <= cache.pos_t
+            att = F.scaled_dot_product_attention(q, K.repeat_interleave(rep, dim=1), V.repeat_interleave(rep, dim=1),
+                                                 attn_mask=seen)
+        else:
+            pos = torch.arange(pos0, pos0 + T, device=h.device)
+            q, k = rotary(q, pos, self.theta), rotary(k, pos, self.theta)
+            if cache.kv[layer_idx] is not None:
+                pk, pv = cache.kv[layer_idx]
+                k, v = torch.cat([pk, k], dim=2), torch.cat([pv, v], dim=2)
+            cache.kv[layer_idx] = (k, v)
+            att = F.scaled_dot_product_attention(q, k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1),
+                                                 is_causal=(T > 1))
         h = h + self.o_proj(att.transpose(1, 2).reshape(B, T, self.nq * self.hd))
         x = self.canon_c(self.post_attention_layernorm(h), attention_mask=mask, cache=cache, layer_idx=layer_idx)
         gate, up = self.gate_proj(x), self.up_proj(x)
@@ -132,6 +145,72 @@ class VibyShaped(nn.Module):
             if s + 1 < steps:
                 logits.append(self.forward(nxt[:, None], cache, mask))
         return torch.stack(toks, dim=1), torch.stack(logits), cache
+
+
+@torch.no_grad()
+def generate_graphed(model: VibyShaped, ids: torch.Tensor, steps: int, capture: bool = True):
+    """Prefill eagerly, then ONE captured HIP graph per generated token (all layers: 72 Canon update launches,
+    projections, attention over a preallocated KV buffer, head, argmax, feeding the token back), replayed
+    steps-1 times without any host work in between.  With capture=False the same step function is called
+    eagerly instead (same kernels, launched one by one): the reference the replays must match bit for bit.
+    Returns (tokens [B, steps], logits [steps, B, V])."""
+    dev = ids.device
+    B, T = ids.shape
+    n = model.cfg.num_hidden_layers
+    cache = model.new_cache()
+    mask = torch.ones(B, T, dtype=torch.int64, device=dev)
+    logits0 = model.forward(ids, cache, mask)
+    # move the prefill's K / V into buffers of the final length
+    cache.static_kv = []
+    for k, v in cache.kv:
+        K = torch.zeros(k.shape[0], k.shape[1], T + steps, k.shape[3], dtype=k.dtype, device=dev)
+        V = torch.zeros_like(K)
+        K[:, :, :T].copy_(k)
+        V[:, :, :T].copy_(v)
+        cache.static_kv.append((K, V))
+    cache.kv = [None] * n
+    cache.pos_t = torch.tensor([T], device=dev)
+    tok = logits0.argmax(dim=-1)[:, None].clone()       # static input of the step
+    one = torch.ones(B, 1, dtype=torch.int64, device=dev)  # mask column of the new token
+    out_logits = torch.empty_like(logits0)
+
+    def step():
+        lg = model.forward(tok, cache, one)
+        out_logits.copy_(lg)
+        tok.copy_(lg.argmax(dim=-1)[:, None])
+        cache.pos_t.add_(1)
+
+    # warm-up on a side stream (library handles, allocator), then put every carried state back
+    sites = [name for name in ("a", "b", "c", "d") if hasattr(cache, f"canon_cache_{name}")]
+    saved = {name: [t.clone() for t in getattr(cache, f"canon_cache_{name}")] for name in sites}
+    tok0 = tok.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for name in sites:
+        for t, old in zip(getattr(cache, f"canon_cache_{name}"), saved[name]):
+            t.copy_(old)
+    tok.copy_(tok0)
+    cache.pos_t.fill_(T)
+
+    graph = None
+    if capture:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+    toks, logits = [tok0[:, 0].clone()], [logits0]
+    for _ in range(steps - 1):
+        if capture:
+            graph.replay()
+        else:
+            step()
+        logits.append(out_logits.clone())
+        toks.append(tok[:, 0].clone())
+    torch.cuda.synchronize()
+    return torch.stack(toks, dim=1), torch.stack(logits)
 
 
 def init_weights(model: nn.Module, seed: int, dtype, device) -> nn.Module:

@@ -356,20 +356,20 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 }
 
 template <int DT, int W, int R, bool MASK, bool NT>
-__global__ __launch_bounds__(256) void canon_fwd_blc_kernel(const FwdArgs a)
+__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_kernel(const FwdArgs a)
 {
     blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
 }
 
 // the same over packed variable-length sequences (seq_idx)
 template <int DT, int W, int R, bool MASK>
-__global__ __launch_bounds__(256) void canon_fwd_blc_seq_kernel(const FwdArgs a)
+__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_seq_kernel(const FwdArgs a)
 {
     blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
 template <int DT, int W, int R, bool MASK, bool NT>
-__global__ __launch_bounds__(256) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
+__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
 {
     const uint32_t p = part_of_block(m, blockIdx.x);
     blc_block<DT, W, R, MASK, NT>(m.part[p], blockIdx.x - m.first_block[p]);
@@ -479,15 +479,15 @@ template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, 
 template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
 {
     if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
-    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
 }
 
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 {
     const bool mask = pl.args.mask != nullptr;
     if (pl.args.seq) {   // only the channel-contiguous kernel is planned with seq_idx
-        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(256), 0, s, pl.args);
-        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
         return;
     }
     // the streaming (non-temporal) variants exist for width 4 only
@@ -516,7 +516,7 @@ template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
 template <int DT, bool MASK, bool NT>
 void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(256), 0, s, m);
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(64 * kBlcWaves), 0, s, m);
 }
 
 template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)

@@ -115,7 +115,10 @@ template <typename Args> struct PartTable {
 // ---------------------------------------------------------------------------
 // kernel geometry (needed by the planner and by the kernels)
 // ---------------------------------------------------------------------------
-constexpr int kBlcWaves = 4;   // waves (time slabs) per block
+#ifndef CANON_BLC_WAVES
+#define CANON_BLC_WAVES 4
+#endif
+constexpr int kBlcWaves = CANON_BLC_WAVES;   // waves (time slabs) per block
 constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 % faster than 16 (half the registers, twice the waves)
 constexpr int kBwdSlab = 8;    // time steps per wave and tile
 constexpr int kBwdWaves = 4;

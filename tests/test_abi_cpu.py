@@ -97,8 +97,11 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
         assert plan(fwd_params(C=C, layout="bcl")) == "bcl_vec"
         assert plan(fwd_params(C=C, layout="blc")) == "blc_vec"
     assert plan(fwd_params(B=1, C=640, L=1024, dtype=0)) == "bcl_vec"     # BASELINE config 1
-    # ragged sizes, misalignment, eager rounding -> strided kernel
-    assert plan(fwd_params(L=1023)) == "generic"
+    # time-contiguous rows that are not a whole number of vectors keep the vector kernel (edge elements aside)
+    # as long as x and out share their strides
+    assert plan(fwd_params(L=1023)) == "bcl_vec"
+    assert plan(fwd_params(L=1023, out_stride_c=1024, out_stride_b=3456 * 1024)) == "generic"
+    # ragged channel counts, misaligned base pointers, eager rounding -> strided kernel
     assert plan(fwd_params(C=3457, layout="blc")) == "generic"
     assert plan(fwd_params(x=FAKE_X + 2)) == "generic"
     assert plan(fwd_params(round_mode=1)) == "generic"

@@ -482,3 +482,32 @@ def test_more_than_2_31_elements(cc):
         assert torch.equal(bits(state[B - 1:, C - 8:, :]), bits(want_state)), layout
         del x, out, state
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_time_contiguous_rows_off_the_16_byte_grid(cc, dtype):
+    """Row lengths that are not a multiple of the vector size: every row starts at a different misalignment,
+    the aligned middle takes the vector code, the few elements around it are computed one per lane."""
+    g = torch.Generator().manual_seed(91)
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    for (B, C, L), W in itertools.product([(2, 24, 16 * E + 1), (3, 7, 1023), (1, 40, 16 * E + E - 1), (2, 5, 2049),
+                                           (2, 16, 700)], [2, 3, 4]):
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, W, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+        init = torch.randn(B, C, 5, generator=g).to(dtype)
+        for act, res, m, st in [(None, False, None, False), ("silu", "masked", mask, True), (None, "unmasked", mask, False),
+                                ("silu", True, None, True)]:
+            want = co.conv1d_fwd(x, w, b, mask=m, activation=act, residual=res,
+                                 initial_state=init if st else None, final_state_len=8 if st else None)
+            xg = x.to(DEV)
+            assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec", (B, C, L)
+            got = run_fwd(cc, xg, w, b, act=act, mask=m, residual=res, init=init if st else None, S_out=8 if st else None)
+            what = f"edge/{dtype}/{B}x{C}x{L}/W{W}/{act}/{res}/mask{m is not None}/state{st}"
+            xm = x if m is None else (x.float() * m[:, None, :].float()).to(dtype)
+            if st:
+                assert_parity(got[0], want[0], exact=act is None, what=what, res=xm if res else None)
+                assert torch.equal(bits(got[1]), bits(want[1])), what
+            else:
+                assert_parity(got, want, exact=act is None, what=what, res=xm if res else None)

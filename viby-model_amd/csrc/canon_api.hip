@@ -119,6 +119,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
+    plan->edge = false;
     plan->grid = 0;
     plan->kind = FWD_GENERIC;
     if (empty) return CANON_OK;
@@ -130,9 +131,12 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
     // packed sequences: the channel-contiguous kernel has a variant (the index is uniform per time row);
     // time-contiguous rows take the strided kernel
-    const bool bcl_ok = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L % E == 0 &&
-                        a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0 &&
-                        a.L / E >= 16;
+    const bool bcl_rows = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L / E >= 16;
+    // every row starts on a 16-byte boundary and is a whole number of vectors ...
+    const bool bcl_aligned = a.L % E == 0 && a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0;
+    // ... or x and out share one geometry, so that a row is misaligned by the same amount in both
+    const bool bcl_edge = !bcl_aligned && a.x_sb == a.o_sb && a.x_sc == a.o_sc && a.x_sb >= 0 && a.x_sc >= 0;
+    const bool bcl_ok = bcl_rows && (bcl_aligned || bcl_edge);
     const uint32_t EB = kBlcVecBytes / elem_bytes(p->x_dtype);   // channels per lane of the channel-contiguous kernel
     const bool ptr8_ok = (((uintptr_t)p->x | (uintptr_t)p->out) & (kBlcVecBytes - 1)) == 0;
     const bool blc_ok = fused && ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
@@ -141,17 +145,20 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
 
     if (bcl_ok) {
         const uint32_t nvec = a.L / E;
-        // vectors per lane: as many as keep >= 2048 waves in flight, at most 4
+        // vectors per lane (1, 2 or 4): the largest that leaves no more lane slots idle than one vector
+        // per lane would and still keeps >= 2048 waves in flight
         int U = 1;
+        const uint64_t slots1 = (nvec + 63u) / 64u;
         for (int cand = 2; cand <= 4; cand *= 2) {
             const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
-            if (nvec >= 64u * cand && rows * nseg >= 2048) U = cand;
+            if (nseg * cand <= slots1 && rows * nseg >= 2048) U = cand;
         }
         const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
         const uint64_t ntasks = rows * nseg;
         if (ntasks < (1ull << 31)) {
             plan->kind = FWD_BCL;
             plan->U = U;
+            plan->edge = !bcl_aligned;
             a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
             a.div_nseg = make_fastdiv(a.nseg); a.div_C = make_fastdiv(a.C);
             a.nblocks = (uint32_t)((ntasks + 3) / 4);

@@ -7,15 +7,17 @@ namespace canon {
 // ---------------------------------------------------------------------------
 // backward of the prefill: dx, and per-chunk partial sums of dweight / dbias
 //
-// One lane owns E channels and walks a chunk of time steps from its END to its
-// start: dx[t] needs dz[t .. t+W-1] (the three later steps are carried in
-// registers), z[t] needs xm[t-3 .. t] (a sliding window refilled with one row
-// per step, fetched R rows ahead).  The three dz values just past the chunk are
-// recomputed from memory.  dweight / dbias accumulate in registers over the
-// chunk and go to partial[(b * nchunk + chunk) * C + c][5] (w0..w3, bias);
-// canon_bwd_reduce_kernel sums the partial sets in a fixed order.
-//   VEC:  channel-contiguous tensors, E = elements per 16 bytes, vector access
-//   !VEC: E = 1, any strides (the fallback for every other layout)
+// Every kernel of this file writes dx and one entry per channel of a partial
+// set, partial[(b * nchunk + chunk) * C + c][5] (w0..w3, bias);
+// canon_bwd_reduce_kernel sums the sets in a fixed order.
+//
+// canon_bwd_walk_kernel, the fallback for layouts without a vector kernel
+// (instantiated with E = 1, VEC = false: any strides): one lane owns a channel
+// and walks a chunk of time steps from its END to its start.  dx[t] needs
+// dz[t .. t+W-1] (the three later steps are carried in registers), z[t] needs
+// xm[t-3 .. t] (a sliding window refilled with one row per step, fetched R
+// rows ahead).  The three dz values just past the chunk are recomputed from
+// memory.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float silu_grad(float z)
 {
@@ -839,8 +841,18 @@ __global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *part
     const uint32_t ncols = C * 5u;
     const uint32_t i = blockIdx.x * 32u + col;   // (c, j), j in 0..4
     double acc = 0.0;
-    if (i < ncols)
-        for (uint32_t s = slice; s < nsets; s += 8u) acc += (double)partial[(int64_t)s * ncols + i];
+    if (i < ncols) {
+        uint32_t s = slice;
+        for (; s + 24u < nsets; s += 32u) {   // four loads in flight, added in set order
+            const float v0 = partial[(int64_t)s * ncols + i], v1 = partial[(int64_t)(s + 8u) * ncols + i];
+            const float v2 = partial[(int64_t)(s + 16u) * ncols + i], v3 = partial[(int64_t)(s + 24u) * ncols + i];
+            acc += (double)v0;
+            acc += (double)v1;
+            acc += (double)v2;
+            acc += (double)v3;
+        }
+        for (; s < nsets; s += 8u) acc += (double)partial[(int64_t)s * ncols + i];
+    }
     part[slice][col] = acc;
     __syncthreads();
     if (slice != 0 || i >= ncols) return;

@@ -31,7 +31,68 @@ namespace canon {
 // unmasked path is ~130 VALU instructions per 2 KB row and hides under the
 // memory time.
 // ---------------------------------------------------------------------------
-template <int DT, int W, int U, bool MASK, bool NT>
+// One element of the row computed on its own (the few elements of a row that do not fill an aligned
+// 16-byte vector, see EDGE below): scalar loads of its window, same arithmetic.  The loads are
+// issued with the row's vector loads (bcl_edge_issue) and consumed after the vector work
+// (bcl_edge_finish), so they cost the wave no round trip of their own.
+struct EdgeWindow {
+    float x[4];   // raw x[t-3 .. t] (0 where t-3+k < 0 and there is no initial state)
+    float m[4];   // their mask entries
+};
+
+template <int DT, int W, bool MASK>
+__device__ __forceinline__ void bcl_edge_issue(const FwdArgs &a, const char *xrow, uint32_t b, uint32_t c, int64_t t,
+                                               EdgeWindow &e)
+{
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        e.x[k] = 0.0f;
+        e.m[k] = 1.0f;
+    }
+#pragma unroll
+    for (int k = 4 - W; k < 4; ++k) {
+        const int64_t tt = t - 3 + k;
+        if (tt >= 0) e.x[k] = load1<DT>(xrow, tt);
+        else if (a.init) e.x[k] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + tt) * a.i_ss);
+    }
+    if constexpr (MASK) {
+        // the four entries as one run from max(t-3, 0) (rows are at least 16 vectors long)
+        const int64_t first = t - 3 > 0 ? t - 3 : 0;
+        const int shift = (int)(first - (t - 3));   // 0 .. 3 window slots lie before the row
+        int64_t base[1] = {b * a.m_sb + first * a.m_sl};
+        float run[1][4];
+        load_mask_vec<4, 1>(a.mask, base, a.m_sl, a.mask_dtype, false, run);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int j = k - shift;
+            e.m[k] = j == 0 ? run[0][0] : j == 1 ? run[0][1] : j == 2 ? run[0][2] : j == 3 ? run[0][3] : 1.0f;
+        }
+    }
+}
+
+template <int DT, int W, bool MASK>
+__device__ __forceinline__ void bcl_edge_finish(const FwdArgs &a, const float (*w)[W], float bv, char *orow, int64_t t,
+                                                const EdgeWindow &e)
+{
+    float win[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        win[k] = e.x[k];
+        if constexpr (MASK) {
+            if (t - 3 + k >= 0) win[k] = mul_round<DT>(e.x[k], e.m[k]);   // history from the initial state is not masked
+        }
+    }
+    float acc = bv;
+#pragma unroll
+    for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], win[(4 - W) + k], acc);
+    store1<DT>(orow, t, finish(acc, a.act, a.res_mode, win[3], e.x[3]));
+}
+
+// EDGE: the rows are contiguous in time but do not start on 16-byte boundaries (a length or a
+// row stride that is not a multiple of E).  The aligned middle of every row runs through the
+// same vector code, shifted by `head` elements; the up to E-1 elements before it and after it
+// are computed one per lane by the waves that own the first and the last segment.
+template <int DT, int W, int U, bool MASK, bool NT, bool EDGE = false>
 __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
@@ -46,9 +107,19 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     const uint32_t b = fdiv(row, a.div_C);
     const uint32_t c = row - b * a.C;
 
-    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
+    const int64_t row_off = (int64_t)b * a.x_sb + (int64_t)c * a.x_sc;   // in elements; the same for x and out
+    const char *xrow = a.x + row_off * Elem<DT>::bytes;
     char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
     const uint32_t v0 = seg * (64u * U) + lane;
+    // head: elements of the row before its first aligned vector; nvec: aligned vectors of this row
+    uint32_t head = 0, nvec = a.nvec;
+    if constexpr (EDGE) {
+        head = (uint32_t)((E - (row_off % E)) % E);
+        if (head > a.L) head = a.L;
+        nvec = (a.L - head) / E;
+    }
+    const char *xvec = xrow + (int64_t)head * Elem<DT>::bytes;   // 16-byte aligned
+    char *ovec = orow + (int64_t)head * Elem<DT>::bytes;
 
     // row data first (the long latency), then the taps (scalar-cache hits)
     uint4 X[U];
@@ -56,7 +127,18 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     for (int u = 0; u < U; ++u) {
         const uint32_t v = v0 + u * 64u;
         X[u] = make_uint4(0, 0, 0, 0);
-        if (v < a.nvec) X[u] = load_vec<NT>(xrow + (int64_t)v * 16);
+        if (v < nvec) X[u] = load_vec<NT>(xvec + (int64_t)v * 16);
+    }
+
+    // EDGE: lanes 0 .. head-1 of the first segment take the elements before the first vector,
+    // lanes 32 .. 32+tail-1 of the last segment the elements after the last one
+    EdgeWindow edge;
+    int64_t edge_t = -1;
+    if constexpr (EDGE) {
+        const uint32_t tail = a.L - head - nvec * E;
+        if (seg == 0 && (uint32_t)lane < head) edge_t = lane;
+        if (seg == a.nseg - 1 && lane >= 32 && (uint32_t)(lane - 32) < tail) edge_t = (int64_t)head + (int64_t)nvec * E + (lane - 32);
+        if (edge_t >= 0) bcl_edge_issue<DT, W, MASK>(a, xrow, b, c, edge_t, edge);
     }
 
     RawTaps<1> raw;
@@ -69,9 +151,14 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t v = v0 + u * 64u;
-            mbase[u] = b * a.m_sb + (int64_t)(v < a.nvec ? v : a.nvec - 1u) * E * a.m_sl;   // idle lanes shadow the last vector
+            // idle lanes shadow the last vector (a row without any aligned vector reads from its start)
+            const int64_t vv = v < nvec ? v : (nvec ? nvec - 1u : 0u);
+            mbase[u] = b * a.m_sb + ((int64_t)head + vv * E) * a.m_sl;
+            if constexpr (EDGE) {
+                if (nvec == 0) mbase[u] = b * a.m_sb;
+            }
         }
-        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+        load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, !EDGE && a.m_vec != 0, M);
     }
 
     float w[1][W], bvv[1];
@@ -81,14 +168,19 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     // history of the segment's first vector (only lane 0's copy is consumed)
     float carry[3] = {0.0f, 0.0f, 0.0f};
     if (lane == 0) {
-        if (seg > 0) {
-            const int64_t t0 = (int64_t)v0 * E;
+        if (seg > 0 || (EDGE && head > 0)) {
+            const int64_t t0 = (int64_t)head + (int64_t)v0 * E;
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
-                float v = load1<DT>(xrow, t0 - 3 + j);
-                if constexpr (MASK)
-                    v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + (t0 - 3 + j) * a.m_sl, a.mask_dtype));
-                carry[j] = v;
+                const int64_t t = t0 - 3 + j;
+                if (j < 3 - (W - 1)) continue;
+                if (t >= 0) {
+                    float v = load1<DT>(xrow, t);
+                    if constexpr (MASK) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+                    carry[j] = v;
+                } else if (a.init) {
+                    carry[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+                }
             }
         } else if (a.init) {
 #pragma unroll
@@ -140,7 +232,11 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 #pragma unroll
             for (int j = 0; j < E; ++j) o[j] += xm[j];
         }
-        if (v < a.nvec) store_vec<NT>(orow + (int64_t)v * 16, pack_vec<DT>(o));
+        if (v < nvec) store_vec<NT>(ovec + (int64_t)v * 16, pack_vec<DT>(o));
+    }
+
+    if constexpr (EDGE) {
+        if (edge_t >= 0) bcl_edge_finish<DT, W, MASK>(a, w, bv, orow, edge_t, edge);
     }
 
     if (a.fin && seg == a.nseg - 1) capture_row_state<DT>(a, b, c, lane);
@@ -466,14 +562,20 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
 // ---------------------------------------------------------------------------
 namespace {
 
-template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+template <int DT, int W, bool MASK, bool NT, bool EDGE> void launch_bcl_e(const FwdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
     switch (pl.U) {
-    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, NT>), g, b, 0, s, pl.args); break;
-    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, NT>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, NT>), g, b, 0, s, pl.args); break;
+    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
+    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
     }
+}
+
+template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+{
+    if (pl.edge) launch_bcl_e<DT, W, MASK, NT, true>(pl, s);
+    else launch_bcl_e<DT, W, MASK, NT, false>(pl, s);
 }
 
 template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)

@@ -139,6 +139,7 @@ constexpr int kBwdHalfBlocksPerCU = 3;   // grid target of the channel-contiguou
 struct FwdPlan {
     FwdKind kind;
     int U;
+    bool edge;   // bcl: rows do not start on 16-byte boundaries
     FwdArgs args;
     uint32_t grid;
 };

@@ -131,7 +131,9 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
     // packed sequences: the channel-contiguous kernel has a variant (the index is uniform per time row);
     // time-contiguous rows take the strided kernel
-    const bool bcl_rows = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L / E >= 16;
+    // shorter rows leave most of a wave idle: measured slower than the strided kernel below 16 vectors
+    const uint32_t kBclMinVectors = 16;
+    const bool bcl_rows = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L / E >= kBclMinVectors;
     // every row starts on a 16-byte boundary and is a whole number of vectors ...
     const bool bcl_aligned = a.L % E == 0 && a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0;
     // ... or x and out share one geometry, so that a row is misaligned by the same amount in both

@@ -464,50 +464,32 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         for (int k = 0; k < W; ++k) dw[e][k] = 0.0f;
     }
 
-    // rows of x and dout, the three rows of x before the slab (first wave) and the mask entries of one tile;
-    // requested one tile ahead, so that they arrive while the tile before is being computed
-    uint2 Xn[R], Gn[R], Hn[3];
-    float mmn[R + 3];   // mask of steps t0-3 .. t0+R-1
-    auto request = [&](int it) {
-        const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
-            Xn[r] = *(const uint2 *)(xb + t * xs);
-            Gn[r] = *(const uint2 *)(gb + t * gs);
-        }
-#pragma unroll
-        for (int j = 0; j < 3; ++j) Hn[j] = make_uint2(0, 0);
-        if (wv == 0) {
-#pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                const int64_t t = t0 - 3 + j;
-                if (t >= 0) Hn[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < R + 3; ++j) mmn[j] = 1.0f;
-        if constexpr (MASK) load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mmn);
-    };
-    request(ntiles - 1);
-
     for (int it = ntiles - 1; it >= 0; --it) {
         const int64_t t0 = t_chunk + ((int64_t)it * NW + wv) * R;
         const int64_t left = (int64_t)a.L - t0;
         const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
 
+        // ---- all loads of the tile (issuing them one tile ahead was measured: no gain, 14 more registers)
         uint2 X[R], G[R], H[3];
-        float mm[R + 3];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            X[r] = Xn[r];
-            G[r] = Gn[r];
+            const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
+            X[r] = *(const uint2 *)(xb + t * xs);
+            G[r] = *(const uint2 *)(gb + t * gs);
         }
 #pragma unroll
-        for (int j = 0; j < 3; ++j) H[j] = Hn[j];
+        for (int j = 0; j < 3; ++j) H[j] = make_uint2(0, 0);
+        if (wv == 0) {
 #pragma unroll
-        for (int j = 0; j < R + 3; ++j) mm[j] = mmn[j];
-        if (it > 0) request(it - 1);
+            for (int j = 0; j < 3; ++j) {
+                const int64_t t = t0 - 3 + j;
+                if (t >= 0) H[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+            }
+        }
+        float mm[R + 3];   // mask of steps t0-3 .. t0+R-1
+#pragma unroll
+        for (int j = 0; j < R + 3; ++j) mm[j] = 1.0f;
+        if constexpr (MASK) load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mm);
 
         // dz of the three steps after the slab; the last wave's are the previous iteration's head of wave 0
         float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed

@@ -120,7 +120,10 @@ template <typename Args> struct PartTable {
 #endif
 constexpr int kBlcWaves = CANON_BLC_WAVES;   // waves (time slabs) per block
 constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 % faster than 16 (half the registers, twice the waves)
-constexpr int kBwdSlab = 8;    // time steps per wave and tile
+#ifndef CANON_BWD_SLAB
+#define CANON_BWD_SLAB 8
+#endif
+constexpr int kBwdSlab = CANON_BWD_SLAB;    // time steps per wave and tile
 constexpr int kBwdWaves = 4;
 enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };

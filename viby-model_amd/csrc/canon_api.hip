@@ -486,7 +486,7 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         // time steps per block: as long as possible (few partial sets to write and to add up, taps and
         // chunk-end work amortised) while the grid still has one and a half blocks per CU
         uint32_t chunk = tile;
-        for (uint32_t cand = 2 * tile; cand <= 32 * tile; cand *= 2) {
+        for (uint32_t cand = 2 * tile; cand <= (uint32_t)kBwdMaxChunk; cand *= 2) {
             const uint64_t blocks = (uint64_t)a.B * ((a.L + cand - 1) / cand) * nct;
             if (2 * blocks >= 256ull * kBwdHalfBlocksPerCU) chunk = cand;
         }

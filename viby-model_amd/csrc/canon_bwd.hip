@@ -273,6 +273,8 @@ __device__ __forceinline__ uint2 bwd_mask_row(const uint2 &raw, float m, bool ex
 {
     uint2 v = raw;
     if constexpr (MASK) {
+      // m is the same for the whole wave and 1 for every valid token of a padded batch: x * 1 is x, bit for bit
+      if (m != 1.0f) {
         if constexpr (DT == CANON_DTYPE_F32) {
             v.x = f_bits(bits_f(raw.x) * m);
             v.y = f_bits(bits_f(raw.y) * m);
@@ -286,6 +288,7 @@ __device__ __forceinline__ uint2 bwd_mask_row(const uint2 &raw, float m, bool ex
             }
             v = pack_half<DT>(f);
         }
+      }
     }
     if (!exists) v = make_uint2(0, 0);
     return v;
@@ -357,8 +360,10 @@ __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W],
             for (int e = 0; e < E; ++e) o[e] += g[e];
         }
         if constexpr (MASK) {
+            if (mm[3 + r] != 1.0f) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) o[e] *= mm[3 + r];
+                for (int e = 0; e < E; ++e) o[e] *= mm[3 + r];
+            }
         }
         if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
 #pragma unroll
@@ -387,6 +392,10 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     __shared__ uint2 tailx[NW][3][64];            // last three xm rows of each wave's slab (storage bits)
     __shared__ float headdz[NW][3][E][64];        // dz of the first three steps of each wave's slab
     __shared__ float red[NW - 1][5 * E][64];      // dweight / dbias sums of waves 1..3
+    // mask entries of steps t_chunk-3 .. t_chunk+chunk+2 as floats.  Staged once per block: inside the
+    // time loop (after the first store to dx) the compiler can no longer use scalar loads for them, and
+    // as vector loads in the tile's load group they cost 20 % of the kernel.
+    __shared__ float smask[MASK ? kBwdMaxChunk + 6 : 1];
 
     // blockIdx = (b * nchunk + ch) * nct + ct : channel tile fastest, i.e. memory order
     const uint32_t bc = fdiv(blockIdx.x, a.div_nct);
@@ -410,6 +419,14 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     RawTaps<E> rawt;
     fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, rawt);
     float w[E][W], bias[E];
+    if constexpr (MASK) {
+        for (uint32_t i = threadIdx.x; i < a.chunk + 6u; i += 64u * NW) {
+            int64_t t = t_chunk - 3 + (int64_t)i;
+            t = t < 0 ? 0 : (t > Lm1 ? Lm1 : t);
+            smask[i] = load_mask(a.mask, (int64_t)b * a.m_sb + t * a.m_sl, a.mask_dtype);
+        }
+        __syncthreads();
+    }
 
     // The tiles are walked from the last to the first, so the dz of the three steps after a tile
     // are the head of the tile done just before (still in headdz[0]).  For the chunk's last tile
@@ -437,7 +454,10 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
                 const int64_t t = te + j;
                 GE[j] = *(const uint2 *)(gb + (t < Lm1 ? t : Lm1) * gs);
             }
-            if constexpr (MASK) load_mask_rows<6>(a.mask, (int64_t)b * a.m_sb, te - 3, a.L, a.m_sl, a.mask_dtype, me);
+            if constexpr (MASK) {
+#pragma unroll
+                for (int j = 0; j < 6; ++j) me[j] = smask[a.chunk + j];   // steps te-3 .. te+2
+            }
         }
         decode_taps<DT, W, E>(rawt, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
         if (wv == NW - 1) {
@@ -489,7 +509,11 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         float mm[R + 3];   // mask of steps t0-3 .. t0+R-1
 #pragma unroll
         for (int j = 0; j < R + 3; ++j) mm[j] = 1.0f;
-        if constexpr (MASK) load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mm);
+        if constexpr (MASK) {
+            const uint32_t first = ((uint32_t)it * NW + wv) * R;   // index of step t0 - 3 in smask
+#pragma unroll
+            for (int j = 0; j < R + 3; ++j) mm[j] = smask[first + j];
+        }
 
         // dz of the three steps after the slab; the last wave's are the previous iteration's head of wave 0
         float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed

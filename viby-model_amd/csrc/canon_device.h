@@ -173,10 +173,51 @@ __device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
 // and every case is straight-line code, so all N loads are issued back to back
 // and waited for once (a per-entry switch puts a wait after every load, which
 // also waits for -- and so serialises -- the row loads issued before it).
+template <int N, bool RUN>
+__device__ __forceinline__ void load_mask_entries(const void *p, int64_t first, const int64_t *idx, int dt, float *m)
+{
+    // RUN: the entries are first, first+1, .. (constant offsets: the loads merge); else idx[j]
+    switch (dt) {
+    case CANON_MASK_U8:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[RUN ? first + j : idx[j]];
+        break;
+    case CANON_MASK_I32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[RUN ? first + j : idx[j]];
+        break;
+    case CANON_MASK_I64: {
+        uint2 q[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) q[j] = ((const uint2 *)p)[RUN ? first + j : idx[j]];
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = i64_words_to_float(q[j].x, q[j].y);
+        break;
+    }
+    case CANON_MASK_F32:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[RUN ? first + j : idx[j]];
+        break;
+    case CANON_MASK_BF16:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, RUN ? first + j : idx[j]);
+        break;
+    default:
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, RUN ? first + j : idx[j]);
+        break;
+    }
+}
+
 template <int N>
 __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
                                                int dt, float *m)
 {
+    if (stride == 1 && t_first >= 0 && t_first + N <= L) {
+        // the common case, away from the ends of the sequence: one contiguous run, no clamping
+        load_mask_entries<N, true>(p, row_base + t_first, nullptr, dt, m);
+        return;
+    }
     int64_t idx[N];
 #pragma unroll
     for (int j = 0; j < N; ++j) {
@@ -184,36 +225,7 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
         t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
         idx[j] = row_base + t * stride;
     }
-    switch (dt) {
-    case CANON_MASK_U8:
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[idx[j]];
-        break;
-    case CANON_MASK_I32:
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[idx[j]];
-        break;
-    case CANON_MASK_I64: {
-        uint2 q[N];
-#pragma unroll
-        for (int j = 0; j < N; ++j) q[j] = ((const uint2 *)p)[idx[j]];
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = i64_words_to_float(q[j].x, q[j].y);
-        break;
-    }
-    case CANON_MASK_F32:
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = ((const float *)p)[idx[j]];
-        break;
-    case CANON_MASK_BF16:
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, idx[j]);
-        break;
-    default:
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, idx[j]);
-        break;
-    }
+    load_mask_entries<N, false>(p, 0, idx, dt, m);
 }
 
 // A lane's access unit in the channel-contiguous kernels: 16 bytes, or 8 bytes (half the registers

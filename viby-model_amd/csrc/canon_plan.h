@@ -125,6 +125,7 @@ constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 %
 #endif
 constexpr int kBwdSlab = CANON_BWD_SLAB;    // time steps per wave and tile
 constexpr int kBwdWaves = 4;
+constexpr int kBwdMaxChunk = 32 * kBwdSlab * kBwdWaves;   // most time steps one block of the channel-contiguous backward walks
 enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 

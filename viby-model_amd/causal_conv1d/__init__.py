@@ -116,7 +116,9 @@ def _prep_bias(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> Optional[t
 
 
 _NARROW_MIN_ELEMENTS = 1 << 20
-_narrow_cache = [None, None, None]   # key, the source mask (kept alive so its address stays unique), converted mask
+# (key, the source mask (kept alive so its address stays unique), converted mask); replaced as one object, so
+# threads that race here each see a consistent entry
+_narrow_cache = (None, None, None)
 
 
 def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tensor:
@@ -133,10 +135,13 @@ def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tenso
     if (mask.dtype.is_floating_point or mask.element_size() <= x.element_size()
             or numel < _NARROW_MIN_ELEMENTS):
         return mask
+    global _narrow_cache
     key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, x.dtype, mask.device)
-    if _narrow_cache[0] != key:
-        _narrow_cache[:] = [key, mask, mask.to(x.dtype)]
-    return _narrow_cache[2]
+    entry = _narrow_cache
+    if entry[0] != key:
+        entry = (key, mask, mask.to(x.dtype))
+        _narrow_cache = entry
+    return entry[2]
 
 
 def _stream(dev: torch.device) -> ctypes.c_void_p:

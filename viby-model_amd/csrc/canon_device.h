@@ -177,10 +177,17 @@ template <int N, bool RUN>
 __device__ __forceinline__ void load_mask_entries(const void *p, int64_t first, const int64_t *idx, int dt, float *m)
 {
     // RUN: the entries are first, first+1, .. (constant offsets: the loads merge); else idx[j]
+    // 1- and 2-byte entries are taken out of the aligned 32-bit word that holds them: a wave-uniform
+    // 32-bit load can be a scalar-memory load, a byte or short load cannot
+    const uint32_t *words = (const uint32_t *)((uintptr_t)p & ~(uintptr_t)3);
+    const int64_t byte0 = (int64_t)((uintptr_t)p & 3u);
     switch (dt) {
     case CANON_MASK_U8:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = (float)((const uint8_t *)p)[RUN ? first + j : idx[j]];
+        for (int j = 0; j < N; ++j) {
+            const int64_t i = (RUN ? first + j : idx[j]) + byte0;
+            m[j] = (float)((words[i >> 2] >> (8 * (uint32_t)(i & 3))) & 0xFFu);
+        }
         break;
     case CANON_MASK_I32:
 #pragma unroll
@@ -200,11 +207,19 @@ __device__ __forceinline__ void load_mask_entries(const void *p, int64_t first, 
         break;
     case CANON_MASK_BF16:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_BF16>(p, RUN ? first + j : idx[j]);
+        for (int j = 0; j < N; ++j) {
+            const int64_t i = (RUN ? first + j : idx[j]) + (byte0 >> 1);
+            const uint32_t wd = words[i >> 1];
+            m[j] = bits_f((i & 1) ? (wd & 0xFFFF0000u) : (wd << 16));
+        }
         break;
     default:
 #pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = load1<CANON_DTYPE_F16>(p, RUN ? first + j : idx[j]);
+        for (int j = 0; j < N; ++j) {
+            const int64_t i = (RUN ? first + j : idx[j]) + (byte0 >> 1);
+            const uint32_t wd = words[i >> 1];
+            m[j] = (float)__builtin_bit_cast(_Float16, (uint16_t)((i & 1) ? (wd >> 16) : (wd & 0xFFFFu)));
+        }
         break;
     }
 }

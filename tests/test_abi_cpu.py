@@ -358,3 +358,9 @@ def test_seq_idx_plan_and_validation():
     assert "4-byte aligned" in last_error()
     assert plan(fwd_params(layout="blc", seq_idx=FAKE_SEQ, final_state=FAKE_STATE, final_len=3)) is None
     assert "seq_idx excludes" in last_error()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "single-GPU" in (r.stderr + r.stdout)

@@ -46,8 +46,18 @@ def decode_bytes(b, c, s, esize=2, wsize=2):
     return b * c * (2 * s + 2) * esize + c * W * wsize + c * wsize
 
 
+CLOCK_RAMP_S = 0.03   # untimed load before the warm-up steps: the first ~10 ms after idle run ~1 % slower (clocks ramping)
+
+
 def time_region(fn, steps, warmup):
     import torch
+    t_end = time.perf_counter() + CLOCK_RAMP_S
+    i = 0
+    while time.perf_counter() < t_end:
+        for _ in range(100):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -68,13 +78,18 @@ def bench_prefill(layout, steps, warmup, nbuf):
     g = torch.Generator(device=dev).manual_seed(0)
     w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
     bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    # all buffer pairs are carved out of ONE allocation, as an arena-allocating runtime would hold them:
+    # measured 1 % faster than separately allocated tensors (fewer, larger address-translation fragments)
+    n = B * C * L
+    pool = torch.empty(2 * nbuf * n, dtype=torch.bfloat16, device=dev)
     xs, outs, params = [], [], []
-    for _ in range(nbuf):
+    for i in range(nbuf):
+        x, o = pool[2 * i * n:(2 * i + 1) * n], pool[(2 * i + 1) * n:(2 * i + 2) * n]
         if layout == "bcl":
-            x = torch.randn(B, C, L, generator=g, device=dev).bfloat16()
+            x, o = x.view(B, C, L), o.view(B, C, L)
         else:
-            x = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
-        o = torch.empty_like(x)
+            x, o = x.view(B, L, C).transpose(1, 2), o.view(B, L, C).transpose(1, 2)
+        x.copy_(torch.randn(x.shape, generator=g, device=dev))
         xs.append(x)
         outs.append(o)
         params.append(cc._fill_fwd(x, o, w, bias, None, None, None, 0, 1, 0))

@@ -158,8 +158,11 @@ typedef struct canon_conv1d_update_params {
     const void *bias;
     const void *token_mask;         /* [batch], or NULL */
     int64_t mask_stride_b;
-    const int32_t *cache_seqlens;        /* upstream's circular-buffer mode: must be NULL */
-    const int32_t *conv_state_indices;   /* upstream's batch indirection:    must be NULL */
+    const int32_t *cache_seqlens;        /* [batch] or NULL.  Upstream's circular-buffer mode: conv_state is not
+                                            shifted; the token is written to slot cache_seqlens[b] % state_len and
+                                            the W-1 slots before it (cyclically) are the history.  Strided kernel. */
+    const int32_t *conv_state_indices;   /* [batch] or NULL.  Upstream's batch indirection: batch entry b uses row
+                                            conv_state_indices[b] of conv_state (a state pool of any number of rows). */
 } canon_conv1d_update_params;
 
 /*

@@ -286,3 +286,55 @@ int canon_oracle_update(const void *x, void *conv_state, const void *weight, con
     }
     return 0;
 }
+
+/*
+ * Decode update with the two state-addressing modes of the upstream call
+ * signature that the reference never uses (model/model.py:305-311 passes
+ * neither; the signature slots are listed at causal_conv1d_mps/__init__.py:304-312):
+ *   conv_state_indices[b]  row of conv_state (a pool of `rows` rows) used by batch entry b
+ *   cache_seqlens[b]       circular-buffer mode: the token is written to slot
+ *                          cache_seqlens[b] % S, the W-1 slots before it
+ *                          (cyclically) are the history, nothing is shifted
+ * Fused rounding only.  PARITY UNPINNED against upstream (absent from the
+ * reference tree); pinned by its equivalence with canon_oracle_update: the same
+ * tokens fed with cache_seqlens = 0, 1, 2, .. give the same outputs, and the
+ * buffer read cyclically from the write position is the shifted state.
+ */
+int canon_oracle_update_ext(const void *x, void *conv_state, const void *weight, const void *bias, void *out,
+                            int64_t B, int64_t C, int W, int S, int dtype, int w_dtype, int use_silu,
+                            int residual, const int32_t *cache_seqlens, const int32_t *conv_state_indices)
+{
+    if (W < 1 || W > 8 || S < 1 || S < W - 1 || B < 0 || C < 0) return -1;
+    const size_t es = (dtype == CANON_F32) ? 4 : 2;
+    for (int64_t b = 0; b < B; ++b) {
+        const int64_t srow = conv_state_indices ? conv_state_indices[b] : b;
+        for (int64_t c = 0; c < C; ++c) {
+            const int64_t r = b * C + c, sr = srow * C + c;
+            float w[8], window[8];
+            for (int k = 0; k < W; ++k) w[k] = round_to(load_elem(weight, c * W + k, w_dtype), dtype);
+            const float bv = bias ? round_to(load_elem(bias, c, w_dtype), dtype) : 0.0f;
+            const float xv = load_elem(x, r, dtype);
+            int pos = -1;
+            if (cache_seqlens) pos = (int)(((cache_seqlens[b] % S) + S) % S);
+            for (int k = 0; k < W - 1; ++k) {
+                int slot = S - (W - 1) + k;
+                if (pos >= 0) slot = ((pos - (W - 1) + k) % S + S) % S;
+                window[k] = load_elem(conv_state, sr * S + slot, dtype);
+            }
+            window[W - 1] = xv;
+            float acc = bv;
+            for (int k = 0; k < W; ++k) acc = fmaf(w[k], window[k], acc);
+            if (use_silu) acc = silu(acc);
+            if (residual) acc += xv;
+            store_elem(out, r, dtype, acc);
+            char *row = (char *)conv_state + (size_t)sr * S * es;
+            if (pos >= 0) {
+                memcpy(row + (size_t)pos * es, (const char *)x + (size_t)r * es, es);
+            } else {
+                memmove(row, row + es, (size_t)(S - 1) * es);
+                memcpy(row + (size_t)(S - 1) * es, (const char *)x + (size_t)r * es, es);
+            }
+        }
+    }
+    return 0;
+}

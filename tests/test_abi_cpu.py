@@ -164,9 +164,11 @@ def test_update_plan_and_validation():
     assert uplan(update_params(C=3457)) == "update_generic"
     assert uplan(update_params(state_stride_s=2, state_stride_c=6, state_stride_b=3456 * 6)) == "update_generic"
     assert uplan(update_params(round_mode=1)) == "update_generic"
+    assert uplan(update_params(conv_state_indices=FAKE_STATE + 64)) == "update_vec"       # state pool: row indirection
+    assert uplan(update_params(cache_seqlens=FAKE_STATE + 64)) == "update_generic"        # circular buffer
     for over, needle in [(dict(S=2), "state_len"), (dict(width=7), "width"),
-                         (dict(cache_seqlens=FAKE_STATE), "cache_seqlens"),
-                         (dict(conv_state_indices=FAKE_STATE), "conv_state_indices"),
+                         (dict(cache_seqlens=FAKE_STATE + 2), "4-byte aligned"),
+                         (dict(conv_state_indices=FAKE_STATE + 1), "4-byte aligned"),
                          (dict(conv_state=0), "NULL"), (dict(struct_size=4), "struct_size")]:
         if "S" in over:
             p = update_params(S=over["S"])
@@ -210,9 +212,12 @@ def test_wrapper_errors_match_reference_conventions():
         cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4), torch.randn(4, 4))
     with pytest.raises(ValueError, match="doesn't match conv_state"):
         cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(3, 4, 4), torch.randn(4, 4))
-    with pytest.raises(NotImplementedError, match="cache_seqlens"):
+    with pytest.raises(ValueError, match="cache_seqlens must be a contiguous int32 tensor"):
         cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4, 4), torch.randn(4, 4),
-                                cache_seqlens=torch.zeros(2, dtype=torch.int32))
+                                cache_seqlens=torch.zeros(2, dtype=torch.int64))
+    with pytest.raises(ValueError, match="conv_state_indices must be a contiguous int32 tensor"):
+        cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(7, 4, 4), torch.randn(4, 4),
+                                conv_state_indices=torch.zeros(3, dtype=torch.int32))
     with pytest.raises(ValueError, match="must be on a ROCm GPU device"):
         cc.causal_conv1d_update(torch.randn(2, 4), torch.zeros(2, 4, 4), torch.randn(4, 4))
     with pytest.raises(ValueError, match="Expected 3D input tensor"):

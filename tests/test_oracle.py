@@ -416,3 +416,34 @@ def test_seq_idx_oracle_brute_force_and_separate_sequences():
         a = co.conv1d_fwd_seq(x, w, None, same, mask=mask, activation=act, residual=res)
         b_ = co.conv1d_fwd(x, w, None, mask=mask, activation=act, residual=res)
         assert torch.equal(a.view(torch.int16), b_.view(torch.int16))
+
+
+def test_ring_buffer_and_state_pool_update_equal_the_shift_register():
+    g = torch.Generator().manual_seed(83)
+    for dtype, W, S in itertools.product([torch.float32, torch.bfloat16], [2, 3, 4], [3, 4, 7, 8]):
+        if S < W - 1:
+            continue
+        B, C, rows = 3, 5, 7
+        w = torch.randn(C, W, generator=g).to(dtype)
+        b = torch.randn(C, generator=g).to(dtype)
+        start = torch.randn(B, C, S, generator=g).to(dtype)
+        shift = start.clone()
+        ring = start.clone()                      # ring position 0 = oldest entry = shift-register slot 0
+        pool = torch.randn(rows, C, S, generator=g).to(dtype)
+        rows_of = torch.tensor([5, 0, 3], dtype=torch.int32)
+        pool[rows_of.long()] = start
+        untouched = pool.clone()
+        for step in range(2 * S + 3):
+            x = torch.randn(B, C, generator=g).to(dtype)
+            want = co.conv1d_update(x, shift, w, b, activation="silu", residual=True)
+            got = co.conv1d_update_ext(x, ring, w, b, activation="silu", residual=True,
+                                       cache_seqlens=torch.full((B,), step, dtype=torch.int32))
+            assert torch.equal(got.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                               want.view(torch.int16 if dtype != torch.float32 else torch.int32)), (dtype, W, S, step)
+            pos = (step + 1) % S
+            assert torch.equal(torch.cat([ring[:, :, pos:], ring[:, :, :pos]], dim=2), shift), (dtype, W, S, step)
+            got2 = co.conv1d_update_ext(x, pool, w, b, activation="silu", residual=True, conv_state_indices=rows_of)
+            assert torch.equal(got2, want)
+            assert torch.equal(pool[rows_of.long()], shift)
+        others = [r for r in range(rows) if r not in rows_of.tolist()]
+        assert torch.equal(pool[others], untouched[others])

@@ -511,3 +511,35 @@ def test_time_contiguous_rows_off_the_16_byte_grid(cc, dtype):
                 assert torch.equal(bits(got[1]), bits(want[1])), what
             else:
                 assert_parity(got, want, exact=act is None, what=what, res=xm if res else None)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_update_ring_buffer_and_state_pool(cc, dtype):
+    """cache_seqlens (ring buffer) and conv_state_indices (rows of a state pool) against the oracle, whose
+    two modes are pinned by their equivalence with the shift register."""
+    g = torch.Generator().manual_seed(85)
+    for (B, C), W, S in itertools.product([(4, 264), (3, 20), (64, 3456)], [2, 4], [3, 4, 8, 6]):
+        if S < W - 1:
+            continue
+        rows = B + 3
+        w = (torch.randn(C, W, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        pool_ref = torch.randn(rows, C, S, generator=g).to(dtype)
+        ring_ref = torch.randn(B, C, S, generator=g).to(dtype)
+        idx = torch.randperm(rows, generator=g)[:B].to(torch.int32)
+        pool_gpu, ring_gpu = pool_ref.to(DEV), ring_ref.to(DEV)
+        expect_plan = "update_vec" if (S in (3, 4, 8) and C % (16 // w.element_size()) == 0) else "update_generic"
+        assert cc.kernel_plan_update(torch.empty(B, C, dtype=dtype, device=DEV), pool_gpu[:B], w.to(DEV)) == expect_plan
+        for step in range(S + 2):
+            x = torch.randn(B, C, generator=g).to(dtype)
+            seqlens = torch.randint(0, 1000, (B,), generator=g).to(torch.int32) if step else torch.zeros(B, dtype=torch.int32)
+            what = f"{dtype}/{B}x{C}/W{W}/S{S}/step{step}"
+            want = co.conv1d_update_ext(x, pool_ref, w, b, activation="silu", residual=True, conv_state_indices=idx)
+            got = cc.causal_conv1d_update(x.to(DEV), pool_gpu, w.to(DEV), b.to(DEV), activation="silu", residual=True,
+                                          conv_state_indices=idx.to(DEV))
+            assert_parity(got, want, exact=False, what="pool/" + what, res=x)
+            assert torch.equal(bits(pool_gpu), bits(pool_ref)), what
+            want = co.conv1d_update_ext(x, ring_ref, w, b, activation=None, residual=False, cache_seqlens=seqlens)
+            got = cc.causal_conv1d_update(x.to(DEV), ring_gpu, w.to(DEV), b.to(DEV), cache_seqlens=seqlens.to(DEV))
+            assert_parity(got, want, exact=True, what="ring/" + what)
+            assert torch.equal(bits(ring_gpu), bits(ring_ref)), what

@@ -422,6 +422,11 @@ def causal_conv1d_update(
 
     ``out = act(bias + sum_{k<W-1} w[k]*state[S-(W-1)+k] + w[W-1]*x)``.
 
+    cache_seqlens       (batch,) int32: upstream's circular-buffer mode.  ``conv_state`` is not
+                shifted; the token is written to slot ``cache_seqlens % state_len`` and the W-1
+                slots before it (cyclically) are the history.
+    conv_state_indices  (batch,) int32: batch entry b uses row ``conv_state_indices[b]`` of
+                ``conv_state`` (a pool of any number of rows).
     token_mask  (batch,) multiplies the token before everything else
                 (``model/model.py:277-282``).
     residual    False | True ('masked': adds the masked token,
@@ -432,10 +437,6 @@ def causal_conv1d_update(
     act = _activation_flag(activation)
     res = _residual_mode(residual)
     rnd = _round_mode(rounding)
-    if cache_seqlens is not None:
-        raise NotImplementedError("cache_seqlens (circular conv_state) is not supported")
-    if conv_state_indices is not None:
-        raise NotImplementedError("conv_state_indices is not supported")
     squeeze_back = False
     if x.dim() == 3:
         if x.shape[2] != 1:
@@ -451,11 +452,17 @@ def causal_conv1d_update(
     if conv_state.dim() != 3:
         raise ValueError(f"Expected 3D conv_state tensor (batch, dim, state_len), got {conv_state.dim()}D")
     batch, dim = x2.shape
-    if tuple(conv_state.shape[:2]) != (batch, dim):
+    if conv_state_indices is None and tuple(conv_state.shape[:2]) != (batch, dim):
         raise ValueError(
             f"Input shape {tuple(x2.shape)} doesn't match conv_state batch/dim {tuple(conv_state.shape[:2])}")
+    if conv_state_indices is not None and conv_state.shape[1] != dim:
+        raise ValueError(f"Input dim {dim} doesn't match conv_state dim {conv_state.shape[1]}")
     if conv_state.dtype != x.dtype or conv_state.device != x.device:
         raise ValueError("conv_state must have the dtype and device of x")
+    for name, t in (("cache_seqlens", cache_seqlens), ("conv_state_indices", conv_state_indices)):
+        if t is not None and (t.dim() != 1 or t.shape[0] != batch or t.dtype != torch.int32 or t.device != x.device
+                              or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous int32 tensor of shape (batch,) = ({batch},) on the device of x")
     _check_shapes(dim, weight, bias)
     _require_gpu(x, "Input tensor")
     _check_devices(weight, bias, x.device)
@@ -472,6 +479,10 @@ def causal_conv1d_update(
     out = torch.empty((batch, dim), dtype=x.dtype, device=x.device)
     if out.numel():
         p = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
+        if cache_seqlens is not None:
+            p.cache_seqlens = cache_seqlens.data_ptr()
+        if conv_state_indices is not None:
+            p.conv_state_indices = conv_state_indices.data_ptr()
         with torch.cuda.device(x.device):
             rc = _lib.lib().canon_conv1d_update(ctypes.byref(p), _stream(x.device))
         _lib.check(rc, "causal_conv1d_update")
@@ -660,16 +671,14 @@ def short_conv_update(
     """Single-token step with the argument order of
     ``causal_conv1d_mps.short_conv_update`` (``causal_conv1d_mps/__init__.py:304-419``).
 
-    The state is a shift register (newest token last), the layout the prefill
-    path and the eager step (``model/model.py:385-386``) use; the reference's
-    Metal kernel instead indexes it as a ring through ``cache_seqlens``
-    (``causal_conv1d.metal:755-775``), which is not reproduced: passing
-    ``cache_seqlens`` raises.
+    Without ``cache_seqlens`` the state is a shift register (newest token last), the layout the
+    prefill path and the eager step (``model/model.py:385-386``) use.  With it the state is a ring
+    written at ``cache_seqlens % state_len``, as in the reference's Metal kernel
+    (``causal_conv1d.metal:755-775``); a state filled by the prefill is right-aligned, so the
+    first ring position consistent with it is ``cache_seqlens = 0 (mod state_len)``.
     """
-    if cache_seqlens is not None:
-        raise NotImplementedError("cache_seqlens (ring-buffer conv_state) is not supported; the state is a shift register")
     return causal_conv1d_update(x, conv_state, weight, bias, activation="silu" if activation else None,
-                                residual="masked" if residual else False)
+                                cache_seqlens=cache_seqlens, residual="masked" if residual else False)
 
 
 # ---------------------------------------------------------------------------

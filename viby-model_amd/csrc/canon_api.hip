@@ -212,8 +212,10 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
     if (p->round_mode != CANON_ROUND_FUSED && p->round_mode != CANON_ROUND_EAGER)
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
-    if (p->cache_seqlens) return fail(CANON_ERR_UNSUPPORTED, "cache_seqlens (circular conv_state) is not supported");
-    if (p->conv_state_indices) return fail(CANON_ERR_UNSUPPORTED, "conv_state_indices is not supported");
+    if (((uintptr_t)p->cache_seqlens | (uintptr_t)p->conv_state_indices) & 3u)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "cache_seqlens and conv_state_indices must be 4-byte aligned");
+    if (p->cache_seqlens && p->width - 1 > p->state_len)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_len %d is shorter than width-1 = %d", p->state_len, p->width - 1);
     if (p->batch < 0 || p->channels < 0)
         return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld)", (long long)p->batch, (long long)p->channels);
     if (p->batch >= (1ll << 31) || p->channels >= (1ll << 31) || p->batch * p->channels >= (1ll << 31))
@@ -230,6 +232,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     memset(&a, 0, sizeof(a));
     a.x = (const char *)p->x; a.out = (char *)p->out; a.state = (char *)p->conv_state;
     a.weight = p->weight; a.bias = p->bias; a.tmask = p->token_mask;
+    a.seqlens = p->cache_seqlens; a.indices = p->conv_state_indices;
     a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c;
     a.s_sb = p->state_stride_b; a.s_sc = p->state_stride_c; a.s_ss = p->state_stride_s;
     a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k; a.m_sb = p->mask_stride_b;
@@ -244,7 +247,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
 
     const int E = 16 / elem_bytes(p->x_dtype);
     const int S = p->state_len;
-    const bool vec_ok = p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
+    const bool vec_ok = !p->cache_seqlens && p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
                         aligned16(p->x) && aligned16(p->out) && aligned16(p->conv_state) &&
                         a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb % E == 0 && a.o_sb % E == 0 &&
                         a.s_ss == 1 && a.s_sc == S && a.s_sb % E == 0;

@@ -63,6 +63,8 @@ struct UpdArgs {
     const void *weight;
     const void *bias;
     const void *tmask;
+    const int32_t *seqlens;   // circular-buffer mode: conv_state is written at seqlens[b] % S, not shifted
+    const int32_t *indices;   // conv_state row of batch entry b (state pool shared by many sequences)
     int64_t x_sb, x_sc, o_sb, o_sc;
     int64_t s_sb, s_sc, s_ss;
     int64_t w_sc, w_sk;

@@ -56,13 +56,15 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
     uint4 X[NB];
     uint4 ST[NB][S];
     float tm[NB];
+    uint32_t srow[NB];   // conv_state row of each batch entry
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
         const uint32_t b = bg * NB + n;
         tm[n] = 1.0f;
         if (b < a.B) {
             X[n] = *(const uint4 *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
-            const uint4 *sp = (const uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
+            srow[n] = a.indices ? (uint32_t)a.indices[b] : b;
+            const uint4 *sp = (const uint4 *)(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY);
 #pragma unroll
             for (int k = 0; k < S; ++k) ST[n][k] = sp[k];
         }
@@ -131,7 +133,7 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
 #pragma unroll
             for (int e = 0; e < E; ++e) raw[e * S + S - 1] = StateRun<DT>::raw_of(xt[e]);
         }
-        uint4 *dp = (uint4 *)(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY);
+        uint4 *dp = (uint4 *)(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY);
 #pragma unroll
         for (int k = 0; k < S; ++k) {
             uint4 q;
@@ -175,11 +177,25 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
     for (int k = 0; k < W; ++k)
         w[4 - W + k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
     const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
-    const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
+    const uint32_t srow = a.indices ? (uint32_t)a.indices[b] : b;
+    const int64_t so = (int64_t)srow * a.s_sb + (int64_t)c * a.s_sc;
+    // circular-buffer mode: the token goes to slot pos, the W-1 slots before it (cyclically) are the history
+    int pos = -1;
+    if (a.seqlens) {
+        pos = a.seqlens[b] % S;
+        if (pos < 0) pos += S;
+    }
     const float xr = load1<DT>(a.x, (int64_t)b * a.x_sb + (int64_t)c * a.x_sc);
     float xt = xr;
     if (a.tmask) xt = mul_round<DT>(xr, load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype));
-    for (int k = 0; k < W - 1; ++k) win[4 - W + k] = load1<DT>(a.state, so + (int64_t)(S - (W - 1) + k) * a.s_ss);
+    for (int k = 0; k < W - 1; ++k) {
+        int slot = S - (W - 1) + k;
+        if (pos >= 0) {
+            slot = pos - (W - 1) + k;
+            if (slot < 0) slot += S;
+        }
+        win[4 - W + k] = load1<DT>(a.state, so + (int64_t)slot * a.s_ss);
+    }
     win[3] = xt;
     float acc;
     if (!a.eager) {
@@ -199,6 +215,10 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
         else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc = __fadd_rn(acc, xr);
     }
     store1<DT>(a.out, (int64_t)b * a.o_sb + (int64_t)c * a.o_sc, acc);
+    if (pos >= 0) {
+        store1<DT>(a.state, so + (int64_t)pos * a.s_ss, xt);
+        return;
+    }
     // shift left by one (ascending order: each slot is read before it is overwritten)
     for (int k = 0; k < S - 1; ++k) {
         if constexpr (DT == CANON_DTYPE_F32)

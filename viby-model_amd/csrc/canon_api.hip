@@ -368,7 +368,7 @@ int plan_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_pa
         }
         c0 += parts[i].channels;
     }
-    pp->single = nparts > 1 && all_vec && p->width == 4 && nvec_total > 0;
+    pp->single = nparts > 1 && all_vec && p->width == 4 && !p->conv_state_indices && nvec_total > 0;
     pp->grid = 0;
     if (pp->single) {
         // batch rows per lane chosen on the whole token, the same for every part

@@ -42,7 +42,7 @@ template <int DT> struct StateRun {
     }
 };
 
-template <int DT, int W, int S, int NB>
+template <int DT, int W, int S, int NB, bool POOL = false>
 __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_t blk)
 {
     constexpr int E = Elem<DT>::per_vec;
@@ -63,7 +63,7 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
         tm[n] = 1.0f;
         if (b < a.B) {
             X[n] = *(const uint4 *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
-            srow[n] = a.indices ? (uint32_t)a.indices[b] : b;
+            srow[n] = POOL ? (uint32_t)a.indices[b] : b;   // POOL: rows of a state pool (conv_state_indices)
             const uint4 *sp = (const uint4 *)(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY);
 #pragma unroll
             for (int k = 0; k < S; ++k) ST[n][k] = sp[k];
@@ -156,6 +156,13 @@ __global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
     update_vec_block<DT, W, S, NB>(a, blockIdx.x);
 }
 
+// the same with batch entry b using row conv_state_indices[b] of a state pool
+template <int DT, int W, int S, int NB>
+__global__ __launch_bounds__(256) void canon_update_vec_pool_kernel(const UpdArgs a)
+{
+    update_vec_block<DT, W, S, NB, true>(a, blockIdx.x);
+}
+
 // the token of one step given as several channel ranges (separate projections), one launch
 template <int DT, int W, int S, int NB>
 __global__ __launch_bounds__(256) void canon_update_vec_parts_kernel(const PartTable<UpdArgs> m)
@@ -237,6 +244,14 @@ namespace {
 template <int DT, int W, int NB> void launch_update_vec_nb(const UpdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
+    if (pl.args.indices) {
+        switch (pl.args.S) {
+        case 3: hipLaunchKernelGGL((canon_update_vec_pool_kernel<DT, W, 3, NB>), g, b, 0, s, pl.args); break;
+        case 4: hipLaunchKernelGGL((canon_update_vec_pool_kernel<DT, W, 4, NB>), g, b, 0, s, pl.args); break;
+        default: hipLaunchKernelGGL((canon_update_vec_pool_kernel<DT, W, 8, NB>), g, b, 0, s, pl.args); break;
+        }
+        return;
+    }
     switch (pl.args.S) {
     case 3: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 3, NB>), g, b, 0, s, pl.args); break;
     case 4: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 4, NB>), g, b, 0, s, pl.args); break;

@@ -96,7 +96,7 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     for C in (640, 960, 3456):
         assert plan(fwd_params(C=C, layout="bcl")) == "bcl_vec"
         assert plan(fwd_params(C=C, layout="blc")) == "blc_vec"
-    assert plan(fwd_params(B=1, C=640, L=1024, dtype=0)) == "bcl_vec"     # BASELINE config 1
+    assert plan(fwd_params(B=1, C=640, L=1024, dtype=0)) == "bcl_vec"     # benchmark configuration 1 (fp32, CPU-runnable)
     # time-contiguous rows that are not a whole number of vectors keep the vector kernel (edge elements aside)
     # as long as x and out share their strides
     assert plan(fwd_params(L=1023)) == "bcl_vec"

@@ -146,7 +146,7 @@ def test_backward_finite_differences_like_the_reference_tests(cc):
 @pytest.mark.parametrize("layout", ["blc", "bcl"])
 def test_backward_at_model_shape_is_deterministic_and_correct(cc, layout):
     g = torch.Generator().manual_seed(23)
-    B, C, L = 4, 3456, 1024                      # Canon-D channel count, BASELINE sequence length
+    B, C, L = 4, 3456, 1024                      # Canon-D channel count, benchmark sequence length
     x = torch.randn(B, C, L, generator=g).bfloat16()
     w = (torch.randn(C, 4, generator=g) * 0.3).bfloat16()
     b = (torch.randn(C, generator=g) * 0.1).bfloat16()

@@ -70,7 +70,7 @@ def test_canon_layer_golden_vectors(case, rounding):
 
 @pytest.mark.parametrize("site,C", [("a", 640), ("b", 960), ("d", 3456)])
 def test_canon_layer_prefill_then_decode_at_model_shapes(site, C):
-    """BASELINE shapes of the four call sites: prefill with a padding mask, then 8 decode steps."""
+    """Benchmark shapes of the four call sites: prefill with a padding mask, then 8 decode steps."""
     torch.manual_seed(5)
     B, T = 4, 256
     dtype = torch.bfloat16

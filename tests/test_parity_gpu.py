@@ -42,7 +42,7 @@ def run_fwd(cc, x, w, b, act=None, mask=None, residual=False, init=None, S_out=N
     return r
 
 
-# ---- BASELINE config 1 ------------------------------------------------------
+# ---- benchmark configuration 1: fp32 x[1,640,1024], Canon-A ------------------------------------------------------
 def test_config1_fp32_canon_a(cc):
     torch.manual_seed(0)
     x = torch.randn(1, 640, 1024)
@@ -56,7 +56,7 @@ def test_config1_fp32_canon_a(cc):
         assert_parity(got, want, exact=True, what=f"config1/{name}")
 
 
-# ---- BASELINE config 2 ------------------------------------------------------
+# ---- benchmark configuration 2: bf16 B8 L1024, C in {640, 960, 3456} ------------------------------------------------------
 @pytest.mark.parametrize("C", [640, 960, 3456])
 @pytest.mark.parametrize("act", [None, "silu"])
 def test_config2_bf16_prefill(cc, C, act):
@@ -71,7 +71,7 @@ def test_config2_bf16_prefill(cc, C, act):
         assert_parity(got, want, exact=act is None, what=f"config2/C{C}/{act}/{name}")
 
 
-# ---- BASELINE config 3 ------------------------------------------------------
+# ---- benchmark configuration 3: ragged right-padded batch of 32 ------------------------------------------------------
 @pytest.mark.parametrize("residual", ["masked", "unmasked"])
 def test_config3_ragged_padded_prefill(cc, residual):
     g = torch.Generator().manual_seed(3)
@@ -95,7 +95,7 @@ def test_config3_ragged_padded_prefill(cc, residual):
     assert torch.equal(bits(a), bits(c))
 
 
-# ---- BASELINE config 4 ------------------------------------------------------
+# ---- benchmark configuration 4: decode, B256, state 3, 64 carried steps ------------------------------------------------------
 @pytest.mark.parametrize("S", [3, 4, 8])
 def test_config4_decode_64_steps(cc, S):
     g = torch.Generator().manual_seed(4)

@@ -1,4 +1,4 @@
-"""BASELINE config 5: a Viby-shaped model (tests/viby_harness.py) run with the HIP Canon layers
+"""Benchmark configuration 5: a Viby-shaped model (tests/viby_harness.py) run with the HIP Canon layers
 and with reference Canon back ends inside an otherwise identical network."""
 import time
 import types

@@ -162,7 +162,8 @@ typedef struct canon_conv1d_update_params {
                                             shifted; the token is written to slot cache_seqlens[b] % state_len and
                                             the W-1 slots before it (cyclically) are the history.  Strided kernel. */
     const int32_t *conv_state_indices;   /* [batch] or NULL.  Upstream's batch indirection: batch entry b uses row
-                                            conv_state_indices[b] of conv_state (a state pool of any number of rows). */
+                                            conv_state_indices[b] of conv_state (a state pool of any number of rows;
+                                            the caller guarantees the indices are valid and distinct). */
 } canon_conv1d_update_params;
 
 /*

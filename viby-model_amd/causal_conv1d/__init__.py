@@ -144,8 +144,21 @@ def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tenso
     return entry[2]
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the handle without building a Stream object
+
+
 def _stream(dev: torch.device) -> ctypes.c_void_p:
+    if _raw_stream is not None and dev.index is not None:
+        return ctypes.c_void_p(_raw_stream(dev.index))
     return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _call(fn, dev: torch.device, *args) -> int:
+    """Launch on the current stream of ``dev`` with ``dev`` current (switching only if it is not already)."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return fn(*args, _stream(dev))
+    with torch.cuda.device(dev):
+        return fn(*args, _stream(dev))
 
 
 def _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx=None) -> FwdParams:
@@ -303,8 +316,7 @@ def _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, r
     if x.numel() == 0:
         return out
     p = _fill_fwd(x, out, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx)
-    with torch.cuda.device(x.device):
-        rc = _lib.lib().canon_conv1d_fwd(ctypes.byref(p), _stream(x.device))
+    rc = _call(_lib.lib().canon_conv1d_fwd, x.device, ctypes.byref(p))
     _lib.check(rc, "causal_conv1d_fn")
     return out
 
@@ -370,8 +382,7 @@ class _CanonConvFn(torch.autograd.Function):
         workspace = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=x.device)
         p.workspace = workspace.data_ptr()
         p.workspace_bytes = workspace.numel()
-        with torch.cuda.device(x.device):
-            rc = L.canon_conv1d_bwd(ctypes.byref(p), _stream(x.device))
+        rc = _call(L.canon_conv1d_bwd, x.device, ctypes.byref(p))
         _lib.check(rc, "causal_conv1d_fn backward")
         return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
                 None, None, None, None, None)
@@ -483,8 +494,7 @@ def causal_conv1d_update(
             p.cache_seqlens = cache_seqlens.data_ptr()
         if conv_state_indices is not None:
             p.conv_state_indices = conv_state_indices.data_ptr()
-        with torch.cuda.device(x.device):
-            rc = _lib.lib().canon_conv1d_update(ctypes.byref(p), _stream(x.device))
+        rc = _call(_lib.lib().canon_conv1d_update, x.device, ctypes.byref(p))
         _lib.check(rc, "causal_conv1d_update")
     return out.unsqueeze(-1) if squeeze_back else out
 
@@ -572,8 +582,7 @@ def causal_conv1d_fn_parts(
         p.channels = dim
         p.x = p.out = None
         arr = _part_array(xs, outs)
-        with torch.cuda.device(xs[0].device):
-            rc = _lib.lib().canon_conv1d_fwd_parts(ctypes.byref(p), arr, len(xs), _stream(xs[0].device))
+        rc = _call(_lib.lib().canon_conv1d_fwd_parts, xs[0].device, ctypes.byref(p), arr, len(xs))
         _lib.check(rc, "causal_conv1d_fn_parts")
     return (outs, final_states) if final_states is not None else outs
 
@@ -627,8 +636,7 @@ def causal_conv1d_update_parts(
         p.channels = dim
         p.x = p.out = None
         arr = _part_array(xs, outs)
-        with torch.cuda.device(x0.device):
-            rc = _lib.lib().canon_conv1d_update_parts(ctypes.byref(p), arr, len(xs), _stream(x0.device))
+        rc = _call(_lib.lib().canon_conv1d_update_parts, x0.device, ctypes.byref(p), arr, len(xs))
         _lib.check(rc, "causal_conv1d_update_parts")
     return outs
 

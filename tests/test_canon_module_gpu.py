@@ -140,3 +140,50 @@ def test_decode_token_as_one_hip_graph():
         for k in states_g:
             assert torch.equal(bits(states_g[k]), bits(states_e[k])), (replay, k)
             assert torch.equal(bits(outs_g[k]), bits(outs_e[k])), (replay, k)
+
+
+def test_unmodified_model_call_pattern():
+    """What the reference's own CanonLayer does around the two package calls on its accelerated branch
+    (model/model.py:454-491 prefill, :299-313 decode), spelled out with the package's functions and the
+    reference's keywords: mask multiply, transpose to (B, D, T), conv, state = last K masked inputs,
+    `x + output`; then `x_token + update(...)` on that state.  Checked against the CPU oracle."""
+    import causal_conv1d as cc
+    from oracle import canon_oracle as co
+    torch.manual_seed(33)
+    B, T, D, K = 4, 50, 640, 4
+    dtype = torch.bfloat16
+    x = torch.randn(B, T, D).to(dtype)
+    weight = (torch.randn(D, 1, K) * 0.3).to(dtype)           # the module's parameter shape
+    mask = right_padded_mask([50, 31, 4, 17], T)
+    for activation in (None, "silu"):
+        xg, wg, mg = x.to(DEV), weight.to(DEV), mask.to(DEV)
+        masked_x = xg * mg.unsqueeze(-1)
+        x_conv = masked_x.transpose(1, 2)
+        y_conv = cc.causal_conv1d_fn(x=x_conv, weight=wg.squeeze(1), bias=None, activation=activation, seq_idx=None)
+        assert y_conv.stride() == x_conv.stride()
+        out = xg + y_conv.transpose(1, 2)
+        conv_state = torch.zeros(B, D, K, device=DEV, dtype=dtype)
+        conv_state[:, :, :] = x_conv[:, :, -K:]
+
+        xm = (x.float() * mask[:, :, None].float()).to(dtype)
+        want_y, want_state = co.conv1d_fwd(xm.transpose(1, 2).contiguous(), weight.squeeze(1), None,
+                                           activation=activation, final_state_len=K)
+        if activation is None:
+            assert torch.equal(bits(y_conv.contiguous()), bits(want_y))
+        else:
+            assert (y_conv.float().cpu() - want_y.float()).abs().max() <= 2 ** -7 * want_y.float().abs().max()
+        assert torch.equal(bits(conv_state), bits(want_state))
+        want_out = (x.float() + want_y.transpose(1, 2).float()).to(dtype)      # the eager add rounds once more
+        assert (out.float().cpu() - want_out.float()).abs().max() <= 2 ** -6 * want_out.float().abs().max()
+
+        for step in range(3):
+            x_token = torch.randn(B, D).to(dtype)
+            held = conv_state
+            y = cc.causal_conv1d_update(x=x_token.to(DEV), conv_state=conv_state, weight=wg.squeeze(1), bias=None,
+                                        activation=activation)
+            want = co.conv1d_update(x_token, want_state, weight.squeeze(1), None, activation=activation)
+            assert conv_state is held and torch.equal(bits(conv_state), bits(want_state))
+            if activation is None:
+                assert torch.equal(bits(y), bits(want))
+            else:
+                assert (y.float().cpu() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max()

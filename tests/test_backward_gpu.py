@@ -231,3 +231,35 @@ def test_backward_more_than_2_31_elements(cc):
         w.grad = None
         del x, dout
         torch.cuda.empty_cache()
+
+
+def test_backward_randomised(cc):
+    """60 seeded random backward calls across layouts, sizes around the tile boundaries, dtypes, widths and options
+    against float64 autograd of the eager formulation."""
+    g = torch.Generator().manual_seed(777)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    def pick(seq):
+        return seq[ri(0, len(seq) - 1)]
+
+    for case in range(60):
+        dtype = pick([torch.bfloat16, torch.float32, torch.float16])
+        W = pick([2, 3, 4])
+        B, C = ri(1, 3), pick([1, 4, 8, 12, 64, 100, 260])
+        L = pick([1, 2, 3, 5, 31, 32, 33, 64, 65, 127, 128, 129, 200, 257])
+        layout = pick(["bcl", "blc"])
+        act, res = pick([None, "silu"]), pick([False, "masked", "unmasked"])
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, W, generator=g) * 0.5).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.2).to(dtype) if ri(0, 1) else None
+        dout = torch.randn(B, C, L, generator=g).to(dtype)
+        mask = right_padded_mask([ri(1, L) for _ in range(B)], L) if ri(0, 1) else None
+        dx, dw, db, _ = gpu_grads(cc, x, w, b, dout, layout, mask, act, res)
+        rdx, rdw, rdb, _ = conv1d_grads(x, w, b, dout, mask, act, res)
+        what = f"case {case}: {dtype} {layout} {B}x{C}x{L} W{W} {act} {res} mask{mask is not None} bias{b is not None}"
+        check(dx, rdx, dtype, what + " dx")
+        check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
+        if b is not None:
+            check(db, rdb, dtype, what + " dbias", sum_terms=B * L)

@@ -543,3 +543,116 @@ def test_update_ring_buffer_and_state_pool(cc, dtype):
             got = cc.causal_conv1d_update(x.to(DEV), ring_gpu, w.to(DEV), b.to(DEV), cache_seqlens=seqlens.to(DEV))
             assert_parity(got, want, exact=True, what="ring/" + what)
             assert torch.equal(bits(ring_gpu), bits(ring_ref)), what
+
+
+def test_randomised_shapes_layouts_and_options(cc):
+    """300 seeded random calls across layouts (time-contiguous, channel-contiguous, both as slices of larger
+    tensors), sizes around every vector / tile boundary, dtypes, widths and options, each against the oracle."""
+    g = torch.Generator().manual_seed(2024)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    def pick(seq):
+        return seq[ri(0, len(seq) - 1)]
+
+    plans = {}
+    for case in range(300):
+        dtype = pick([torch.bfloat16, torch.float32, torch.float16])
+        W = pick([2, 3, 4])
+        B = ri(1, 3)
+        C = pick([1, 3, 4, 8, 12, 20, 64, 100, 256, 260, 520])
+        L = pick([1, 2, 3, 5, 8, 31, 32, 33, 64, 127, 128, 129, 136, 200, 255, 257, 515])
+        layout = pick(["bcl", "blc", "bcl_slice", "blc_slice"])
+        act = pick([None, "silu"])
+        res = pick([False, "masked", "unmasked"])
+        use_mask = ri(0, 1)
+        use_bias = ri(0, 1)
+        mode = pick(["plain", "plain", "state", "seq"])
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, W, generator=g) * 0.4).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.2).to(dtype) if use_bias else None
+        mask = right_padded_mask([ri(1, L) for _ in range(B)], L, dtype=pick([torch.int64, torch.bool, torch.float32])) \
+            if use_mask else None
+        if layout == "bcl":
+            xg = x.to(DEV)
+        elif layout == "blc":
+            xg = x.to(DEV).transpose(1, 2).contiguous().transpose(1, 2)
+        elif layout == "bcl_slice":
+            big = torch.zeros(B, C + 3, L + 8, dtype=dtype, device=DEV)
+            big[:, 1:C + 1, 8:] = x.to(DEV)
+            xg = big[:, 1:C + 1, 8:]
+        else:
+            big = torch.zeros(B, L + 2, C + 8, dtype=dtype, device=DEV)
+            big[:, 1:L + 1, 8:] = x.to(DEV).transpose(1, 2)
+            xg = big[:, 1:L + 1, 8:].transpose(1, 2)
+        kw = dict(activation=act, residual=res, attention_mask=None if mask is None else mask.to(DEV))
+        what = f"case {case}: {dtype} {layout} {B}x{C}x{L} W{W} {act} {res} mask{use_mask} bias{use_bias} {mode}"
+        xm = x if mask is None else (x.float() * mask[:, None, :].float()).to(dtype)
+        if mode == "seq":
+            seq = packed_seq_idx(B, L, g)
+            want = co.conv1d_fwd_seq(x, w, b, seq, mask=mask, activation=act, residual=res)
+            got = cc.causal_conv1d_fn(xg, w.to(DEV), None if b is None else b.to(DEV), seq_idx=seq.to(DEV), **kw)
+            plan = cc.kernel_plan_fwd(xg, w.to(DEV), seq_idx=seq.to(DEV))
+        elif mode == "state":
+            S_in, S_out = ri(W - 1, 9), ri(1, 9)
+            init = torch.randn(B, C, S_in, generator=g).to(dtype)
+            want, want_state = co.conv1d_fwd(x, w, b, mask=mask, activation=act, residual=res, initial_state=init,
+                                             final_state_len=S_out)
+            fs = torch.full((B, C, S_out), float("nan"), dtype=dtype, device=DEV)
+            got, _ = cc.causal_conv1d_fn(xg, w.to(DEV), None if b is None else b.to(DEV), initial_states=init.to(DEV),
+                                         final_states_out=fs, **kw)
+            assert torch.equal(bits(fs), bits(want_state)), what
+            plan = cc.kernel_plan_fwd(xg, w.to(DEV))
+        else:
+            want = co.conv1d_fwd(x, w, b, mask=mask, activation=act, residual=res)
+            got = cc.causal_conv1d_fn(xg, w.to(DEV), None if b is None else b.to(DEV), **kw)
+            plan = cc.kernel_plan_fwd(xg, w.to(DEV))
+        plans[plan] = plans.get(plan, 0) + 1
+        added = None if not res else (x if res == "unmasked" else xm)      # the term the sum may cancel against
+        assert_parity(got, want, exact=act is None, what=what, res=added)
+    # the draw reaches every kernel family
+    assert set(plans) >= {"bcl_vec", "blc_vec", "blc_vec_seq", "generic"}, plans
+
+
+def test_randomised_decode_steps(cc):
+    """200 seeded random decode calls: dtypes, widths, state lengths, strided states, token masks, residual
+    modes, ring-buffer and state-pool addressing, each carried for three steps against the oracle."""
+    g = torch.Generator().manual_seed(4048)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    def pick(seq):
+        return seq[ri(0, len(seq) - 1)]
+
+    for case in range(200):
+        dtype = pick([torch.bfloat16, torch.float32, torch.float16])
+        W = pick([2, 3, 4])
+        S = pick([s for s in (1, 2, 3, 4, 5, 8, 9) if s >= W - 1])
+        B, C = ri(1, 5), pick([1, 4, 8, 12, 24, 64, 264, 1032])
+        act = pick([None, "silu"])
+        mode = pick(["plain", "plain", "ring", "pool", "strided"])
+        res = pick([False, True])
+        w = (torch.randn(C, W, generator=g) * 0.4).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.2).to(dtype) if ri(0, 1) else None
+        rows = B + 2 if mode == "pool" else B
+        state_ref = torch.randn(rows, C, S, generator=g).to(dtype)
+        if mode == "strided":
+            big = torch.zeros(rows, C, S + 3, dtype=dtype, device=DEV)
+            state_gpu = big[:, :, 1:S + 1]
+            state_gpu.copy_(state_ref.to(DEV))
+        else:
+            state_gpu = state_ref.to(DEV)
+        idx = torch.randperm(rows, generator=g)[:B].to(torch.int32) if mode == "pool" else None
+        for step in range(3):
+            x = torch.randn(B, C, generator=g).to(dtype)
+            sl = torch.randint(0, 50, (B,), generator=g).to(torch.int32) if mode == "ring" else None
+            want = co.conv1d_update_ext(x, state_ref, w, b, activation=act, residual=res, cache_seqlens=sl,
+                                        conv_state_indices=idx)
+            got = cc.causal_conv1d_update(x.to(DEV), state_gpu, w.to(DEV), None if b is None else b.to(DEV), activation=act,
+                                          residual=res, cache_seqlens=None if sl is None else sl.to(DEV),
+                                          conv_state_indices=None if idx is None else idx.to(DEV))
+            what = f"case {case}: {dtype} {B}x{C} W{W} S{S} {act} res{res} {mode} step{step}"
+            assert_parity(got, want, exact=act is None, what=what, res=x if res else None)
+            assert torch.equal(bits(state_gpu), bits(state_ref)), what

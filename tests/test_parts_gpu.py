@@ -227,6 +227,8 @@ def test_parts_gradients_and_errors(cc):
     torch.testing.assert_close(torch.cat([x.grad for x in xs], dim=1), x_cat.grad, rtol=1e-6, atol=1e-6)
     torch.testing.assert_close(w.grad, w2.grad, rtol=1e-6, atol=1e-6)
 
+    assert "CanonConvPartsFn" in type(outs[0].grad_fn).__name__     # one node over the parts, no cat
+
     a = torch.randn(2, 16, 24, device=DEV)
     with pytest.raises(ValueError, match="Input dim 32 does not match weight dim 24"):
         cc.causal_conv1d_fn_parts([a, a], w.detach())
@@ -236,3 +238,47 @@ def test_parts_gradients_and_errors(cc):
         cc.causal_conv1d_fn_parts([a[:, :16], a[:, :8, :20]], w.detach())
     with pytest.raises(ValueError, match="one dtype and device"):
         cc.causal_conv1d_fn_parts([a[:, :16], a[:, :8].half()], w.detach())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_parts_backward_runs_per_part_without_a_cat(cc, dtype):
+    """Gate/up at the model's width: dx of every part is bit-identical to the matching channels of
+    the single-tensor backward on the concatenation (same per-channel arithmetic), dweight / dbias
+    agree to summation order, and against the float64 autograd of the eager formulation."""
+    from oracle.canon_grad import conv1d_grads
+    torch.manual_seed(11)
+    B, L, dims = 4, 256, (1728, 1728)
+    C = sum(dims)
+    big = torch.randn(B, L, C).to(dtype)
+    mask = torch.ones(B, L)
+    mask[1, 200:] = 0
+    mask[3, 31:] = 0
+    w = torch.randn(C, 4) * 0.3
+    bias = torch.randn(C) * 0.1
+    dout = torch.randn(B, L, C).to(dtype)
+
+    def leaf(t):
+        return t.to(DEV).requires_grad_()
+
+    xs = [leaf(big[..., c0:c0 + d].contiguous()) for c0, d in zip((0, dims[0]), dims)]
+    wg, bg = leaf(w), leaf(bias)
+    outs = cc.causal_conv1d_fn_parts([x.transpose(1, 2) for x in xs], wg, bg, activation="silu",
+                                     attention_mask=mask.to(DEV), residual=True)
+    douts = [dout[..., c0:c0 + d].to(DEV).transpose(1, 2) for c0, d in zip((0, dims[0]), dims)]
+    torch.autograd.backward(outs, douts)
+
+    xc = leaf(big)
+    wc, bc = leaf(w), leaf(bias)
+    yc = cc.causal_conv1d_fn(xc.transpose(1, 2), wc, bc, activation="silu", attention_mask=mask.to(DEV),
+                             residual=True)
+    yc.backward(dout.to(DEV).transpose(1, 2))
+    torch.cuda.synchronize()
+    assert torch.equal(bits(torch.cat([o.transpose(1, 2) for o in outs], dim=-1)), bits(yc.transpose(1, 2)))
+    assert torch.equal(bits(torch.cat([x.grad for x in xs], dim=-1)), bits(xc.grad))
+    torch.testing.assert_close(wg.grad, wc.grad, rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(bg.grad, bc.grad, rtol=1e-5, atol=1e-4)
+
+    _, dw64, db64, _ = conv1d_grads(big.transpose(1, 2), w, bias, dout.transpose(1, 2), mask=mask,
+                                    activation="silu", residual="masked")
+    assert (wg.grad.cpu().double() - dw64).abs().max().item() <= 1e-4 * dw64.abs().max().item()
+    assert (bg.grad.cpu().double() - db64).abs().max().item() <= 1e-4 * db64.abs().max().item()

@@ -345,47 +345,55 @@ class _CanonConvFn(torch.autograd.Function):
     def backward(ctx, dout, *unused):
         x, weight, bias, mask = ctx.saved_tensors
         act, res = ctx.flags
-        if dout.dtype != x.dtype:
-            dout = dout.to(x.dtype)
-        if dout.stride() != x.stride():
-            dout = torch.empty_like(x).copy_(dout)       # same layout as x: keeps the vector kernel
-        dx = torch.empty_like(x)
         channels, width = weight.shape
         dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
         dbias = torch.empty(channels, dtype=torch.float32, device=x.device) if bias is not None else None
-        p = _lib.BwdParams()
-        p.struct_size = ctypes.sizeof(_lib.BwdParams)
-        p.x_dtype = _lib.DTYPE_CODE[x.dtype]
-        p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
-        p.width = width
-        p.activation, p.residual_mode = act, res
-        p.batch, p.channels, p.seqlen = x.shape
-        p.x = x.data_ptr()
-        p.x_stride_b, p.x_stride_c, p.x_stride_l = x.stride()
-        p.dout = dout.data_ptr()
-        p.dout_stride_b, p.dout_stride_c, p.dout_stride_l = dout.stride()
-        p.dx = dx.data_ptr()
-        p.dx_stride_b, p.dx_stride_c, p.dx_stride_l = dx.stride()
-        p.weight = weight.data_ptr()
-        p.w_stride_c, p.w_stride_k = weight.stride()
-        p.bias = bias.data_ptr() if bias is not None else None
-        if mask is not None:
-            p.mask = mask.data_ptr()
-            p.mask_dtype = _lib.MASK_CODE[mask.dtype]
-            p.mask_stride_b, p.mask_stride_l = mask.stride()
-        p.dweight = dweight.data_ptr()
-        p.dbias = dbias.data_ptr() if dbias is not None else None
-        L = _lib.lib()
-        nbytes = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(p))
-        if nbytes < 0:
-            _lib.check(_lib.ERR_INVALID_ARGUMENT, "causal_conv1d_fn backward")
-        workspace = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=x.device)
-        p.workspace = workspace.data_ptr()
-        p.workspace_bytes = workspace.numel()
-        rc = _call(L.canon_conv1d_bwd, x.device, ctypes.byref(p))
-        _lib.check(rc, "causal_conv1d_fn backward")
+        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res)
         return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
                 None, None, None, None, None)
+
+
+def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res) -> torch.Tensor:
+    """One backward launch (+ the fixed-order reduction): returns dx with x's strides and fills the
+    fp32 ``dweight`` (channels, W) / ``dbias`` (channels,) given (rows of larger tensors are fine)."""
+    if dout.dtype != x.dtype:
+        dout = dout.to(x.dtype)
+    if dout.stride() != x.stride():
+        dout = torch.empty_like(x).copy_(dout)       # same layout as x: keeps the vector kernel
+    dx = torch.empty_like(x)
+    width = weight.shape[1]
+    p = _lib.BwdParams()
+    p.struct_size = ctypes.sizeof(_lib.BwdParams)
+    p.x_dtype = _lib.DTYPE_CODE[x.dtype]
+    p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
+    p.width = width
+    p.activation, p.residual_mode = act, res
+    p.batch, p.channels, p.seqlen = x.shape
+    p.x = x.data_ptr()
+    p.x_stride_b, p.x_stride_c, p.x_stride_l = x.stride()
+    p.dout = dout.data_ptr()
+    p.dout_stride_b, p.dout_stride_c, p.dout_stride_l = dout.stride()
+    p.dx = dx.data_ptr()
+    p.dx_stride_b, p.dx_stride_c, p.dx_stride_l = dx.stride()
+    p.weight = weight.data_ptr()
+    p.w_stride_c, p.w_stride_k = weight.stride()
+    p.bias = bias.data_ptr() if bias is not None else None
+    if mask is not None:
+        p.mask = mask.data_ptr()
+        p.mask_dtype = _lib.MASK_CODE[mask.dtype]
+        p.mask_stride_b, p.mask_stride_l = mask.stride()
+    p.dweight = dweight.data_ptr()
+    p.dbias = dbias.data_ptr() if dbias is not None else None
+    L = _lib.lib()
+    nbytes = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(p))
+    if nbytes < 0:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "causal_conv1d_fn backward")
+    workspace = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=x.device)
+    p.workspace = workspace.data_ptr()
+    p.workspace_bytes = workspace.numel()
+    rc = _call(L.canon_conv1d_bwd, x.device, ctypes.byref(p))
+    _lib.check(rc, "causal_conv1d_fn backward")
+    return dx
 
 
 def _fill_update(x2, out2, conv_state, weight, bias, token_mask, act, res, rnd) -> UpdateParams:
@@ -551,8 +559,8 @@ def causal_conv1d_fn_parts(
     states cover all channels in the order of the parts.  Returns the tuple of outputs, one per
     part with that part's strides (and the final states when asked for).  This is what Canon-B /
     Canon-D need (``model/model.py:772-789, 962-971`` concatenate q/k/v and gate/up only to call
-    the conv once); results equal the call on the concatenation bit for bit.  When a gradient is
-    required the parts are concatenated and the differentiable single-tensor call is used.
+    the conv once); results equal the call on the concatenation bit for bit.  Differentiable:
+    the backward runs once per part on that part's rows of the weights (no cat there either).
     """
     act = _activation_flag(activation)
     res = _residual_mode(residual)
@@ -567,24 +575,61 @@ def causal_conv1d_fn_parts(
     if batch * dim * seqlen == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
-    if _wants_grad(*xs, weight, bias):
-        result = causal_conv1d_fn(
-            torch.cat(xs, dim=1), weight, bias, initial_states=initial_states, final_states_out=final_states,
-            activation=activation, attention_mask=attention_mask, residual=residual, rounding=rounding)
-        y = result[0] if final_states is not None else result
-        outs = tuple(y.split(dims, dim=1))
-        return (outs, final_states) if final_states is not None else outs
-
     xs = [x if (x.stride(2) == 1 or x.stride(1) == 1) else x.contiguous() for x in xs]
+    if _wants_grad(*xs, weight, bias):
+        if initial_states is not None:
+            raise NotImplementedError("gradients through a call with initial_states are not implemented")
+        result = _CanonConvPartsFn.apply(weight, bias, attention_mask, final_states, act, res, rnd, *xs)
+        outs = tuple(result[:len(xs)])
+    else:
+        outs = _launch_fwd_parts(xs, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+    return (outs, final_states) if final_states is not None else outs
+
+
+def _launch_fwd_parts(xs, weight, bias, mask, initial_states, final_states, act, res, rnd):
     outs = tuple(torch.empty_like(x) for x in xs)
-    if batch * dim * seqlen:
-        p = _fill_fwd(xs[0], outs[0], weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
+    dim = sum(x.shape[1] for x in xs)
+    if xs[0].shape[0] * dim * xs[0].shape[2]:
+        p = _fill_fwd(xs[0], outs[0], weight, bias, mask, initial_states, final_states, act, res, rnd)
         p.channels = dim
         p.x = p.out = None
         arr = _part_array(xs, outs)
         rc = _call(_lib.lib().canon_conv1d_fwd_parts, xs[0].device, ctypes.byref(p), arr, len(xs))
         _lib.check(rc, "causal_conv1d_fn_parts")
-    return (outs, final_states) if final_states is not None else outs
+    return outs
+
+
+class _CanonConvPartsFn(torch.autograd.Function):
+    """Autograd node of the multi-part prefill: one forward launch over all parts; the backward
+    runs the fused backward once per part, on that part's rows of weight / bias, so neither
+    direction concatenates anything."""
+
+    @staticmethod
+    def forward(ctx, weight, bias, mask, final_states, act, res, rnd, *xs):
+        outs = _launch_fwd_parts(xs, weight, bias, mask, None, final_states, act, res, rnd)
+        ctx.save_for_backward(weight, bias, mask, *xs)
+        ctx.flags = (act, res)
+        if final_states is not None:
+            ctx.mark_non_differentiable(final_states)
+            return (*outs, final_states)
+        return outs
+
+    @staticmethod
+    def backward(ctx, *douts):
+        weight, bias, mask, *xs = ctx.saved_tensors
+        act, res = ctx.flags
+        channels, width = weight.shape
+        dev = xs[0].device
+        dweight = torch.empty(channels, width, dtype=torch.float32, device=dev)
+        dbias = torch.empty(channels, dtype=torch.float32, device=dev) if bias is not None else None
+        dxs, c0 = [], 0
+        for x, dout in zip(xs, douts):
+            c1 = c0 + x.shape[1]
+            dxs.append(_launch_bwd(x, dout, weight[c0:c1], bias[c0:c1] if bias is not None else None, mask,
+                                   dweight[c0:c1], dbias[c0:c1] if dbias is not None else None, act, res))
+            c0 = c1
+        return (dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
+                None, None, None, None, None, *dxs)
 
 
 def causal_conv1d_update_parts(

@@ -12,12 +12,11 @@ namespace canon {
 // canon_bwd_reduce_kernel sums the sets in a fixed order.
 //
 // canon_bwd_walk_kernel, the fallback for layouts without a vector kernel
-// (instantiated with E = 1, VEC = false: any strides): one lane owns a channel
-// and walks a chunk of time steps from its END to its start.  dx[t] needs
-// dz[t .. t+W-1] (the three later steps are carried in registers), z[t] needs
-// xm[t-3 .. t] (a sliding window refilled with one row per step, fetched R
-// rows ahead).  The three dz values just past the chunk are recomputed from
-// memory.
+// (any strides): one lane owns a channel and walks a chunk of time steps from
+// its END to its start.  dx[t] needs dz[t .. t+W-1] (the three later steps are
+// carried in registers), z[t] needs xm[t-3 .. t] (a sliding window refilled
+// with one row per step, fetched R rows ahead).  The three dz values just past
+// the chunk are recomputed from memory.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float silu_grad(float z)
 {
@@ -25,21 +24,11 @@ __device__ __forceinline__ float silu_grad(float z)
     return s * (1.0f + z * (1.0f - s));
 }
 
-template <int DT, int E, bool VEC>
-__device__ __forceinline__ void bwd_load_row(const char *base, int64_t row_off, int64_t sc, float *f)
-{
-    // E values of one time step; VEC: 16 contiguous bytes at base + row_off (bytes)
-    if constexpr (VEC) {
-        unpack_vec<DT>(load_vec<false>(base + row_off), f);
-    } else {
-        f[0] = load1<DT>(base + row_off, 0);
-    }
-}
-
-template <int DT, int W, int E, bool VEC, bool MASK, int R>
+template <int DT, int W, bool MASK, int R>
 __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 {
     constexpr int BY = Elem<DT>::bytes;
+    constexpr int E = 1;     // channels per lane
     const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
     if (tid >= a.nthreads) return;
     const uint32_t bc = fdiv(tid, a.div_nvec);
@@ -58,7 +47,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     const int64_t Lm1 = (int64_t)a.L - 1;
 
     RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, VEC && a.w_vec != 0, VEC && a.b_vec != 0, c0, raw);
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, false, false, c0, raw);
 
     // rows t_end-4 .. t_end+2 of xm (window for the last step + the three steps past the chunk)
     float xr7[7][E], m7[7];
@@ -66,19 +55,19 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     for (int j = 0; j < 7; ++j) {
         const int64_t t = t_end - 4 + j;
         const int64_t tc = t < 0 ? 0 : (t > Lm1 ? Lm1 : t);
-        bwd_load_row<DT, E, VEC>(xb, tc * xs, a.x_sc, xr7[j]);
+        xr7[j][0] = load1<DT>(xb + tc * xs, 0);
         m7[j] = 1.0f;
     }
     float g3[3][E];
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
         const int64_t t = t_end + j;
-        bwd_load_row<DT, E, VEC>(gb, (t > Lm1 ? Lm1 : t) * gs, a.g_sc, g3[j]);
+        g3[j][0] = load1<DT>(gb + (t > Lm1 ? Lm1 : t) * gs, 0);
     }
     if constexpr (MASK) load_mask_rows<7>(a.mask, (int64_t)b * a.m_sb, t_end - 4, a.L, a.m_sl, a.mask_dtype, m7);
 
     float w[E][W], bias[E];
-    decode_taps<DT, W, E>(raw, a.w_dtype, VEC && a.w_vec != 0, a.bias != nullptr, w, bias);
+    decode_taps<DT, W, E>(raw, a.w_dtype, false, a.bias != nullptr, w, bias);
 
 #pragma unroll
     for (int j = 0; j < 7; ++j) {
@@ -122,20 +111,15 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     for (int64_t t_hi = t_end - 1; t_hi >= t_begin; t_hi -= R) {
         // this batch: steps t_hi, t_hi-1, .., t_hi-R+1; needs dout of those steps and x rows t-4.
         // Rows are kept as loaded (raw) until their step, to keep the register count down.
-        typename std::conditional<VEC, uint4, float>::type G[R], XN[R];
+        float G[R], XN[R];
         float mk[R], mn[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t t = t_hi - r;
             const int64_t tg = t < 0 ? 0 : t;
             const int64_t tn = t - 4 < 0 ? 0 : t - 4;
-            if constexpr (VEC) {
-                G[r] = load_vec<false>(gb + tg * gs);
-                XN[r] = load_vec<false>(xb + tn * xs);
-            } else {
-                G[r] = load1<DT>(gb + tg * gs, 0);
-                XN[r] = load1<DT>(xb + tn * xs, 0);
-            }
+            G[r] = load1<DT>(gb + tg * gs, 0);
+            XN[r] = load1<DT>(xb + tn * xs, 0);
             mk[r] = 1.0f;
             mn[r] = 1.0f;
         }
@@ -154,13 +138,8 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
             const int64_t t = t_hi - r;
             if (t < t_begin) break;
             float g[E], xn[E], dz[E], o[E];
-            if constexpr (VEC) {
-                unpack_vec<DT>(G[r], g);
-                unpack_vec<DT>(XN[r], xn);
-            } else {
-                g[0] = G[r];
-                xn[0] = XN[r];
-            }
+            g[0] = G[r];
+            xn[0] = XN[r];
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 float z = bias[e];
@@ -213,11 +192,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
                 xw[1][e] = xw[0][e];
                 xw[0][e] = has_row ? v : 0.0f;
             }
-            if constexpr (VEC) {
-                store_vec<false>(db_ + t * ds, pack_vec<DT>(o));
-            } else {
-                store1<DT>(db_ + t * ds, 0, o[0]);
-            }
+            store1<DT>(db_ + t * ds, 0, o[0]);
         }
     }
 
@@ -893,7 +868,7 @@ template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStre
         else hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, false>), g, b, 0, s, pl.args);
     }
     else
-        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, 1, false, MASK, kBwdRows>), g, b, 0, s, pl.args);
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, MASK, kBwdRows>), g, b, 0, s, pl.args);
 }
 
 template <int DT> void launch_bwd(const BwdPlan &pl, hipStream_t s)

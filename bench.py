@@ -226,9 +226,23 @@ def bench_backward(steps, warmup, nbuf):
     return ms, plan, ws.numel()
 
 
-def cpu_baseline(budget_s=12.0):
-    """The reference's eager formulation (mask-free Canon-D call: pad + grouped
-    conv1d + residual, model/model.py:604-675) on the host cores, same shape."""
+def _median_time(fn, budget_s, max_runs):
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < max_runs):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times)
+
+
+def cpu_baseline(budget_s=10.0):
+    """The reference's eager formulation on the host cores, same shapes: the mask-free Canon-D
+    block call (pad + grouped conv1d + residual, model/model.py:604-675) on all threads torch
+    uses and on one, and the single-token step (roll + write + multiply + sum,
+    model/model.py:372-398) at the decode shape."""
     import torch
     from oracle.canon_eager import EagerCanon
     cores = torch.get_num_threads()
@@ -237,20 +251,32 @@ def cpu_baseline(budget_s=12.0):
     w = (torch.randn(C, W, generator=g) * 0.02).bfloat16()
     bias = (torch.randn(C, generator=g) * 0.01).bfloat16()
     layer = EagerCanon(w, bias, False)
-    layer.forward(x)
-    times = []
-    t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
-        t0 = time.perf_counter()
-        layer.forward(x)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    med, n = _median_time(lambda: layer.forward(x), budget_s, 50)
+
+    cache = {}
+    tok = torch.randn(DEC_B, 1, C, generator=g).bfloat16()
+    layer.forward(tok, cache=cache, key=0)      # creates the 8-slot state the eager module keeps
+    med_dec, n_dec = _median_time(lambda: layer.forward(tok, cache=cache, key=0), budget_s / 4, 50)
+    dec_bytes = decode_bytes(DEC_B, C, 8)
+
+    torch.set_num_threads(1)
+    try:
+        med1, n1 = _median_time(lambda: layer.forward(x), budget_s / 2, 10)
+    finally:
+        torch.set_num_threads(cores)
+    nbytes = prefill_bytes(B, C, L)
     return {
-        "value": round(prefill_bytes(B, C, L) / med / 1e9, 3), "unit": "GB/s", "cores": cores,
+        "value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": cores,
         "kind": "port",
-        "sample": f"{len(times)} passes of the full bf16 [8,3456,1024] step, eager torch restatement "
+        "sample": f"{n} passes of the full bf16 [8,3456,1024] step, eager torch restatement "
                   f"(oracle/canon_eager.py), median {med * 1e3:.1f} ms",
+        "ms": round(med * 1e3, 2), "tokens_per_s": round(B * L / med),
+        "one_core": {"value": round(nbytes / med1 / 1e9, 3), "unit": "GB/s", "ms": round(med1 * 1e3, 1),
+                     "sample": f"{n1} passes, torch.set_num_threads(1)"},
+        "decode": {"us_per_step": round(med_dec * 1e6, 1), "GB/s": round(dec_bytes / med_dec / 1e9, 3),
+                   "cores": cores,
+                   "sample": f"{n_dec} single-token steps, bf16 [{DEC_B},{C}] token, 8-slot state "
+                             f"(the eager module's), roll + write + multiply + sum"},
     }
 
 

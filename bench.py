@@ -106,6 +106,21 @@ def bench_prefill(layout, steps, warmup, nbuf):
     return ms, plan
 
 
+def bench_copy(steps, warmup, nbuf):
+    """What the runtime's own device-to-device copy of one x-sized buffer reaches on this GPU with the
+    same buffer rotation: the same bytes as a kernel that reads x once and writes out once."""
+    import torch
+    n = B * C * L
+    pool = torch.empty(2 * nbuf * n, dtype=torch.bfloat16, device="cuda:0").normal_()
+    pairs = [(pool[2 * i * n:(2 * i + 1) * n], pool[(2 * i + 1) * n:(2 * i + 2) * n]) for i in range(nbuf)]
+
+    def step(i):
+        src, dst = pairs[i % nbuf]
+        dst.copy_(src)
+
+    return time_region(step, steps, warmup)
+
+
 def bench_prefill_parts(steps, warmup, nbuf):
     """Canon-D as the model produces it: gate and up projections as two (B, L, C/2) tensors, convolved
     by one multi-part launch (no torch.cat, outputs stay split)."""
@@ -307,6 +322,7 @@ def main():
 
     nbuf = 6  # 6 x 113 MB = 680 MB of distinct traffic between reuses
     ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
+    ms_copy = bench_copy(args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
     ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
     dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
@@ -323,6 +339,9 @@ def main():
                                "bias, residual fused, no activation", "kernel": plan,
                    "rotating_buffer_pairs": nbuf},
         "tokens_per_s": round(B * L / (ms * 1e-3)),
+        "device_copy_same_bytes": {"ms_per_step": round(ms_copy, 6),
+                                   "GB/s": round(2 * B * C * L * 2 / (ms_copy * 1e-3) / 1e9, 1),
+                                   "what": "torch copy_ (the runtime's device-to-device copy) of one x-sized buffer, same rotation"},
         "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
                                  "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1)},
         "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",

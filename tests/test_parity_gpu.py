@@ -528,7 +528,8 @@ def test_update_ring_buffer_and_state_pool(cc, dtype):
         ring_ref = torch.randn(B, C, S, generator=g).to(dtype)
         idx = torch.randperm(rows, generator=g)[:B].to(torch.int32)
         pool_gpu, ring_gpu = pool_ref.to(DEV), ring_ref.to(DEV)
-        expect_plan = "update_vec" if (S in (3, 4, 8) and C % (16 // w.element_size()) == 0) else "update_generic"
+        lane_channels = 2 if (w.element_size() == 2 and S != 8) else 1     # a lane owns 12..16 bytes of state
+        expect_plan = "update_vec" if (S in (3, 4, 8) and C % lane_channels == 0) else "update_generic"
         assert cc.kernel_plan_update(torch.empty(B, C, dtype=dtype, device=DEV), pool_gpu[:B], w.to(DEV)) == expect_plan
         for step in range(S + 2):
             x = torch.randn(B, C, generator=g).to(dtype)

@@ -241,21 +241,28 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
     a.b_vec = p->bias && aligned16(p->bias);
+    a.tap_mode = TAPS_ANY;
+    if (a.w_vec && (uintptr_t)p->bias % 4 == 0) {
+        if (p->w_dtype == p->x_dtype) a.tap_mode = TAPS_SAME;
+        else if (p->w_dtype == CANON_DTYPE_F32) a.tap_mode = TAPS_WIDE;
+    }
     plan->kind = UPD_GENERIC;
     plan->grid = 0;
     if (empty) return CANON_OK;
 
-    const int E = 16 / elem_bytes(p->x_dtype);
     const int S = p->state_len;
+    const int BY = elem_bytes(p->x_dtype);
+    const int E = upd_lane_channels(BY, S);           // channels per lane
+    const int XB = E * BY;                            // bytes of x / out per lane (2 or 4)
     const bool vec_ok = !p->cache_seqlens && p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
-                        aligned16(p->x) && aligned16(p->out) && aligned16(p->conv_state) &&
-                        a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb % E == 0 && a.o_sb % E == 0 &&
-                        a.s_ss == 1 && a.s_sc == S && a.s_sb % E == 0;
+                        ((uintptr_t)p->x | (uintptr_t)p->out) % XB == 0 && (uintptr_t)p->conv_state % 4 == 0 &&
+                        a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb * BY % XB == 0 && a.o_sb * BY % XB == 0 &&
+                        a.s_ss == 1 && a.s_sc == S && a.s_sb * BY % 4 == 0;
     if (vec_ok) {
         plan->kind = UPD_VEC;
         a.nvec = a.C / E;
         // two batch rows per lane halve the tap loads; with little work, more waves matter more
-        a.nb = ((uint64_t)a.nvec * a.B / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        a.nb = (S != 8 && (uint64_t)a.nvec * a.B / kUpdNB >= 512 * 64) ? kUpdNB : 1;
         a.bgroups = (a.B + a.nb - 1) / a.nb;
         a.nthreads = a.nvec * a.bgroups;
         a.div_nvec = make_fastdiv(a.nvec);
@@ -372,7 +379,7 @@ int plan_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_pa
     pp->grid = 0;
     if (pp->single) {
         // batch rows per lane chosen on the whole token, the same for every part
-        const uint32_t nb = (nvec_total * (uint64_t)p->batch / kUpdNB >= 512 * 64) ? kUpdNB : 1;
+        const uint32_t nb = (p->state_len != 8 && nvec_total * (uint64_t)p->batch / kUpdNB >= 512 * 64) ? kUpdNB : 1;
         uint64_t blocks = 0;
         for (int i = 0; i < nparts; ++i) {
             UpdPlan &u = pp->part[i];

@@ -7,6 +7,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stddef.h>
 #include <string.h>
 
 #include "canon_conv1d.h"
@@ -56,27 +57,48 @@ struct FwdArgs {
     FastDiv div_nct, div_ntt;
 };
 
+// How a lane of the vectorised update gets its taps and bias.  The two common layouts are straight-line
+// code (every load of the kernel is in flight before the first wait; the general path branches on the
+// run-time weight type between its loads, which costs a wait per branch); which one runs is wave-uniform.
+enum TapMode {
+    TAPS_SAME,   // contiguous, 16-byte aligned [C, 4] weights of x's type (bias too, 4-byte aligned)
+    TAPS_WIDE,   // the same with fp32 weights and bias and 16-bit x
+    TAPS_ANY     // any strides, width and type
+};
+
 struct UpdArgs {
+    // The fields the vectorised kernel reads on its usual path come first, within three 64-byte lines of the
+    // kernel-argument segment: the kernel lives for a few microseconds, so every scalar-cache miss a wave
+    // takes in turn before its first memory request shows in the total.
     const char *x;
     char *out;
     char *state;
     const void *weight;
     const void *bias;
     const void *tmask;
-    const int32_t *seqlens;   // circular-buffer mode: conv_state is written at seqlens[b] % S, not shifted
+    uint32_t nthreads;
+    uint32_t B;
+    uint32_t nvec;      // lanes per batch row (channels / channels per lane)
+    int32_t tap_mode;
+    // second line
+    int64_t x_sb, o_sb, s_sb, m_sb;
+    FastDiv div_nvec;
+    int32_t act, res_mode, mask_dtype, w_dtype;
+    // third line: what the vectorised kernel reads off its usual path (state pool, general tap path)
     const int32_t *indices;   // conv_state row of batch entry b (state pool shared by many sequences)
-    int64_t x_sb, x_sc, o_sb, o_sc;
-    int64_t s_sb, s_sc, s_ss;
     int64_t w_sc, w_sk;
-    int64_t m_sb;
-    uint32_t B, C;
-    int32_t W, S, w_dtype, mask_dtype, act, res_mode, eager, w_vec, b_vec;
-    uint32_t nvec;      // channel vectors per batch row
+    int32_t w_vec, b_vec;
+    // the rest: strided kernel, ring buffer, launch geometry
+    const int32_t *seqlens;   // circular-buffer mode: conv_state is written at seqlens[b] % S, not shifted
+    int64_t x_sc, o_sc;
+    int64_t s_sc, s_ss;
+    uint32_t C;
+    int32_t W, S, eager;
     uint32_t bgroups;   // batch groups (each thread walks nb batch rows)
     uint32_t nb;
-    uint32_t nthreads;
-    FastDiv div_nvec;
 };
+static_assert(offsetof(UpdArgs, x_sb) == 64 && offsetof(UpdArgs, indices) == 128 && offsetof(UpdArgs, x_sc) <= 192,
+              "fields the vectorised update reads: three 64-byte lines");
 
 struct BwdArgs {
     const char *x;
@@ -135,6 +157,9 @@ constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar k
 constexpr int kBlcRows = CANON_BLC_ROWS;   // time steps per wave in the channel-contiguous kernel
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work
+// channels a lane of the vectorised update owns: as many as make its piece of the [B, C, S] state one run
+// of 12 or 16 bytes (fp32 with 8 slots: 32)
+constexpr int upd_lane_channels(int elem_bytes, int S) { return (elem_bytes == 2 && S != 8) ? 2 : 1; }
 enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
 constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
 constexpr int kBwdHalfBlocksPerCU = 3;   // grid target of the channel-contiguous backward, in half blocks per CU

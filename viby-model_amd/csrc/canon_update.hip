@@ -6,27 +6,71 @@ namespace canon {
 
 // ---------------------------------------------------------------------------
 // decode update, vectorised: contiguous [B, C, S] state, channel-contiguous
-// x / out.  One lane owns E adjacent channels: it reads the E*S state
-// elements as S 16-byte vectors (they are one contiguous 16*S-byte run),
-// computes E outputs, and writes the run back shifted by one element per
-// channel with the new token in the last slot -- one fused gather / shift /
-// write, no second pass.  Each lane walks NB batch rows so the taps are
-// fetched once per NB tokens.
+// x / out.  One lane owns the state rows of E adjacent channels, E chosen so
+// that they are ONE run of at most 16 bytes (16-bit: two channels for S = 3 or
+// 4, one for S = 8; fp32: one channel, 32 bytes for S = 8): a wave then reads
+// and writes one dense stretch of the state per instruction, which is what
+// the memory pipeline wants -- wider lanes (eight channels each, the lanes of
+// a wave 48..128 bytes apart) ran 1.5-2x slower.  The lane computes its E
+// outputs and writes the run back shifted by one element per channel with the
+// new token in the last slot: one fused gather / shift / write, no second
+// pass.  Each lane walks NB batch rows so the taps are fetched once per NB
+// tokens.
 // ---------------------------------------------------------------------------
-template <int DT> struct StateRun {
-    // element i of a run of uint4 vectors, as raw bits of the storage type
-    static __device__ __forceinline__ uint32_t get(const uint4 *v, int i)
+typedef uint32_t words2_t __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t words3_t __attribute__((ext_vector_type(3), aligned(4)));
+typedef uint32_t words4_t __attribute__((ext_vector_type(4), aligned(4)));
+
+// N consecutive 32-bit words at a 4-byte aligned address
+template <int N> __device__ __forceinline__ void load_words(const char *p, uint32_t *d)
+{
+    if constexpr (N == 1) {
+        d[0] = *(const uint32_t *)p;
+    } else if constexpr (N == 2) {
+        const words2_t q = *(const words2_t *)p;
+        d[0] = q.x; d[1] = q.y;
+    } else if constexpr (N == 3) {
+        const words3_t q = *(const words3_t *)p;
+        d[0] = q.x; d[1] = q.y; d[2] = q.z;
+    } else if constexpr (N == 4) {
+        const words4_t q = *(const words4_t *)p;
+        d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+    } else {
+        load_words<4>(p, d);
+        load_words<N - 4>(p + 16, d + 4);
+    }
+}
+
+template <int N> __device__ __forceinline__ void store_words(char *p, const uint32_t *d)
+{
+    if constexpr (N == 1) {
+        *(uint32_t *)p = d[0];
+    } else if constexpr (N == 2) {
+        words2_t q; q.x = d[0]; q.y = d[1];
+        *(words2_t *)p = q;
+    } else if constexpr (N == 3) {
+        words3_t q; q.x = d[0]; q.y = d[1]; q.z = d[2];
+        *(words3_t *)p = q;
+    } else if constexpr (N == 4) {
+        words4_t q; q.x = d[0]; q.y = d[1]; q.z = d[2]; q.w = d[3];
+        *(words4_t *)p = q;
+    } else {
+        store_words<4>(p, d);
+        store_words<N - 4>(p + 16, d + 4);
+    }
+}
+
+// elements of the storage type packed in 32-bit words, handled as raw bits
+template <int DT> struct Packed {
+    static __device__ __forceinline__ uint32_t get(const uint32_t *d, int i)
     {
-        if constexpr (DT == CANON_DTYPE_F32) {
-            const uint4 &q = v[i >> 2];
-            const int d = i & 3;
-            return d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
-        } else {
-            const uint4 &q = v[i >> 3];
-            const int d = (i >> 1) & 3;
-            const uint32_t u = d == 0 ? q.x : d == 1 ? q.y : d == 2 ? q.z : q.w;
-            return (i & 1) ? (u >> 16) : (u & 0xFFFFu);
-        }
+        if constexpr (DT == CANON_DTYPE_F32) return d[i];
+        else return (i & 1) ? (d[i >> 1] >> 16) : (d[i >> 1] & 0xFFFFu);
+    }
+    static __device__ __forceinline__ void put(uint32_t *d, int i, uint32_t raw)   // d starts as zeros
+    {
+        if constexpr (DT == CANON_DTYPE_F32) d[i] = raw;
+        else d[i >> 1] |= (i & 1) ? (raw << 16) : raw;
     }
     static __device__ __forceinline__ float as_float(uint32_t raw)
     {
@@ -34,7 +78,7 @@ template <int DT> struct StateRun {
         else if constexpr (DT == CANON_DTYPE_BF16) return bits_f(raw << 16);
         else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
     }
-    static __device__ __forceinline__ uint32_t raw_of(float f)   // exact for values already representable
+    static __device__ __forceinline__ uint32_t raw_of(float f)   // rounds to nearest even
     {
         if constexpr (DT == CANON_DTYPE_F32) return f_bits(f);
         else if constexpr (DT == CANON_DTYPE_BF16) return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
@@ -42,35 +86,37 @@ template <int DT> struct StateRun {
     }
 };
 
-template <int DT, int W, int S, int NB, bool POOL = false>
-__device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_t blk)
+template <int DT, int W, int S, int NB, int MODE>
+__device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t bg, const uint32_t c0,
+                                                const uint32_t (*X)[(upd_lane_channels(Elem<DT>::bytes, S) * Elem<DT>::bytes + 3) / 4],
+                                                const uint32_t (*ST)[upd_lane_channels(Elem<DT>::bytes, S) * S * Elem<DT>::bytes / 4],
+                                                const uint32_t *srow)
 {
-    constexpr int E = Elem<DT>::per_vec;
     constexpr int BY = Elem<DT>::bytes;
-    const uint32_t tid = blk * 256u + threadIdx.x;
-    if (tid >= a.nthreads) return;
-    const uint32_t bg = fdiv(tid, a.div_nvec);
-    const uint32_t cv = tid - bg * a.nvec;
-    const uint32_t c0 = cv * E;
+    constexpr int E = upd_lane_channels(BY, S);
+    constexpr int ND = E * S * BY / 4;
+    constexpr int NX = (E * BY + 3) / 4;
+    constexpr int WDT = MODE == TAPS_WIDE ? CANON_DTYPE_F32 : DT;      // weight type of the straight-line modes
+    constexpr int WBY = Elem<WDT>::bytes;
+    constexpr int NT = MODE == TAPS_ANY ? 1 : E * WBY;                  // words of taps: 4 * WBY bytes per channel
+    constexpr int NBW = MODE == TAPS_ANY ? 1 : (E * WBY + 3) / 4;       // words of bias
 
-    uint4 X[NB];
-    uint4 ST[NB][S];
-    float tm[NB];
-    uint32_t srow[NB];   // conv_state row of each batch entry
-#pragma unroll
-    for (int n = 0; n < NB; ++n) {
-        const uint32_t b = bg * NB + n;
-        tm[n] = 1.0f;
-        if (b < a.B) {
-            X[n] = *(const uint4 *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
-            srow[n] = POOL ? (uint32_t)a.indices[b] : b;   // POOL: rows of a state pool (conv_state_indices)
-            const uint4 *sp = (const uint4 *)(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY);
-#pragma unroll
-            for (int k = 0; k < S; ++k) ST[n][k] = sp[k];
+    uint32_t tw[NT], tb[NBW] = {};
+    RawTaps<E> raw;
+    if constexpr (MODE == TAPS_ANY) {
+        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
+    } else {
+        static_assert(MODE == TAPS_ANY || W == 4, "the contiguous tap layouts are [C, 4]");
+        load_words<NT>((const char *)a.weight + (int64_t)c0 * 4 * WBY, tw);
+        if (a.bias) {
+            const char *bp = (const char *)a.bias + (int64_t)c0 * WBY;
+            if constexpr (E * WBY == 2) tb[0] = *(const uint16_t *)bp;
+            else load_words<NBW>(bp, tb);
         }
     }
-    RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_vec != 0, c0, raw);
+    float tm[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) tm[n] = 1.0f;
     if (a.tmask) {
         // token masks last and in one go (one element-type switch, one wait)
         int64_t mbase[NB];
@@ -85,14 +131,25 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
         for (int n = 0; n < NB; ++n) tm[n] = tmv[n][0];
     }
     float w[E][W], bias[E];
-    decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+    if constexpr (MODE == TAPS_ANY) {
+        decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+    } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int k = 0; k < W; ++k)
+                w[e][k] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(tw, e * 4 + k)));
+            bias[e] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(tb, e)));   // zero bits without a bias
+        }
+    }
 
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
         const uint32_t b = bg * NB + n;
         if (b >= a.B) continue;
         float xr[E], xt[E], o[E];
-        unpack_vec<DT>(X[n], xr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) xr[e] = Packed<DT>::as_float(Packed<DT>::get(X[n], e));
         if (a.tmask) {
 #pragma unroll
             for (int e = 0; e < E; ++e) xt[e] = mul_round<DT>(xr[e], tm[n]);
@@ -105,7 +162,7 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
             float acc = bias[e];
 #pragma unroll
             for (int k = 0; k < W - 1; ++k)
-                acc = fmaf(w[e][k], StateRun<DT>::as_float(StateRun<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
+                acc = fmaf(w[e][k], Packed<DT>::as_float(Packed<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
             o[e] = fmaf(w[e][W - 1], xt[e], acc);
         }
         if (a.act) {
@@ -119,35 +176,69 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
 #pragma unroll
             for (int e = 0; e < E; ++e) o[e] += xr[e];
         }
-        *(uint4 *)(a.out + ((int64_t)b * a.o_sb + c0) * BY) = pack_vec<DT>(o);
+        uint32_t ow[NX] = {};
+#pragma unroll
+        for (int e = 0; e < E; ++e) Packed<DT>::put(ow, e, Packed<DT>::raw_of(o[e]));
+        char *op = a.out + ((int64_t)b * a.o_sb + c0) * BY;
+        if constexpr (E * BY == 2) *(uint16_t *)op = (uint16_t)ow[0];
+        else store_words<NX>(op, ow);
 
-        // new run: element (e, k) <- old (e, k+1); (e, S-1) <- token
-        uint32_t raw[E * S];
+        // new run: element (e, k) <- old (e, k+1); (e, S-1) <- token (its own bits unless a mask scaled it)
+        uint32_t nw[ND] = {};
 #pragma unroll
         for (int e = 0; e < E; ++e) {
 #pragma unroll
-            for (int k = 0; k < S - 1; ++k) raw[e * S + k] = StateRun<DT>::get(ST[n], e * S + k + 1);
-            raw[e * S + S - 1] = StateRun<DT>::get(&X[n], e);   // the token's own bits
+            for (int k = 0; k < S - 1; ++k) Packed<DT>::put(nw, e * S + k, Packed<DT>::get(ST[n], e * S + k + 1));
+            const uint32_t tok = a.tmask ? Packed<DT>::raw_of(xt[e]) : Packed<DT>::get(X[n], e);
+            Packed<DT>::put(nw, e * S + S - 1, tok);
         }
-        if (a.tmask) {
+        store_words<ND>(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY, nw);
+    }
+}
+
+template <int DT, int W, int S, int NB, bool POOL = false>
+__device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_t blk)
+{
+    constexpr int BY = Elem<DT>::bytes;
+    constexpr int E = upd_lane_channels(BY, S);
+    constexpr int ND = E * S * BY / 4;          // words of state per lane and batch entry
+    constexpr int NX = (E * BY + 3) / 4;        // words of token / output
+    static_assert(E * S * BY % 4 == 0, "a lane's piece of the state must be whole words");
+    const uint32_t tid = blk * 256u + threadIdx.x;
+    // the test reads a field of each 64-byte line of the arguments this kernel uses (the divisor is never 0,
+    // the flag never negative), so that all are requested together instead of one after the other
+    if ((tid >= a.nthreads) | (a.div_nvec.d == 0) | (a.w_vec < 0)) return;   // '|': one test, no short circuit
+    const uint32_t bg = fdiv(tid, a.div_nvec);
+    const uint32_t cv = tid - bg * a.nvec;
+    const uint32_t c0 = cv * E;
+
+    uint32_t X[NB][NX];
+    uint32_t ST[NB][ND];
+    uint32_t srow[NB];   // conv_state row of each batch entry
 #pragma unroll
-            for (int e = 0; e < E; ++e) raw[e * S + S - 1] = StateRun<DT>::raw_of(xt[e]);
-        }
-        uint4 *dp = (uint4 *)(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY);
-#pragma unroll
-        for (int k = 0; k < S; ++k) {
-            uint4 q;
-            if constexpr (DT == CANON_DTYPE_F32) {
-                q.x = raw[4 * k]; q.y = raw[4 * k + 1]; q.z = raw[4 * k + 2]; q.w = raw[4 * k + 3];
-            } else {
-                q.x = raw[8 * k] | (raw[8 * k + 1] << 16);
-                q.y = raw[8 * k + 2] | (raw[8 * k + 3] << 16);
-                q.z = raw[8 * k + 4] | (raw[8 * k + 5] << 16);
-                q.w = raw[8 * k + 6] | (raw[8 * k + 7] << 16);
-            }
-            dp[k] = q;
+    for (int n = 0; n < NB; ++n) {
+        const uint32_t b = bg * NB + n;
+        if (b < a.B) {
+            const char *xp = a.x + ((int64_t)b * a.x_sb + c0) * BY;
+            if constexpr (E * BY == 2) X[n][0] = *(const uint16_t *)xp;
+            else load_words<NX>(xp, X[n]);
+            srow[n] = POOL ? (uint32_t)a.indices[b] : b;   // POOL: rows of a state pool (conv_state_indices)
+            load_words<ND>(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
         }
     }
+    if constexpr (W == 4) {
+        if (a.tap_mode == TAPS_SAME) {
+            update_vec_body<DT, W, S, NB, TAPS_SAME>(a, bg, c0, X, ST, srow);
+            return;
+        }
+        if constexpr (DT != CANON_DTYPE_F32) {
+            if (a.tap_mode == TAPS_WIDE) {
+                update_vec_body<DT, W, S, NB, TAPS_WIDE>(a, bg, c0, X, ST, srow);
+                return;
+            }
+        }
+    }
+    update_vec_body<DT, W, S, NB, TAPS_ANY>(a, bg, c0, X, ST, srow);
 }
 
 template <int DT, int W, int S, int NB>

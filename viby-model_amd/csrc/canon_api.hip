@@ -32,6 +32,14 @@ bool valid_mask_dtype(int d) { return d >= CANON_MASK_U8 && d <= CANON_MASK_F16;
 int elem_bytes(int d) { return d == CANON_DTYPE_F32 ? 4 : 2; }
 bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+// tap layout the channel-contiguous kernels can read with straight-line loads (see TapMode)
+int tap_mode_of(bool w_vec, const void *bias, int x_dtype, int w_dtype)
+{
+    if (!w_vec || ((uintptr_t)bias & 3u) != 0) return TAPS_ANY;
+    if (w_dtype == x_dtype) return TAPS_SAME;
+    return w_dtype == CANON_DTYPE_F32 ? TAPS_WIDE : TAPS_ANY;
+}
+
 FastDiv make_fastdiv(uint32_t d)
 {
     // floor(n / d) for 0 <= n < 2^32 (Granlund-Montgomery round-up method)
@@ -116,6 +124,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.S_out = p->final_state ? p->final_len : 0;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
     a.b_vec = p->bias && aligned16(p->bias);
+    a.tap_mode = tap_mode_of(a.w_vec != 0, p->bias, p->x_dtype, p->w_dtype);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
@@ -241,11 +250,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
     a.b_vec = p->bias && aligned16(p->bias);
-    a.tap_mode = TAPS_ANY;
-    if (a.w_vec && (uintptr_t)p->bias % 4 == 0) {
-        if (p->w_dtype == p->x_dtype) a.tap_mode = TAPS_SAME;
-        else if (p->w_dtype == CANON_DTYPE_F32) a.tap_mode = TAPS_WIDE;
-    }
+    a.tap_mode = tap_mode_of(a.w_vec != 0, p->bias, p->x_dtype, p->w_dtype);
     plan->kind = UPD_GENERIC;
     plan->grid = 0;
     if (empty) return CANON_OK;

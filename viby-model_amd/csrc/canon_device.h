@@ -621,6 +621,114 @@ __device__ __forceinline__ void decode_taps(const RawTaps<NC> &r, int w_dtype, b
     else decode_taps_typed<DT, CANON_DTYPE_F16, W, NC>(r, vec, has_bias, w, bv);
 }
 
+// ---------------------------------------------------------------------------
+// Runs of 32-bit words at 4-byte aligned addresses, and elements of a storage
+// type packed in such words (raw bits)
+// ---------------------------------------------------------------------------
+typedef uint32_t words2_t __attribute__((ext_vector_type(2), aligned(4)));
+typedef uint32_t words3_t __attribute__((ext_vector_type(3), aligned(4)));
+typedef uint32_t words4_t __attribute__((ext_vector_type(4), aligned(4)));
+
+// N consecutive 32-bit words at a 4-byte aligned address
+template <int N> __device__ __forceinline__ void load_words(const char *p, uint32_t *d)
+{
+    if constexpr (N == 1) {
+        d[0] = *(const uint32_t *)p;
+    } else if constexpr (N == 2) {
+        const words2_t q = *(const words2_t *)p;
+        d[0] = q.x; d[1] = q.y;
+    } else if constexpr (N == 3) {
+        const words3_t q = *(const words3_t *)p;
+        d[0] = q.x; d[1] = q.y; d[2] = q.z;
+    } else if constexpr (N == 4) {
+        const words4_t q = *(const words4_t *)p;
+        d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+    } else {
+        load_words<4>(p, d);
+        load_words<N - 4>(p + 16, d + 4);
+    }
+}
+
+template <int N> __device__ __forceinline__ void store_words(char *p, const uint32_t *d)
+{
+    if constexpr (N == 1) {
+        *(uint32_t *)p = d[0];
+    } else if constexpr (N == 2) {
+        words2_t q; q.x = d[0]; q.y = d[1];
+        *(words2_t *)p = q;
+    } else if constexpr (N == 3) {
+        words3_t q; q.x = d[0]; q.y = d[1]; q.z = d[2];
+        *(words3_t *)p = q;
+    } else if constexpr (N == 4) {
+        words4_t q; q.x = d[0]; q.y = d[1]; q.z = d[2]; q.w = d[3];
+        *(words4_t *)p = q;
+    } else {
+        store_words<4>(p, d);
+        store_words<N - 4>(p + 16, d + 4);
+    }
+}
+
+// elements of the storage type packed in 32-bit words, handled as raw bits
+template <int DT> struct Packed {
+    static __device__ __forceinline__ uint32_t get(const uint32_t *d, int i)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return d[i];
+        else return (i & 1) ? (d[i >> 1] >> 16) : (d[i >> 1] & 0xFFFFu);
+    }
+    static __device__ __forceinline__ void put(uint32_t *d, int i, uint32_t raw)   // d starts as zeros
+    {
+        if constexpr (DT == CANON_DTYPE_F32) d[i] = raw;
+        else d[i >> 1] |= (i & 1) ? (raw << 16) : raw;
+    }
+    static __device__ __forceinline__ float as_float(uint32_t raw)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return bits_f(raw);
+        else if constexpr (DT == CANON_DTYPE_BF16) return bits_f(raw << 16);
+        else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+    }
+    static __device__ __forceinline__ uint32_t raw_of(float f)   // rounds to nearest even
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return f_bits(f);
+        else if constexpr (DT == CANON_DTYPE_BF16) return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
+        else return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    }
+};
+
+// Taps and bias of E adjacent channels from a contiguous [C, 4] weight array of
+// type WDT (16-byte aligned; bias 4-byte aligned): straight-line loads, no
+// branch on a run-time type between them, so a kernel can have them in flight
+// together with everything else it requests.
+template <int WDT, int E> struct TapWords {
+    static constexpr int NW = E * Elem<WDT>::bytes;               // 4 taps per channel
+    static constexpr int NB = (E * Elem<WDT>::bytes + 3) / 4;
+    uint32_t w[NW];
+    uint32_t b[NB];
+};
+
+template <int WDT, int E>
+__device__ __forceinline__ void fetch_taps_contiguous(const void *weight, const void *bias, uint32_t c0, TapWords<WDT, E> &r)
+{
+    constexpr int WBY = Elem<WDT>::bytes;
+    load_words<TapWords<WDT, E>::NW>((const char *)weight + (int64_t)c0 * 4 * WBY, r.w);
+    // no branch around the bias load (a merge of "loaded" and "zero" costs a wait): without a bias the same
+    // bytes are read from the weights, which are at least as long, and ignored when decoding
+    const char *bp = (const char *)(bias ? bias : weight) + (int64_t)c0 * WBY;
+    if constexpr (E * WBY == 2) r.b[0] = *(const uint16_t *)bp;
+    else load_words<TapWords<WDT, E>::NB>(bp, r.b);
+}
+
+// ... converted to float and rounded to the storage type DT of x (zero bias when there is none)
+template <int DT, int WDT, int E>
+__device__ __forceinline__ void decode_taps_contiguous(const TapWords<WDT, E> &r, bool has_bias, float (*w)[4], float *bv)
+{
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) w[e][k] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(r.w, e * 4 + k)));
+        bv[e] = has_bias ? round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(r.b, e))) : 0.0f;
+    }
+}
+
 template <typename Args>
 __device__ __forceinline__ uint32_t part_of_block(const PartTable<Args> &m, uint32_t blk)
 {

@@ -299,14 +299,15 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
     if (active) VecIO<VB>::template store<NT>(optr, VecIO<VB>::template pack<DT>(o));
 }
 
-template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
-__device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
+template <int DT, int W, int R, bool MASK, bool NT, bool SEQ, int VB, int MODE>
+__device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t blk,
+                                               typename VecIO<VB>::type (*tail)[3][64])   // LDS: raw last three rows of each wave's slab
 {
     constexpr int E = VB / Elem<DT>::bytes;
+    constexpr int WDT = MODE == TAPS_WIDE ? CANON_DTYPE_F32 : DT;   // weight type of the straight-line tap modes
     using V = VecIO<VB>;
     using vec_t = typename V::type;
     static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
-    __shared__ vec_t tail[kBlcWaves][3][64];   // raw last three rows of each wave's slab
 
     // blocks in plain memory order (an XCD-contiguous remap measured 3 % slower here)
     // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
@@ -328,12 +329,15 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
     const int64_t t_last = (int64_t)a.L - 1;
 
-    // slab rows, then (first wave only) the three rows before the block, then the taps.
+    // taps (contiguous layouts: first, they come from the cache and nothing waits for them before the rows
+    // are requested), slab rows, then (first wave only) the three rows before the block.
     // Rows past the end of the sequence are clamped to the last row (loaded, never used).
     vec_t X[R], H[3];
     float m[R], mh[3];
     int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
+    TapWords<WDT, E> tw;
+    if constexpr (MODE != TAPS_ANY) fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         X[r] = V::zero();
@@ -360,7 +364,8 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
             }
         }
         // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
-        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
+        if constexpr (MODE == TAPS_ANY)
+            fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
         if constexpr (SEQ) load_seq_rows<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, sq);
         if constexpr (MASK) {
             // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
@@ -404,7 +409,8 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
         }
     }
     float w[E][W], bias[E];
-    decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+    if constexpr (MODE == TAPS_ANY) decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+    else decode_taps_contiguous<DT, WDT, E>(tw, a.bias != nullptr, w, bias);
 
     if constexpr (SEQ) {
 #pragma unroll
@@ -449,6 +455,27 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
                 store1<DT>(a.fin, b * a.f_sb + (int64_t)(c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
         }
     }
+}
+
+// The block's code once per tap layout (wave-uniform choice): the contiguous layouts are straight-line
+// loads, the general one branches on the run-time weight type between its loads and waits there.
+template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
+__device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
+{
+    __shared__ typename VecIO<VB>::type tail[kBlcWaves][3][64];
+    if constexpr (W == 4) {
+        if (a.tap_mode == TAPS_SAME) {
+            blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_SAME>(a, blk, tail);
+            return;
+        }
+        if constexpr (DT != CANON_DTYPE_F32) {
+            if (a.tap_mode == TAPS_WIDE) {
+                blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_WIDE>(a, blk, tail);
+                return;
+            }
+        }
+    }
+    blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_ANY>(a, blk, tail);
 }
 
 template <int DT, int W, int R, bool MASK, bool NT>

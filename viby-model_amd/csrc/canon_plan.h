@@ -24,6 +24,15 @@ struct FastDiv {
     uint32_t d, m, s1, s2;
 };
 
+// How a lane of the channel-contiguous kernels (prefill, decode update) gets its taps and bias.  The two common layouts are straight-line
+// code (every load of the kernel is in flight before the first wait; the general path branches on the
+// run-time weight type between its loads, which costs a wait per branch); which one runs is wave-uniform.
+enum TapMode {
+    TAPS_SAME,   // contiguous, 16-byte aligned [C, 4] weights of x's type (bias too, 4-byte aligned)
+    TAPS_WIDE,   // the same with fp32 weights and bias and 16-bit x
+    TAPS_ANY     // any strides, width and type
+};
+
 // ---------------------------------------------------------------------------
 // kernel argument blocks (device copies of the validated ABI structs)
 // ---------------------------------------------------------------------------
@@ -44,7 +53,7 @@ struct FwdArgs {
     int64_t i_sb, i_sc, i_ss;
     int64_t f_sb, f_sc, f_ss;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt, tap_mode;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
     uint32_t nseg;      // bcl: segments per row       generic: time chunks per row
@@ -55,15 +64,6 @@ struct FwdArgs {
     // blc: tiles
     uint32_t nct, ntt;  // channel tiles per row, time tiles per sequence
     FastDiv div_nct, div_ntt;
-};
-
-// How a lane of the vectorised update gets its taps and bias.  The two common layouts are straight-line
-// code (every load of the kernel is in flight before the first wait; the general path branches on the
-// run-time weight type between its loads, which costs a wait per branch); which one runs is wave-uniform.
-enum TapMode {
-    TAPS_SAME,   // contiguous, 16-byte aligned [C, 4] weights of x's type (bias too, 4-byte aligned)
-    TAPS_WIDE,   // the same with fp32 weights and bias and 16-bit x
-    TAPS_ANY     // any strides, width and type
 };
 
 struct UpdArgs {

@@ -17,75 +17,6 @@ namespace canon {
 // pass.  Each lane walks NB batch rows so the taps are fetched once per NB
 // tokens.
 // ---------------------------------------------------------------------------
-typedef uint32_t words2_t __attribute__((ext_vector_type(2), aligned(4)));
-typedef uint32_t words3_t __attribute__((ext_vector_type(3), aligned(4)));
-typedef uint32_t words4_t __attribute__((ext_vector_type(4), aligned(4)));
-
-// N consecutive 32-bit words at a 4-byte aligned address
-template <int N> __device__ __forceinline__ void load_words(const char *p, uint32_t *d)
-{
-    if constexpr (N == 1) {
-        d[0] = *(const uint32_t *)p;
-    } else if constexpr (N == 2) {
-        const words2_t q = *(const words2_t *)p;
-        d[0] = q.x; d[1] = q.y;
-    } else if constexpr (N == 3) {
-        const words3_t q = *(const words3_t *)p;
-        d[0] = q.x; d[1] = q.y; d[2] = q.z;
-    } else if constexpr (N == 4) {
-        const words4_t q = *(const words4_t *)p;
-        d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
-    } else {
-        load_words<4>(p, d);
-        load_words<N - 4>(p + 16, d + 4);
-    }
-}
-
-template <int N> __device__ __forceinline__ void store_words(char *p, const uint32_t *d)
-{
-    if constexpr (N == 1) {
-        *(uint32_t *)p = d[0];
-    } else if constexpr (N == 2) {
-        words2_t q; q.x = d[0]; q.y = d[1];
-        *(words2_t *)p = q;
-    } else if constexpr (N == 3) {
-        words3_t q; q.x = d[0]; q.y = d[1]; q.z = d[2];
-        *(words3_t *)p = q;
-    } else if constexpr (N == 4) {
-        words4_t q; q.x = d[0]; q.y = d[1]; q.z = d[2]; q.w = d[3];
-        *(words4_t *)p = q;
-    } else {
-        store_words<4>(p, d);
-        store_words<N - 4>(p + 16, d + 4);
-    }
-}
-
-// elements of the storage type packed in 32-bit words, handled as raw bits
-template <int DT> struct Packed {
-    static __device__ __forceinline__ uint32_t get(const uint32_t *d, int i)
-    {
-        if constexpr (DT == CANON_DTYPE_F32) return d[i];
-        else return (i & 1) ? (d[i >> 1] >> 16) : (d[i >> 1] & 0xFFFFu);
-    }
-    static __device__ __forceinline__ void put(uint32_t *d, int i, uint32_t raw)   // d starts as zeros
-    {
-        if constexpr (DT == CANON_DTYPE_F32) d[i] = raw;
-        else d[i >> 1] |= (i & 1) ? (raw << 16) : raw;
-    }
-    static __device__ __forceinline__ float as_float(uint32_t raw)
-    {
-        if constexpr (DT == CANON_DTYPE_F32) return bits_f(raw);
-        else if constexpr (DT == CANON_DTYPE_BF16) return bits_f(raw << 16);
-        else return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-    }
-    static __device__ __forceinline__ uint32_t raw_of(float f)   // rounds to nearest even
-    {
-        if constexpr (DT == CANON_DTYPE_F32) return f_bits(f);
-        else if constexpr (DT == CANON_DTYPE_BF16) return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
-        else return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
-    }
-};
-
 template <int DT, int W, int S, int NB, int MODE>
 __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t bg, const uint32_t c0,
                                                 const uint32_t (*X)[(upd_lane_channels(Elem<DT>::bytes, S) * Elem<DT>::bytes + 3) / 4],
@@ -97,22 +28,14 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
     constexpr int ND = E * S * BY / 4;
     constexpr int NX = (E * BY + 3) / 4;
     constexpr int WDT = MODE == TAPS_WIDE ? CANON_DTYPE_F32 : DT;      // weight type of the straight-line modes
-    constexpr int WBY = Elem<WDT>::bytes;
-    constexpr int NT = MODE == TAPS_ANY ? 1 : E * WBY;                  // words of taps: 4 * WBY bytes per channel
-    constexpr int NBW = MODE == TAPS_ANY ? 1 : (E * WBY + 3) / 4;       // words of bias
 
-    uint32_t tw[NT], tb[NBW] = {};
+    TapWords<WDT, E> tw;
     RawTaps<E> raw;
     if constexpr (MODE == TAPS_ANY) {
         fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
     } else {
         static_assert(MODE == TAPS_ANY || W == 4, "the contiguous tap layouts are [C, 4]");
-        load_words<NT>((const char *)a.weight + (int64_t)c0 * 4 * WBY, tw);
-        if (a.bias) {
-            const char *bp = (const char *)a.bias + (int64_t)c0 * WBY;
-            if constexpr (E * WBY == 2) tb[0] = *(const uint16_t *)bp;
-            else load_words<NBW>(bp, tb);
-        }
+        fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
     }
     float tm[NB];
 #pragma unroll
@@ -131,17 +54,8 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
         for (int n = 0; n < NB; ++n) tm[n] = tmv[n][0];
     }
     float w[E][W], bias[E];
-    if constexpr (MODE == TAPS_ANY) {
-        decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
-    } else {
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-#pragma unroll
-            for (int k = 0; k < W; ++k)
-                w[e][k] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(tw, e * 4 + k)));
-            bias[e] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(tb, e)));   // zero bits without a bias
-        }
-    }
+    if constexpr (MODE == TAPS_ANY) decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+    else decode_taps_contiguous<DT, WDT, E>(tw, a.bias != nullptr, w, bias);
 
 #pragma unroll
     for (int n = 0; n < NB; ++n) {

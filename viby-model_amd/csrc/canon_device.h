@@ -160,12 +160,25 @@ template <bool NT> __device__ __forceinline__ void store_vec(void *p, const uint
     else *(u32x4_t *)p = q;
 }
 
-// (float) of a 64-bit integer given as two words; masks are 0/1 in practice, so
-// the value almost always fits 32 bits and one conversion instruction does it
-__device__ __forceinline__ float i64_words_to_float(uint32_t lo, uint32_t hi)
+// (float) of N 64-bit integers given as word pairs.  When every value of the whole wave fits 32 bits (the
+// usual 0/1 mask) it is one conversion instruction each; otherwise the full conversions run one after the
+// other.  Written as per-value selects, the N full conversions are scheduled side by side and their
+// temporaries (a dozen registers each) set the register count of every kernel that can meet an int64 mask.
+template <int N> __device__ __forceinline__ void i64_words_to_float_n(const uint32_t *lo, const uint32_t *hi, float *m)
 {
-    if ((int32_t)hi == ((int32_t)lo >> 31)) return (float)(int32_t)lo;
-    return (float)(int64_t)(((uint64_t)hi << 32) | lo);
+    bool wide = false;
+#pragma unroll
+    for (int j = 0; j < N; ++j) wide |= (int32_t)hi[j] != ((int32_t)lo[j] >> 31);
+    if (__builtin_amdgcn_ballot_w64(wide) == 0) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) m[j] = (float)(int32_t)lo[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            m[j] = (float)(int64_t)(((uint64_t)hi[j] << 32) | lo[j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
 }
 
 // N mask entries of consecutive time steps t_first .. t_first+N-1 (clamped to
@@ -194,11 +207,14 @@ __device__ __forceinline__ void load_mask_entries(const void *p, int64_t first, 
         for (int j = 0; j < N; ++j) m[j] = (float)((const int32_t *)p)[RUN ? first + j : idx[j]];
         break;
     case CANON_MASK_I64: {
-        uint2 q[N];
+        uint32_t lo[N], hi[N];
 #pragma unroll
-        for (int j = 0; j < N; ++j) q[j] = ((const uint2 *)p)[RUN ? first + j : idx[j]];
-#pragma unroll
-        for (int j = 0; j < N; ++j) m[j] = i64_words_to_float(q[j].x, q[j].y);
+        for (int j = 0; j < N; ++j) {
+            const uint2 q = ((const uint2 *)p)[RUN ? first + j : idx[j]];
+            lo[j] = q.x;
+            hi[j] = q.y;
+        }
+        i64_words_to_float_n<N>(lo, hi, m);
         break;
     }
     case CANON_MASK_F32:
@@ -328,33 +344,37 @@ __device__ __forceinline__ void load_mask_vec(const void *p, const int64_t *base
             return;
         }
         case CANON_MASK_I32: {
-            uint4 q[U][N / 4];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
+            for (int u = 0; u < U; ++u) {   // one vector at a time, as for int64 below
+                uint4 q[N / 4 > 0 ? N / 4 : 1];   // (N < 4 never takes the vector path)
 #pragma unroll
-                for (int i = 0; i < N / 4; ++i) q[u][i] = ((const uint4 *)((const int32_t *)p + base[u]))[i];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
+                for (int i = 0; i < N / 4; ++i) q[i] = ((const uint4 *)((const int32_t *)p + base[u]))[i];
 #pragma unroll
                 for (int i = 0; i < N / 4; ++i) {
-                    m[u][4 * i] = (float)(int32_t)q[u][i].x; m[u][4 * i + 1] = (float)(int32_t)q[u][i].y;
-                    m[u][4 * i + 2] = (float)(int32_t)q[u][i].z; m[u][4 * i + 3] = (float)(int32_t)q[u][i].w;
+                    m[u][4 * i] = (float)(int32_t)q[i].x; m[u][4 * i + 1] = (float)(int32_t)q[i].y;
+                    m[u][4 * i + 2] = (float)(int32_t)q[i].z; m[u][4 * i + 3] = (float)(int32_t)q[i].w;
                 }
+                if (u + 1 < U) __builtin_amdgcn_sched_barrier(0);
+            }
             return;
         }
         case CANON_MASK_I64: {
-            uint4 q[U][N / 2];
+            // one vector's entries (N / 2 16-byte loads) at a time: holding the raw words of all U vectors would
+            // set the register count of the whole kernel (all mask types share it) and cost a wave per SIMD
 #pragma unroll
-            for (int u = 0; u < U; ++u)
+            for (int u = 0; u < U; ++u) {
+                uint4 q[N / 2 > 0 ? N / 2 : 1];
 #pragma unroll
-                for (int i = 0; i < N / 2; ++i) q[u][i] = ((const uint4 *)((const int64_t *)p + base[u]))[i];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
+                for (int i = 0; i < N / 2; ++i) q[i] = ((const uint4 *)((const int64_t *)p + base[u]))[i];
+                uint32_t lo[N], hi[N];
 #pragma unroll
                 for (int i = 0; i < N / 2; ++i) {
-                    m[u][2 * i] = i64_words_to_float(q[u][i].x, q[u][i].y);
-                    m[u][2 * i + 1] = i64_words_to_float(q[u][i].z, q[u][i].w);
+                    lo[2 * i] = q[i].x; hi[2 * i] = q[i].y;
+                    lo[2 * i + 1] = q[i].z; hi[2 * i + 1] = q[i].w;
                 }
+                i64_words_to_float_n<N>(lo, hi, m[u]);
+                if (u + 1 < U) __builtin_amdgcn_sched_barrier(0);   // keep the next vector's loads behind this conversion
+            }
             return;
         }
         case CANON_MASK_F32: {
@@ -410,9 +430,16 @@ __device__ __forceinline__ void load_mask_vec(const void *p, const int64_t *base
         break;
     case CANON_MASK_I64:
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int u = 0; u < U; ++u) {
+            uint32_t lo[N], hi[N];
 #pragma unroll
-            for (int j = 0; j < N; ++j) m[u][j] = (float)((const int64_t *)p)[base[u] + j * stride];
+            for (int j = 0; j < N; ++j) {
+                const uint2 q = ((const uint2 *)p)[base[u] + j * stride];
+                lo[j] = q.x;
+                hi[j] = q.y;
+            }
+            i64_words_to_float_n<N>(lo, hi, m[u]);
+        }
         break;
     case CANON_MASK_F32:
 #pragma unroll

@@ -144,9 +144,12 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     RawTaps<1> raw;
     fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
 
-    // all mask entries of the segment, requested before anything is consumed
-    float M[MASK ? U : 1][E];
+    // all mask entries of the segment, requested before anything is consumed; the masked inputs are formed
+    // at once and kept in storage format (XM): eight mask floats per vector held until the main loop would
+    // cost the kernel a wave per SIMD
+    uint4 XM[MASK ? U : 1];
     if constexpr (MASK) {
+        float M[U][E];
         int64_t mbase[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -159,6 +162,14 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
             }
         }
         load_mask_vec<E, U>(a.mask, mbase, a.m_sl, a.mask_dtype, !EDGE && a.m_vec != 0, M);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float xr[E], xm[E];
+            unpack_vec<DT>(X[u], xr);
+#pragma unroll
+            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
+            XM[u] = pack_vec<DT>(xm);   // exact: the products are already rounded to the storage type
+        }
     }
 
     float w[1][W], bvv[1];
@@ -196,10 +207,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
         float xr[E], xm_store[MASK ? E : 1];
         float *xm = MASK ? xm_store : xr;
         unpack_vec<DT>(X[u], xr);
-        if constexpr (MASK) {
-#pragma unroll
-            for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[u][j]);
-        }
+        if constexpr (MASK) unpack_vec<DT>(XM[u], xm);
         // seq[0..2] = the three masked inputs before this vector
         float seq[E + 3];
         seq[0] = wave_shift_up(xm[E - 3], carry[0]);

@@ -570,9 +570,10 @@ def test_randomised_shapes_layouts_and_options(cc):
         use_mask = ri(0, 1)
         use_bias = ri(0, 1)
         mode = pick(["plain", "plain", "state", "seq"])
+        wdt = pick([dtype, dtype, torch.float32])      # x's own type, or fp32 master weights
         x = torch.randn(B, C, L, generator=g).to(dtype)
-        w = (torch.randn(C, W, generator=g) * 0.4).to(dtype)
-        b = (torch.randn(C, generator=g) * 0.2).to(dtype) if use_bias else None
+        w = (torch.randn(C, W, generator=g) * 0.4).to(wdt)
+        b = (torch.randn(C, generator=g) * 0.2).to(wdt) if use_bias else None
         mask = right_padded_mask([ri(1, L) for _ in range(B)], L, dtype=pick([torch.int64, torch.bool, torch.float32])) \
             if use_mask else None
         if layout == "bcl":
@@ -588,7 +589,7 @@ def test_randomised_shapes_layouts_and_options(cc):
             big[:, 1:L + 1, 8:] = x.to(DEV).transpose(1, 2)
             xg = big[:, 1:L + 1, 8:].transpose(1, 2)
         kw = dict(activation=act, residual=res, attention_mask=None if mask is None else mask.to(DEV))
-        what = f"case {case}: {dtype} {layout} {B}x{C}x{L} W{W} {act} {res} mask{use_mask} bias{use_bias} {mode}"
+        what = f"case {case}: {dtype} w{wdt} {layout} {B}x{C}x{L} W{W} {act} {res} mask{use_mask} bias{use_bias} {mode}"
         xm = x if mask is None else (x.float() * mask[:, None, :].float()).to(dtype)
         if mode == "seq":
             seq = packed_seq_idx(B, L, g)
@@ -635,8 +636,9 @@ def test_randomised_decode_steps(cc):
         act = pick([None, "silu"])
         mode = pick(["plain", "plain", "ring", "pool", "strided"])
         res = pick([False, True])
-        w = (torch.randn(C, W, generator=g) * 0.4).to(dtype)
-        b = (torch.randn(C, generator=g) * 0.2).to(dtype) if ri(0, 1) else None
+        wdt = pick([dtype, dtype, torch.float32])      # x's own type, or fp32 master weights
+        w = (torch.randn(C, W, generator=g) * 0.4).to(wdt)
+        b = (torch.randn(C, generator=g) * 0.2).to(wdt) if ri(0, 1) else None
         rows = B + 2 if mode == "pool" else B
         state_ref = torch.randn(rows, C, S, generator=g).to(dtype)
         if mode == "strided":
@@ -654,6 +656,6 @@ def test_randomised_decode_steps(cc):
             got = cc.causal_conv1d_update(x.to(DEV), state_gpu, w.to(DEV), None if b is None else b.to(DEV), activation=act,
                                           residual=res, cache_seqlens=None if sl is None else sl.to(DEV),
                                           conv_state_indices=None if idx is None else idx.to(DEV))
-            what = f"case {case}: {dtype} {B}x{C} W{W} S{S} {act} res{res} {mode} step{step}"
+            what = f"case {case}: {dtype} w{wdt} {B}x{C} W{W} S{S} {act} res{res} {mode} step{step}"
             assert_parity(got, want, exact=act is None, what=what, res=x if res else None)
             assert torch.equal(bits(state_gpu), bits(state_ref)), what

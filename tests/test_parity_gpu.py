@@ -653,7 +653,13 @@ def test_randomised_decode_steps(cc):
             sl = torch.randint(0, 50, (B,), generator=g).to(torch.int32) if mode == "ring" else None
             want = co.conv1d_update_ext(x, state_ref, w, b, activation=act, residual=res, cache_seqlens=sl,
                                         conv_state_indices=idx)
-            got = cc.causal_conv1d_update(x.to(DEV), state_gpu, w.to(DEV), None if b is None else b.to(DEV), activation=act,
+            xg = x.to(DEV)
+            if (case + step) % 3 == 0:      # the token as a slice of a wider tensor (odd offsets fail the alignment test)
+                off = (case + step) % 4
+                wide = torch.zeros(B, C + 5, dtype=dtype, device=DEV)
+                wide[:, off:off + C] = xg
+                xg = wide[:, off:off + C]
+            got = cc.causal_conv1d_update(xg, state_gpu, w.to(DEV), None if b is None else b.to(DEV), activation=act,
                                           residual=res, cache_seqlens=None if sl is None else sl.to(DEV),
                                           conv_state_indices=None if idx is None else idx.to(DEV))
             what = f"case {case}: {dtype} w{wdt} {B}x{C} W{W} S{S} {act} res{res} {mode} step{step}"

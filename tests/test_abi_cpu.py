@@ -162,6 +162,20 @@ def test_update_plan_and_validation():
         assert uplan(update_params(S=S)) == "update_vec"
     assert uplan(update_params(S=5)) == "update_generic"
     assert uplan(update_params(C=3457)) == "update_generic"
+    # a lane of the vector kernel owns one 12..16-byte run of the state: two channels with 16-bit elements
+    # and 3 or 4 slots (so the token is read as 4-byte words), one channel otherwise
+    assert uplan(update_params(C=3457, S=8)) == "update_vec"
+    assert uplan(update_params(C=3457, dtype=0)) == "update_vec"
+    assert uplan(update_params(C=3458)) == "update_vec"
+    assert uplan(update_params(x=FAKE_X + 2)) == "update_generic"                  # token off the 4-byte grid
+    assert uplan(update_params(x=FAKE_X + 2, S=8)) == "update_vec"                 # ... one 16-bit channel per lane: fine
+    assert uplan(update_params(x=FAKE_X + 4)) == "update_vec"
+    assert uplan(update_params(x_stride_b=3457)) == "update_generic"               # odd row pitch
+    assert uplan(update_params(out=FAKE_OUT + 2)) == "update_generic"
+    assert uplan(update_params(conv_state=FAKE_STATE + 2)) == "update_generic"
+    assert uplan(update_params(conv_state=FAKE_STATE + 4)) == "update_vec"
+    assert uplan(update_params(state_stride_b=3456 * 3 + 1)) == "update_generic"   # rows of a state pool off the grid
+    assert uplan(update_params(state_stride_b=3456 * 3 + 2)) == "update_vec"
     assert uplan(update_params(state_stride_s=2, state_stride_c=6, state_stride_b=3456 * 6)) == "update_generic"
     assert uplan(update_params(round_mode=1)) == "update_generic"
     assert uplan(update_params(conv_state_indices=FAKE_STATE + 64)) == "update_vec"       # state pool: row indirection

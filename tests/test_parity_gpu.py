@@ -308,6 +308,34 @@ def test_update_residual_exact(cc):
         assert torch.equal(bits(st_gpu), bits(st_ref))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_update_vector_kernel_on_buffers_aligned_to_4_bytes_only(cc, dtype):
+    """State, token and weights carved out of larger buffers at 4-byte offsets: the vector kernel asks for no more."""
+    g = torch.Generator().manual_seed(36)
+    B, C = 5, 264
+    es = torch.empty((), dtype=dtype).element_size()
+    off = 4 // es                      # elements in 4 bytes
+    for S in (3, 4, 8):
+        st = torch.randn(B, C, S, generator=g).to(dtype)
+        x = torch.randn(B, C, generator=g).to(dtype)
+        w = (torch.randn(C, 4, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        flat = torch.zeros(B * C * S + 2 * off, dtype=dtype, device=DEV)
+        st_gpu = flat[off:off + B * C * S].view(B, C, S)
+        st_gpu.copy_(st.to(DEV))
+        xflat = torch.zeros(B * C + 2 * off, dtype=dtype, device=DEV)
+        x_gpu = xflat[off:off + B * C].view(B, C)
+        x_gpu.copy_(x.to(DEV))
+        assert st_gpu.data_ptr() % 16 == 4 and x_gpu.data_ptr() % 16 == 4
+        assert cc.kernel_plan_update(x_gpu, st_gpu, w.to(DEV), b.to(DEV)) == "update_vec"
+        st_ref = st.clone()
+        want = co.conv1d_update(x, st_ref, w, b, activation="silu", residual=True)
+        got = cc.causal_conv1d_update(x_gpu, st_gpu, w.to(DEV), b.to(DEV), activation="silu", residual=True)
+        assert_parity(got, want, exact=False, what=f"4-byte aligned S{S}", res=x)
+        assert torch.equal(bits(st_gpu), bits(st_ref))
+        assert float(flat[:off].abs().sum()) == 0 and float(flat[off + B * C * S:].abs().sum()) == 0   # neighbours untouched
+
+
 def test_noncontiguous_state_takes_strided_kernel_and_stays_in_place(cc):
     g = torch.Generator().manual_seed(35)
     B, C, S = 3, 64, 4

@@ -306,7 +306,7 @@ __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W],
     for (int r = R - 1; r >= 0; --r) {
         float g[E], dz[E], o[E];
         unpack_half<DT>(G[r], g);
-        if (r >= 3) {
+        if (r >= 3 || !ACT) {
             bwd_dz<W, E, ACT>(w, bias, xw[0], xw[1], xw[2], xw[3], g, dz);
             if constexpr (!FULL) {
 #pragma unroll
@@ -364,8 +364,13 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     constexpr int BY = Elem<DT>::bytes;
     constexpr int E = 8 / BY;
     constexpr int R = kBwdSlab, NW = kBwdWaves;
-    __shared__ uint2 tailx[NW][3][64];            // last three xm rows of each wave's slab (storage bits)
-    __shared__ float headdz[NW][3][E][64];        // dz of the first three steps of each wave's slab
+    // With an activation: tailx / headdz, two barriers per tile (dz of a slab's head needs the previous
+    // wave's tail first).  Without one dz IS dout, so the head is handed over as raw rows (headg) together
+    // with the tail, one barrier per tile, both double-buffered (a fast wave publishes the next tile while
+    // a slow one still reads this one).
+    __shared__ uint2 tailx[ACT ? 1 : 2][NW][3][64];            // last three xm rows of each wave's slab (storage bits)
+    __shared__ float headdz[ACT ? NW : 1][3][ACT ? E : 1][64];  // dz of the first three steps of each wave's slab
+    __shared__ uint2 headg[2][ACT ? 1 : NW][3][64];            // ACT == false: the first three dout rows of each slab
     __shared__ float red[NW - 1][5 * E][64];      // dweight / dbias sums of waves 1..3
     // mask entries of steps t_chunk-3 .. t_chunk+chunk+2 as floats.  Staged once per block: inside the
     // time loop (after the first store to dx) the compiler can no longer use scalar loads for them, and
@@ -407,7 +412,26 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     // are the head of the tile done just before (still in headdz[0]).  For the chunk's last tile
     // the last wave computes them here, from six rows of x and three of dout, and leaves them
     // in that slot itself.
-    {
+    float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+#pragma unroll
+        for (int e = 0; e < E; ++e) dzf[j][e] = 0.0f;
+    if constexpr (!ACT) {
+        // no activation: the three dz after the chunk are three rows of dout, kept by the last wave
+        const int64_t te = t_chunk + (int64_t)a.chunk;
+        uint2 GE[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) GE[j] = make_uint2(0, 0);
+        if (wv == NW - 1) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                if (te + j <= Lm1) GE[j] = *(const uint2 *)(gb + (te + j) * gs);
+        }
+        decode_taps<DT, W, E>(rawt, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) unpack_half<DT>(GE[j], dzf[j]);
+    } else {
         const int64_t te = t_chunk + (int64_t)a.chunk;   // first step after the chunk (at least 32)
         uint2 XE[6], GE[3];
         float me[6];
@@ -464,7 +488,8 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         const int64_t left = (int64_t)a.L - t0;
         const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
 
-        // ---- all loads of the tile (issuing them one tile ahead was measured: no gain, 14 more registers)
+        // ---- all loads of the tile.  Requesting the next tile's rows while this one is worked on was measured
+        // twice (before, and after, this tile's rows are waited for): 3-4 % slower, 40 more registers.
         uint2 X[R], G[R], H[3];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -491,12 +516,19 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         }
 
         // dz of the three steps after the slab; the last wave's are the previous iteration's head of wave 0
-        float dzf[3][E];   // dzf[j] = dz[t + 1 + j] for the step t being processed
-        if (wv == NW - 1) {
+        const int pb = it & 1;   // ACT == false: LDS buffer of this tile
+        if constexpr (ACT) {
+            if (wv == NW - 1) {
 #pragma unroll
-            for (int j = 0; j < 3; ++j)
+                for (int j = 0; j < 3; ++j)
 #pragma unroll
-                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[0][j][e][lane];
+                    for (int e = 0; e < E; ++e) dzf[j][e] = headdz[0][j][e][lane];
+            }
+        } else {
+            if (wv == NW - 1 && it != ntiles - 1) {   // (the chunk's last tile: the rows loaded before the loop)
+#pragma unroll
+                for (int j = 0; j < 3; ++j) unpack_half<DT>(headg[pb ^ 1][0][j][lane], dzf[j]);
+            }
         }
 
         // ---- rows become xm (masked, zero where they do not exist), once ----------------
@@ -510,40 +542,63 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
                 for (int j = 0; j < 3; ++j) H[j] = bwd_mask_row<DT, MASK>(H[j], mm[j], true);   // zero already when t < 0
             }
         }
-#pragma unroll
-        for (int j = 0; j < 3; ++j) tailx[wv][j][lane] = X[R - 3 + j];
-        __syncthreads();
-        if (wv > 0) {
-#pragma unroll
-            for (int j = 0; j < 3; ++j) H[j] = tailx[wv - 1][j][lane];
-        }
-
-        // ---- dz of the slab's first three steps, handed to the previous wave ---------
-        float dzh[3][E];
-        {
-            float xq[6][E];   // xm of rows -3 .. 2
-#pragma unroll
-            for (int k = 0; k < 3; ++k) unpack_half<DT>(H[k], xq[k]);
-#pragma unroll
-            for (int k = 0; k < 3; ++k) unpack_half<DT>(X[k], xq[3 + k]);
+        if constexpr (!ACT) {
+            // tail of x and head of dout (zero past the end of the sequence) in one exchange
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
-                float g[E];
-                unpack_half<DT>(G[j], g);
-                bwd_dz<W, E, ACT>(w, bias, xq[j], xq[j + 1], xq[j + 2], xq[j + 3], g, dzh[j]);
+                tailx[pb][wv][j][lane] = X[R - 3 + j];
+                headg[pb][wv][j][lane] = j < rows ? G[j] : make_uint2(0, 0);
+            }
+            __syncthreads();
+            if (wv > 0) {
 #pragma unroll
-                for (int e = 0; e < E; ++e) {
-                    dzh[j][e] = j < rows ? dzh[j][e] : 0.0f;
-                    headdz[wv][j][e][lane] = dzh[j][e];
-                }
+                for (int j = 0; j < 3; ++j) H[j] = tailx[pb][wv - 1][j][lane];
+            }
+            if (wv < NW - 1) {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) unpack_half<DT>(headg[pb][wv + 1][j][lane], dzf[j]);
             }
         }
-        __syncthreads();
-        if (wv < NW - 1) {
+        float dzh[3][E];
 #pragma unroll
-            for (int j = 0; j < 3; ++j)
+        for (int j = 0; j < 3; ++j)
 #pragma unroll
-                for (int e = 0; e < E; ++e) dzf[j][e] = headdz[wv + 1][j][e][lane];
+            for (int e = 0; e < E; ++e) dzh[j][e] = 0.0f;   // (unused without an activation)
+        if constexpr (ACT) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) tailx[0][wv][j][lane] = X[R - 3 + j];
+            __syncthreads();
+            if (wv > 0) {
+#pragma unroll
+                for (int j = 0; j < 3; ++j) H[j] = tailx[0][wv - 1][j][lane];
+            }
+
+            // ---- dz of the slab's first three steps, handed to the previous wave ---------
+            {
+                float xq[6][E];   // xm of rows -3 .. 2
+#pragma unroll
+                for (int k = 0; k < 3; ++k) unpack_half<DT>(H[k], xq[k]);
+#pragma unroll
+                for (int k = 0; k < 3; ++k) unpack_half<DT>(X[k], xq[3 + k]);
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    float g[E];
+                    unpack_half<DT>(G[j], g);
+                    bwd_dz<W, E, ACT>(w, bias, xq[j], xq[j + 1], xq[j + 2], xq[j + 3], g, dzh[j]);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        dzh[j][e] = j < rows ? dzh[j][e] : 0.0f;
+                        headdz[wv][j][e][lane] = dzh[j][e];
+                    }
+                }
+            }
+            __syncthreads();
+            if (wv < NW - 1) {
+#pragma unroll
+                for (int j = 0; j < 3; ++j)
+#pragma unroll
+                    for (int e = 0; e < E; ++e) dzf[j][e] = headdz[wv + 1][j][e][lane];
+            }
         }
 
         // ---- sweep the slab from its last step to its first --------------------------

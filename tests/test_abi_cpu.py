@@ -383,3 +383,29 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0
     assert "single-GPU" in (r.stderr + r.stdout)
+
+
+def test_torch_operators_for_traced_graphs_have_shape_only_twins():
+    """torch.compile traces the launches as operators of the canon_conv1d namespace; their shape-only
+    implementations (what tracing runs) are checked here on meta tensors, no GPU involved."""
+    import causal_conv1d  # noqa: F401  (registers the operators)
+    ops = torch.ops.canon_conv1d
+    x = torch.empty(2, 40, 16, device="meta", dtype=torch.bfloat16).transpose(1, 2)      # channel-contiguous view
+    w = torch.empty(16, 4, device="meta", dtype=torch.float32)
+    b = torch.empty(16, device="meta", dtype=torch.float32)
+    y, fin = ops.fwd(x, w, b, None, None, None, 8, 1, 1, 0)
+    assert y.shape == x.shape and y.stride() == x.stride() and y.dtype == x.dtype
+    assert tuple(fin.shape) == (2, 16, 8) and fin.dtype == x.dtype
+    assert tuple(ops.fwd(x, w, None, None, None, None, 0, 0, 0, 0)[1].shape) == (2, 16, 0)
+    dx, dw, db = ops.bwd(x, x, w, b, None, 0, 1)
+    assert dx.stride() == x.stride() and tuple(dw.shape) == (16, 4) and dw.dtype == w.dtype and tuple(db.shape) == (16,)
+    assert tuple(ops.bwd(x, x, w, None, None, 0, 1)[2].shape) == (0,)
+    st = torch.empty(2, 16, 4, device="meta", dtype=torch.bfloat16)
+    assert tuple(ops.update(x[:, :, 0], st, w, None, None, None, None, 0, 0, 0).shape) == (2, 16)
+    outs = ops.fwd_parts([x[:, :12], x[:, 12:]], w, None, None, None, 3, 0, 0, 0)
+    assert [tuple(t.shape) for t in outs] == [(2, 12, 40), (2, 4, 40), (2, 16, 3)]
+    outs = ops.update_parts([x[:, :12, 0], x[:, 12:, 0]], st, w, None, None, 0, 0, 0)
+    assert [tuple(t.shape) for t in outs] == [(2, 12), (2, 4)]
+    # the state arguments of the decode operators are declared as written to
+    assert "Tensor(a1!) conv_state" in str(ops.update.default._schema)
+    assert "Tensor(a1!) conv_state" in str(ops.update_parts.default._schema)

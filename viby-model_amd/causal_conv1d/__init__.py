@@ -22,7 +22,7 @@ or a rejected call raises.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Tuple, Union
+from typing import List, Optional, Tuple, Union
 
 import torch
 
@@ -135,6 +135,8 @@ def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tenso
     if (mask.dtype.is_floating_point or mask.element_size() <= x.element_size()
             or numel < _NARROW_MIN_ELEMENTS):
         return mask
+    if torch.compiler.is_compiling():
+        return mask.to(x.dtype)      # one node of the traced graph; identical conversions are merged there
     global _narrow_cache
     key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, x.dtype, mask.device)
     entry = _narrow_cache
@@ -300,9 +302,19 @@ def causal_conv1d_fn(
     if x.numel() == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
+    if _wants_grad(x, weight, bias) and initial_states is not None:
+        raise NotImplementedError("gradients through a call with initial_states are not implemented")
+    if torch.compiler.is_compiling():
+        # under torch.compile the launch is one opaque operator of the traced graph (trainer/train_pretrain.py:39
+        # and eval_model.py:157 compile the whole model, the latter with fullgraph=True)
+        result, fin = torch.ops.canon_conv1d.fwd(x, weight, bias, attention_mask, initial_states, seq_idx,
+                                                 final_states.shape[2] if final_states is not None else 0,
+                                                 act, res, rnd)
+        if final_states is None:
+            return result
+        final_states.copy_(fin)
+        return result, final_states
     if _wants_grad(x, weight, bias):
-        if initial_states is not None:
-            raise NotImplementedError("gradients through a call with initial_states are not implemented")
         result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd)
     else:
         result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd, seq_idx)
@@ -495,16 +507,25 @@ def causal_conv1d_update(
         if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x.device:
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
 
-    out = torch.empty((batch, dim), dtype=x.dtype, device=x.device)
+    if torch.compiler.is_compiling():
+        out = torch.ops.canon_conv1d.update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices,
+                                            act, res, rnd)
+    else:
+        out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
+    return out.unsqueeze(-1) if squeeze_back else out
+
+
+def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
+    out = torch.empty(tuple(x2.shape), dtype=x2.dtype, device=x2.device)
     if out.numel():
         p = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
         if cache_seqlens is not None:
             p.cache_seqlens = cache_seqlens.data_ptr()
         if conv_state_indices is not None:
             p.conv_state_indices = conv_state_indices.data_ptr()
-        rc = _call(_lib.lib().canon_conv1d_update, x.device, ctypes.byref(p))
+        rc = _call(_lib.lib().canon_conv1d_update, x2.device, ctypes.byref(p))
         _lib.check(rc, "causal_conv1d_update")
-    return out.unsqueeze(-1) if squeeze_back else out
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -576,9 +597,22 @@ def causal_conv1d_fn_parts(
         raise ValueError("cannot produce final states from an empty input")
 
     xs = [x if (x.stride(2) == 1 or x.stride(1) == 1) else x.contiguous() for x in xs]
-    if _wants_grad(*xs, weight, bias):
-        if initial_states is not None:
-            raise NotImplementedError("gradients through a call with initial_states are not implemented")
+    if _wants_grad(*xs, weight, bias) and initial_states is not None:
+        raise NotImplementedError("gradients through a call with initial_states are not implemented")
+    if torch.compiler.is_compiling():
+        if _wants_grad(*xs, weight, bias):
+            # traced training graphs: the differentiable single-tensor operator on the concatenation
+            y, fin = torch.ops.canon_conv1d.fwd(torch.cat(xs, dim=1), weight, bias, attention_mask, None, None,
+                                                final_states.shape[2] if final_states is not None else 0, act, res, rnd)
+            outs = tuple(y.split(dims, dim=1))
+        else:
+            *outs, fin = torch.ops.canon_conv1d.fwd_parts(xs, weight, bias, attention_mask, initial_states,
+                                                          final_states.shape[2] if final_states is not None else 0,
+                                                          act, res, rnd)
+            outs = tuple(outs)
+        if final_states is not None:
+            final_states.copy_(fin)
+    elif _wants_grad(*xs, weight, bias):
         result = _CanonConvPartsFn.apply(weight, bias, attention_mask, final_states, act, res, rnd, *xs)
         outs = tuple(result[:len(xs)])
     else:
@@ -675,15 +709,123 @@ def causal_conv1d_update_parts(
             raise ValueError(f"token_mask shape {tuple(token_mask.shape)} does not match (batch,) = ({batch},)")
         if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x0.device:
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
+    if torch.compiler.is_compiling():
+        return tuple(torch.ops.canon_conv1d.update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd))
+    return _launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd)
+
+
+def _launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd):
     outs = tuple(torch.empty_like(x, memory_format=torch.contiguous_format) for x in xs)
-    if batch * dim:
+    dim = sum(x.shape[1] for x in xs)
+    if xs[0].shape[0] * dim:
         p = _fill_update(xs[0], outs[0], conv_state, weight, bias, token_mask, act, res, rnd)
         p.channels = dim
         p.x = p.out = None
         arr = _part_array(xs, outs)
-        rc = _call(_lib.lib().canon_conv1d_update_parts, x0.device, ctypes.byref(p), arr, len(xs))
+        rc = _call(_lib.lib().canon_conv1d_update_parts, xs[0].device, ctypes.byref(p), arr, len(xs))
         _lib.check(rc, "causal_conv1d_update_parts")
     return outs
+
+
+# ---------------------------------------------------------------------------
+# The launches as torch operators, for traced graphs (torch.compile).  Eager calls do not go through them
+# (operator dispatch costs more than the launch); a function being traced does, because ctypes calls
+# cannot be traced and the reference compiles its model (trainer/train_pretrain.py:39, train_full_sft.py:54,
+# eval_model.py:157 with fullgraph=True).  Each has a shape-only twin for tracing, and the prefill has its
+# backward registered, so compiled training graphs differentiate through it.
+# ---------------------------------------------------------------------------
+def _new_state(x, channels: int, state_len: int) -> Optional[torch.Tensor]:
+    return torch.empty(x.shape[0], channels, state_len, dtype=x.dtype, device=x.device) if state_len > 0 else None
+
+
+@torch.library.custom_op("canon_conv1d::fwd", mutates_args=(), device_types="cuda")
+def _op_fwd(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], mask: Optional[torch.Tensor],
+            initial_states: Optional[torch.Tensor], seq_idx: Optional[torch.Tensor], state_len: int,
+            act: int, res: int, rnd: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    # functional (an operator with an autograd formula must be): the final states are a second result,
+    # of zero length when none are wanted
+    fin = _new_state(x, x.shape[1], state_len)
+    out = _launch_fwd(x, weight, bias, mask, initial_states, fin, act, res, rnd, seq_idx)
+    return out, fin if fin is not None else x.new_empty((x.shape[0], x.shape[1], 0))
+
+
+@_op_fwd.register_fake
+def _(x, weight, bias, mask, initial_states, seq_idx, state_len, act, res, rnd):
+    return torch.empty_like(x), x.new_empty((x.shape[0], x.shape[1], state_len))
+
+
+@torch.library.custom_op("canon_conv1d::bwd", mutates_args=(), device_types="cuda")
+def _op_bwd(x: torch.Tensor, dout: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+            mask: Optional[torch.Tensor], act: int, res: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    channels, width = weight.shape
+    dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
+    dbias = torch.empty(channels if bias is not None else 0, dtype=torch.float32, device=x.device)
+    dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias if bias is not None else None, act, res)
+    return dx, dweight.to(weight.dtype), dbias.to(bias.dtype if bias is not None else weight.dtype)
+
+
+@_op_bwd.register_fake
+def _(x, dout, weight, bias, mask, act, res):
+    return (torch.empty_like(x), torch.empty_like(weight, memory_format=torch.contiguous_format),
+            weight.new_empty((weight.shape[0] if bias is not None else 0,),
+                             dtype=bias.dtype if bias is not None else weight.dtype))
+
+
+def _op_fwd_setup(ctx, inputs, output):
+    x, weight, bias, mask, _initial, _seq, _state_len, act, res, _rnd = inputs
+    ctx.save_for_backward(x, weight, bias, mask)
+    ctx.flags = (act, res, bias is not None)
+
+
+def _op_fwd_backward(ctx, dout, _dstate):
+    x, weight, bias, mask = ctx.saved_tensors
+    act, res, has_bias = ctx.flags
+    dx, dweight, dbias = torch.ops.canon_conv1d.bwd(x, dout, weight, bias, mask, act, res)
+    return dx, dweight, (dbias if has_bias else None), None, None, None, None, None, None, None
+
+
+_op_fwd.register_autograd(_op_fwd_backward, setup_context=_op_fwd_setup)
+
+
+@torch.library.custom_op("canon_conv1d::update", mutates_args=("conv_state",), device_types="cuda")
+def _op_update(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+               token_mask: Optional[torch.Tensor], cache_seqlens: Optional[torch.Tensor],
+               conv_state_indices: Optional[torch.Tensor], act: int, res: int, rnd: int) -> torch.Tensor:
+    return _launch_update(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
+
+
+@_op_update.register_fake
+def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
+    return x.new_empty(tuple(x.shape))
+
+
+@torch.library.custom_op("canon_conv1d::fwd_parts", mutates_args=(), device_types="cuda")
+def _op_fwd_parts(xs: List[torch.Tensor], weight: torch.Tensor, bias: Optional[torch.Tensor],
+                  mask: Optional[torch.Tensor], initial_states: Optional[torch.Tensor],
+                  state_len: int, act: int, res: int, rnd: int) -> List[torch.Tensor]:
+    # one output per part, then the final states (zero length when none are wanted)
+    channels = sum(x.shape[1] for x in xs)
+    fin = _new_state(xs[0], channels, state_len)
+    outs = list(_launch_fwd_parts(xs, weight, bias, mask, initial_states, fin, act, res, rnd))
+    return outs + [fin if fin is not None else xs[0].new_empty((xs[0].shape[0], channels, 0))]
+
+
+@_op_fwd_parts.register_fake
+def _(xs, weight, bias, mask, initial_states, state_len, act, res, rnd):
+    channels = sum(x.shape[1] for x in xs)
+    return [torch.empty_like(x) for x in xs] + [xs[0].new_empty((xs[0].shape[0], channels, state_len))]
+
+
+@torch.library.custom_op("canon_conv1d::update_parts", mutates_args=("conv_state",), device_types="cuda")
+def _op_update_parts(xs: List[torch.Tensor], conv_state: torch.Tensor, weight: torch.Tensor,
+                     bias: Optional[torch.Tensor], token_mask: Optional[torch.Tensor], act: int, res: int,
+                     rnd: int) -> List[torch.Tensor]:
+    return list(_launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd))
+
+
+@_op_update_parts.register_fake
+def _(xs, conv_state, weight, bias, token_mask, act, res, rnd):
+    return [torch.empty_like(x, memory_format=torch.contiguous_format) for x in xs]
 
 
 # ---------------------------------------------------------------------------

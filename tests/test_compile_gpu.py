@@ -223,3 +223,37 @@ def test_the_reference_modules_accelerated_branch_compiles_whole(cc):
         want = decode(tok, state_e, weight)
         got, seen = graphs_of(decode, tok, state_c, weight)
         assert len(seen) == 1 and torch.equal(bits(got), bits(want)) and torch.equal(bits(state_c), bits(state_e)), step
+
+
+def test_whole_model_with_canon_layers_and_caches_traces_as_one_graph(cc):
+    """A Viby-shaped model (Canon A-D on the HIP CanonLayer, conv states on the cache object, q/k/v and gate/up
+    either concatenated or as parts): prefill and single-token steps each trace without a graph break and
+    reproduce the eager logits."""
+    import viby_harness as vh
+    from causal_conv1d.canon import CanonLayer
+
+    class Cache:   # a plain object, as the HF cache the reference hangs its lists on (model/model.py:227-241)
+        def __init__(self, n):
+            self._max_layers, self.kv, self.seen = n, [None] * n, 0
+
+    cfg = vh.viby_config(num_hidden_layers=2, hidden_size=128, intermediate_size=256, vocab_size=512)
+    for parts in (False, True):
+        model = vh.init_weights(vh.VibyShaped(cfg, lambda C, name: CanonLayer(C, cfg, name), parts=parts), 0,
+                                torch.bfloat16, DEV).eval()
+        ids = torch.randint(0, 512, (2, 40), generator=torch.Generator().manual_seed(7)).to(DEV)
+        steps = [ids] + [torch.randint(0, 512, (2, 1), generator=torch.Generator().manual_seed(8 + i)).to(DEV)
+                         for i in range(2)]
+        with torch.no_grad():
+            cache_e, cache_c = Cache(cfg.num_hidden_layers), Cache(cfg.num_hidden_layers)
+            seen_tokens = 0
+            for i, tok in enumerate(steps):
+                seen_tokens += tok.shape[1]
+                mask = torch.ones(2, seen_tokens, dtype=torch.int64, device=DEV)
+                want = model.forward(tok, cache_e, mask)
+                torch._dynamo.reset()
+                got, seen = graphs_of(model.forward, tok, cache_c, mask)
+                assert len(seen) == 1, (parts, i, len(seen))
+                assert torch.equal(got, want), (parts, i)
+                for site in "abcd":
+                    for a, e in zip(getattr(cache_c, f"canon_cache_{site}"), getattr(cache_e, f"canon_cache_{site}")):
+                        assert torch.equal(bits(a), bits(e)), (parts, i, site)

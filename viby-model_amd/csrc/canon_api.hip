@@ -123,7 +123,6 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.S_in = p->initial_state ? p->initial_len : 0;
     a.S_out = p->final_state ? p->final_len : 0;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
-    a.b_vec = p->bias && aligned16(p->bias);
     a.tap_mode = tap_mode_of(a.w_vec != 0, p->bias, p->x_dtype, p->w_dtype);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
@@ -249,7 +248,6 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode; a.eager = p->round_mode;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
-    a.b_vec = p->bias && aligned16(p->bias);
     a.tap_mode = tap_mode_of(a.w_vec != 0, p->bias, p->x_dtype, p->w_dtype);
     plan->kind = UPD_GENERIC;
     plan->grid = 0;
@@ -449,7 +447,6 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode;
     a.w_vec = p->width == 4 && p->w_stride_k == 1 && p->w_stride_c == 4 && aligned16(p->weight);
-    a.b_vec = p->bias && aligned16(p->bias);
     plan->kind = BWD_GENERIC;
     plan->U = 1;
     plan->grid = 0;

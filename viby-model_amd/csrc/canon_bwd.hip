@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     const int64_t Lm1 = (int64_t)a.L - 1;
 
     RawTaps<E> raw;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, false, false, c0, raw);
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, false, c0, raw);
 
     // rows t_end-4 .. t_end+2 of xm (window for the last step + the three steps past the chunk)
     float xr7[7][E], m7[7];
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     const int ntiles = (int)(a.chunk / (uint32_t)(R * NW));
 
     RawTaps<E> rawt;
-    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, rawt);
+    fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, rawt);
     float w[E][W], bias[E];
     if constexpr (MASK) {
         for (uint32_t i = threadIdx.x; i < a.chunk + 6u; i += 64u * NW) {

@@ -527,7 +527,7 @@ template <int NC> struct RawTaps {
 
 template <int W, int NC>
 __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias, int64_t w_sc, int64_t w_sk,
-                                           int w_dtype, bool vec, bool bvec, uint32_t c0, RawTaps<NC> &r)
+                                           int w_dtype, bool vec, uint32_t c0, RawTaps<NC> &r)
 {
     const bool wide = w_dtype == CANON_DTYPE_F32;
     // bias first: whatever follows the tap loads may wait on them, and nothing must be issued after a wait
@@ -535,13 +535,6 @@ __device__ __forceinline__ void fetch_taps(const void *weight, const void *bias,
         if (wide) {
 #pragma unroll
             for (int e = 0; e < NC; ++e) r.b[e] = ((const uint32_t *)bias)[c0 + e];
-        } else if (NC == 8 && bvec) {
-            // eight 16-bit biases are one aligned 16-byte run (c0 is a multiple of 8)
-            const uint4 q = *(const uint4 *)((const uint16_t *)bias + c0);
-            r.b[0] = q.x & 0xFFFFu; r.b[1 % NC] = q.x >> 16;
-            r.b[2 % NC] = q.y & 0xFFFFu; r.b[3 % NC] = q.y >> 16;
-            r.b[4 % NC] = q.z & 0xFFFFu; r.b[5 % NC] = q.z >> 16;
-            r.b[6 % NC] = q.w & 0xFFFFu; r.b[7 % NC] = q.w >> 16;
         } else {
 #pragma unroll
             for (int e = 0; e < NC; ++e) r.b[e] = ((const uint16_t *)bias)[c0 + e];
@@ -599,9 +592,9 @@ __device__ __forceinline__ void fetch_taps_uniform(const void *weight, const voi
             const uint32_t d = ((const uint32_t *)bias)[c >> 1];
             r.b[0] = (c & 1u) ? (d >> 16) : (d & 0xFFFFu);
         }
-        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, false, c, r);
+        fetch_taps<W, 1>(weight, nullptr, w_sc, w_sk, w_dtype, vec, c, r);
     } else {
-        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, false, c, r);
+        fetch_taps<W, 1>(weight, bias, w_sc, w_sk, w_dtype, vec, c, r);
     }
 }
 

@@ -53,7 +53,7 @@ struct FwdArgs {
     int64_t i_sb, i_sc, i_ss;
     int64_t f_sb, f_sc, f_ss;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_vec, b_pair, m_vec, nt, tap_mode;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_pair, m_vec, nt, tap_mode;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
     uint32_t nseg;      // bcl: segments per row       generic: time chunks per row
@@ -87,7 +87,7 @@ struct UpdArgs {
     // third line: what the vectorised kernel reads off its usual path (state pool, general tap path)
     const int32_t *indices;   // conv_state row of batch entry b (state pool shared by many sequences)
     int64_t w_sc, w_sk;
-    int32_t w_vec, b_vec;
+    int32_t w_vec;
     // the rest: strided kernel, ring buffer, launch geometry
     const int32_t *seqlens;   // circular-buffer mode: conv_state is written at seqlens[b] % S, not shifted
     int64_t x_sc, o_sc;
@@ -116,7 +116,7 @@ struct BwdArgs {
     int64_t w_sc, w_sk;
     int64_t m_sb, m_sl;
     uint32_t B, C, L;
-    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_vec, b_pair, m_vec;
+    int32_t W, w_dtype, mask_dtype, act, res_mode, w_vec, b_pair, m_vec;
     uint32_t nvec;      // channel groups per row (C / E)
     uint32_t nchunk;    // time chunks per sequence
     uint32_t chunk;     // time steps per chunk

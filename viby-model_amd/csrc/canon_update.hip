@@ -32,7 +32,7 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
     TapWords<WDT, E> tw;
     RawTaps<E> raw;
     if constexpr (MODE == TAPS_ANY) {
-        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, false, c0, raw);
+        fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
     } else {
         static_assert(MODE == TAPS_ANY || W == 4, "the contiguous tap layouts are [C, 4]");
         fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);

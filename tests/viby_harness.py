@@ -108,6 +108,17 @@ class Block(nn.Module):
         return h + self.down_proj(F.silu(gate) * up)
 
 
+class DecodeCache:
+    """What the layers hang their per-layer state on: kv[i] = (K, V), the Canon layers' canon_cache_<name>
+    lists (model/model.py:227-241 does the same on the HF cache object).  A plain class, so that attribute
+    reads and writes trace under torch.compile."""
+
+    def __init__(self, n_layers: int):
+        self._max_layers = n_layers
+        self.kv = [None] * n_layers
+        self.seen = 0
+
+
 class VibyShaped(nn.Module):
     def __init__(self, cfg, make_canon, parts: bool = False):
         super().__init__()
@@ -117,8 +128,7 @@ class VibyShaped(nn.Module):
         self.norm = nn.RMSNorm(cfg.hidden_size, eps=cfg.rms_norm_eps)
 
     def new_cache(self):
-        n = self.cfg.num_hidden_layers
-        return types.SimpleNamespace(_max_layers=n, kv=[None] * n, seen=0)
+        return DecodeCache(self.cfg.num_hidden_layers)
 
     def forward(self, ids, cache, mask):
         h = self.embed_tokens(ids)
@@ -148,11 +158,13 @@ class VibyShaped(nn.Module):
 
 
 @torch.no_grad()
-def generate_graphed(model: VibyShaped, ids: torch.Tensor, steps: int, capture: bool = True):
+def generate_graphed(model: VibyShaped, ids: torch.Tensor, steps: int, capture=True, compile_kwargs=None):
     """Prefill eagerly, then ONE captured HIP graph per generated token (all layers: 72 Canon update launches,
     projections, attention over a preallocated KV buffer, head, argmax, feeding the token back), replayed
     steps-1 times without any host work in between.  With capture=False the same step function is called
     eagerly instead (same kernels, launched one by one): the reference the replays must match bit for bit.
+    With capture="compile" the step function goes through torch.compile(fullgraph=True, **compile_kwargs)
+    instead (what eval_model.py:157 does to the reference model).
     Returns (tokens [B, steps], logits [steps, B, V])."""
     dev = ids.device
     B, T = ids.shape
@@ -197,13 +209,15 @@ def generate_graphed(model: VibyShaped, ids: torch.Tensor, steps: int, capture: 
     cache.pos_t.fill_(T)
 
     graph = None
-    if capture:
+    if capture == "compile":
+        step = torch.compile(step, fullgraph=True, **(compile_kwargs or {}))
+    elif capture:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             step()
     toks, logits = [tok0[:, 0].clone()], [logits0]
     for _ in range(steps - 1):
-        if capture:
+        if graph is not None:
             graph.replay()
         else:
             step()

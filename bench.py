@@ -334,10 +334,10 @@ def main():
         "metric": "Canon conv1d HBM GB/s (prefill B8 L1024 C3456 bf16); decode us/step B256",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 storage, f32 accumulate", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: prefill bf16 x[B=8,C=3456,L=1024] time-contiguous, width 4, "
                                "bias, residual fused, no activation", "kernel": plan,
-                   "rotating_buffer_pairs": nbuf},
+                   "storage": "bf16", "accumulate": "f32", "rotating_buffer_pairs": nbuf},
         "tokens_per_s": round(B * L / (ms * 1e-3)),
         "device_copy_same_bytes": {"ms_per_step": round(ms_copy, 6),
                                    "GB/s": round(2 * B * C * L * 2 / (ms_copy * 1e-3) / 1e9, 1),

@@ -508,9 +508,12 @@ __global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_parts_kernel(con
 
 // ---------------------------------------------------------------------------
 // prefill, any strides / any length / either rounding mode: one thread per
-// (b, c, chunk of time steps), scalar accesses.
+// (b, c, chunk of time steps), scalar accesses.  STEPWISE: the chunk is walked
+// step by step (time-contiguous rows); otherwise everything it reads is
+// requested at once.  Two instances because the second needs twice the
+// registers, which costs the first its occupancy.
 // ---------------------------------------------------------------------------
-template <int DT>
+template <int DT, bool STEPWISE>
 __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
@@ -540,53 +543,126 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
     const int64_t t_stop = t_begin + (int64_t)a.chunk;
     const int64_t t_end = t_stop < (int64_t)a.L ? t_stop : (int64_t)a.L;
 
-    float h[3] = {0, 0, 0};
-    int32_t qh[3] = {0, 0, 0};   // with seq_idx: the sequence each history position belongs to
     const int32_t *seq = a.seq ? a.seq + (int64_t)b * a.q_sb : nullptr;
-    for (int j = 4 - W; j < 3; ++j) {
-        const int64_t t = t_begin - 3 + j;
-        if (t >= 0) {
-            float v = load1<DT>(a.x, xo + t * a.x_sl);
-            if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
-            h[j] = v;
-            if (seq) qh[j] = seq[t * a.q_sl];
-        } else if (a.init && a.S_in + t >= 0) {
-            h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+    if constexpr (STEPWISE) {
+        // time-contiguous rows: step by step (a thread's steps are adjacent bytes, the loads after the first
+        // hit the cache; requesting the chunk at once, as below, measured 15 % slower here)
+        float h[3] = {0, 0, 0};
+        int32_t qh[3] = {0, 0, 0};   // with seq_idx: the sequence each history position belongs to
+        for (int j = 4 - W; j < 3; ++j) {
+            const int64_t t = t_begin - 3 + j;
+            if (t >= 0) {
+                float v = load1<DT>(a.x, xo + t * a.x_sl);
+                if (a.mask) v = mul_round<DT>(v, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+                h[j] = v;
+                if (seq) qh[j] = seq[t * a.q_sl];
+            } else if (a.init && a.S_in + t >= 0) {
+                h[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+            }
         }
-    }
-    for (int64_t t = t_begin; t < t_end; ++t) {
-        const float xr = load1<DT>(a.x, xo + t * a.x_sl);
-        float xm = xr;
-        if (a.mask) xm = mul_round<DT>(xr, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
-        float acc = bv;
+        for (int64_t t = t_begin; t < t_end; ++t) {
+            const float xr = load1<DT>(a.x, xo + t * a.x_sl);
+            float xm = xr;
+            if (a.mask) xm = mul_round<DT>(xr, load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype));
+            float acc = bv;
+            if (seq) {
+                // inputs of another packed sequence enter as zeros
+                const int32_t qt = seq[t * a.q_sl];
+                if (W == 4) acc = fmaf(w[0], qh[0] == qt ? h[0] : 0.0f, acc);
+                if (W >= 3) acc = fmaf(w[1], qh[1] == qt ? h[1] : 0.0f, acc);
+                acc = fmaf(w[2], qh[2] == qt ? h[2] : 0.0f, acc);
+                acc = fmaf(w[3], xm, acc);
+                qh[0] = qh[1];
+                qh[1] = qh[2];
+                qh[2] = qt;
+            } else {
+                if (W == 4) acc = fmaf(w[0], h[0], acc);
+                if (W >= 3) acc = fmaf(w[1], h[1], acc);
+                acc = fmaf(w[2], h[2], acc);
+                acc = fmaf(w[3], xm, acc);
+            }
+            if (a.eager) {
+                acc = round_through<DT>(acc);
+                if (a.act) acc = round_through<DT>(silu_precise(acc));
+                if (a.res_mode == CANON_RESIDUAL_MASKED) acc += xm;
+                else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
+            } else {
+                acc = finish(acc, a.act, a.res_mode, xm, xr);
+            }
+            store1<DT>(a.out, oo + t * a.o_sl, acc);
+            h[0] = h[1];
+            h[1] = h[2];
+            h[2] = xm;
+        }
+    } else {
+        // Everything the chunk reads is requested before anything is computed (positions past the end are
+        // clamped to the last one and never used): stepping through the chunk with a load, a wait and a store per
+        // time step costs one memory round trip per step, because the loads cannot be moved above the stores.
+        constexpr int N = (int)kGenericChunk, NH = N + 3;        // the chunk and the three steps before it
+        const int64_t last = (int64_t)a.L - 1;
+        float xr[NH], mk[NH];
+        int32_t sq[NH];
+        int64_t tpos[NH];
+#pragma unroll
+        for (int j = 0; j < NH; ++j) {
+            const int64_t t = t_begin - 3 + j;
+            tpos[j] = t < 0 ? 0 : (t > last ? last : t);
+            xr[j] = load1<DT>(a.x, xo + tpos[j] * a.x_sl);
+            mk[j] = 1.0f;
+            sq[j] = 0;
+        }
         if (seq) {
-            // inputs of another packed sequence enter as zeros
-            const int32_t qt = seq[t * a.q_sl];
-            if (W == 4) acc = fmaf(w[0], qh[0] == qt ? h[0] : 0.0f, acc);
-            if (W >= 3) acc = fmaf(w[1], qh[1] == qt ? h[1] : 0.0f, acc);
-            acc = fmaf(w[2], qh[2] == qt ? h[2] : 0.0f, acc);
-            acc = fmaf(w[3], xm, acc);
-            qh[0] = qh[1];
-            qh[1] = qh[2];
-            qh[2] = qt;
-        } else {
-            if (W == 4) acc = fmaf(w[0], h[0], acc);
-            if (W >= 3) acc = fmaf(w[1], h[1], acc);
-            acc = fmaf(w[2], h[2], acc);
-            acc = fmaf(w[3], xm, acc);
+#pragma unroll
+            for (int j = 0; j < NH; ++j) sq[j] = seq[tpos[j] * a.q_sl];
         }
-        if (a.eager) {
-            acc = round_through<DT>(acc);
-            if (a.act) acc = round_through<DT>(silu_precise(acc));
-            if (a.res_mode == CANON_RESIDUAL_MASKED) acc += xm;
-            else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
-        } else {
-            acc = finish(acc, a.act, a.res_mode, xm, xr);
+        if (a.mask) {
+            int64_t idx[NH];
+#pragma unroll
+            for (int j = 0; j < NH; ++j) idx[j] = (int64_t)b * a.m_sb + tpos[j] * a.m_sl;
+            load_mask_entries<NH, false>(a.mask, 0, idx, a.mask_dtype, mk);
         }
-        store1<DT>(a.out, oo + t * a.o_sl, acc);
-        h[0] = h[1];
-        h[1] = h[2];
-        h[2] = xm;
+        // masked inputs; before the start of the sequence: the initial state, or zero
+        float xm[NH];
+#pragma unroll
+        for (int j = 0; j < NH; ++j) {
+            const int64_t t = t_begin - 3 + j;
+            xm[j] = a.mask ? mul_round<DT>(xr[j], mk[j]) : xr[j];
+            if (t < 0) {
+                xm[j] = 0.0f;
+                if (j >= 4 - W && a.init && a.S_in + t >= 0)
+                    xm[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (a.S_in + t) * a.i_ss);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int64_t t = t_begin + j;
+            if (t >= t_end) break;
+            const float x0 = xm[j], x1 = xm[j + 1], x2 = xm[j + 2], x3 = xm[j + 3];   // steps t-3 .. t
+            float acc = bv;
+            if (seq) {
+                // inputs of another packed sequence enter as zeros (neither do positions before the start count:
+                // they carry no index of their own and the call has no initial state with seq_idx)
+                const int32_t qt = sq[j + 3];
+                if (W == 4) acc = fmaf(w[0], (t >= 3 && sq[j] == qt) ? x0 : 0.0f, acc);
+                if (W >= 3) acc = fmaf(w[1], (t >= 2 && sq[j + 1] == qt) ? x1 : 0.0f, acc);
+                acc = fmaf(w[2], (t >= 1 && sq[j + 2] == qt) ? x2 : 0.0f, acc);
+                acc = fmaf(w[3], x3, acc);
+            } else {
+                if (W == 4) acc = fmaf(w[0], x0, acc);
+                if (W >= 3) acc = fmaf(w[1], x1, acc);
+                acc = fmaf(w[2], x2, acc);
+                acc = fmaf(w[3], x3, acc);
+            }
+            if (a.eager) {
+                acc = round_through<DT>(acc);
+                if (a.act) acc = round_through<DT>(silu_precise(acc));
+                if (a.res_mode == CANON_RESIDUAL_MASKED) acc += x3;
+                else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr[j + 3];
+            } else {
+                acc = finish(acc, a.act, a.res_mode, x3, xr[j + 3]);
+            }
+            store1<DT>(a.out, oo + t * a.o_sl, acc);
+        }
     }
     if (a.fin && ch == a.nseg - 1)
         for (int slot = 0; slot < a.S_out; ++slot) capture_row_state<DT>(a, b, c, slot);
@@ -640,7 +716,8 @@ template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
 {
     if (pl.kind == FWD_GENERIC) {
-        hipLaunchKernelGGL((canon_fwd_generic_kernel<DT>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        if (pl.args.x_sl == 1) hipLaunchKernelGGL((canon_fwd_generic_kernel<DT, true>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_fwd_generic_kernel<DT, false>), dim3(pl.grid), dim3(256), 0, s, pl.args);
         return;
     }
     switch (pl.args.W) {

@@ -259,7 +259,7 @@ int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
 
 /*
  * Name of the kernel family the call above would launch for these arguments
- * ("bcl_vec", "blc_vec", "blc_vec_seq", "generic", "update_vec", "update_generic"), or NULL
+ * ("bcl_vec", "bcl_vec_short", "blc_vec", "blc_vec_seq", "generic", "update_vec", "update_generic"), or NULL
  * if the arguments are rejected.  Launches nothing.  Lets a caller or a test
  * assert that a layout takes the fast path.
  */

@@ -105,7 +105,16 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     assert plan(fwd_params(C=3457, layout="blc")) == "generic"
     assert plan(fwd_params(x=FAKE_X + 2)) == "generic"
     assert plan(fwd_params(round_mode=1)) == "generic"
-    assert plan(fwd_params(L=64)) == "generic"                             # rows too short for a wave
+    # rows too short for a wave of their own: several rows per wave, as long as they are whole aligned vectors
+    assert plan(fwd_params(L=64)) == "bcl_vec_short"
+    assert plan(fwd_params(L=8)) == "bcl_vec_short"
+    assert plan(fwd_params(L=120)) == "bcl_vec_short"
+    assert plan(fwd_params(L=128)) == "bcl_vec_short" and plan(fwd_params(L=256)) == "bcl_vec_short"
+    assert plan(fwd_params(L=264)) == "bcl_vec"
+    assert plan(fwd_params(L=255)) == "bcl_vec"                            # ... not whole vectors, but long enough
+    assert plan(fwd_params(L=60)) == "generic"                             # ... not whole vectors
+    assert plan(fwd_params(L=4)) == "generic"
+    assert plan(fwd_params(L=64, round_mode=1)) == "generic"
     # strided but aligned rows (a channel slice of a bigger tensor) stay vectorised
     assert plan(fwd_params(C=128, x_stride_b=4096 * 1024, x_stride_c=1024)) == "bcl_vec"
 

@@ -542,6 +542,43 @@ def test_time_contiguous_rows_off_the_16_byte_grid(cc, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_short_time_contiguous_rows_share_a_wave(cc, dtype):
+    """Rows of 1..32 whole vectors: 2..64 rows per wave (every power-of-two group size, vector counts on and
+    off the powers of two, row counts that leave the last wave partly empty), all options, both state ends."""
+    g = torch.Generator().manual_seed(92)
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    shapes = [(3, 7, 1), (2, 33, 2), (1, 5, 3), (2, 9, 5), (3, 16, 8), (1, 21, 13), (2, 6, 16), (1, 11, 17), (2, 3, 31), (1, 67, 32)]
+    for (B, C, nvec), W in itertools.product(shapes, [2, 3, 4]):
+        L = nvec * E
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, W, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+        init = torch.randn(B, C, 5, generator=g).to(dtype)
+        for act, res, m, st in [(None, False, None, False), ("silu", "masked", mask, True), (None, "unmasked", mask, False),
+                                ("silu", True, None, True)]:
+            want = co.conv1d_fwd(x, w, b, mask=m, activation=act, residual=res,
+                                 initial_state=init if st else None, final_state_len=8 if st else None)
+            xg = x.to(DEV)
+            assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec_short", (B, C, L)
+            got = run_fwd(cc, xg, w, b, act=act, mask=m, residual=res, init=init if st else None, S_out=8 if st else None)
+            what = f"short/{dtype}/{B}x{C}x{L}/W{W}/{act}/{res}/mask{m is not None}/state{st}"
+            xm = x if m is None else (x.float() * m[:, None, :].float()).to(dtype)
+            if st:
+                assert_parity(got[0], want[0], exact=act is None, what=what, res=xm if res else None)
+                assert torch.equal(bits(got[1]), bits(want[1])), what
+            else:
+                assert_parity(got, want, exact=act is None, what=what, res=xm if res else None)
+    # channel slices of a wider tensor keep the kernel as long as the rows stay on the 16-byte grid
+    big = torch.randn(2, 40, 4 * E, generator=g).to(dtype)
+    w = (torch.randn(24, 4, generator=g) * 0.3).to(dtype)
+    xg = big.to(DEV)[:, 8:32]
+    assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec_short"
+    assert_parity(run_fwd(cc, xg, w, None, residual=True), co.conv1d_fwd(big[:, 8:32].contiguous(), w, None, residual=1),
+                  exact=True, what="short/slice")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_update_ring_buffer_and_state_pool(cc, dtype):
     """cache_seqlens (ring buffer) and conv_state_indices (rows of a state pool) against the oracle, whose
     two modes are pinned by their equivalence with the shift register."""
@@ -642,7 +679,7 @@ def test_randomised_shapes_layouts_and_options(cc):
         added = None if not res else (x if res == "unmasked" else xm)      # the term the sum may cancel against
         assert_parity(got, want, exact=act is None, what=what, res=added)
     # the draw reaches every kernel family
-    assert set(plans) >= {"bcl_vec", "blc_vec", "blc_vec_seq", "generic"}, plans
+    assert set(plans) >= {"bcl_vec", "bcl_vec_short", "blc_vec", "blc_vec_seq", "generic"}, plans
 
 
 def test_randomised_decode_steps(cc):

@@ -251,6 +251,96 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// prefill, time-contiguous rows of at most 32 vectors (whole vectors, 16-byte
+// aligned): a row takes P = 1, 2, 4, .. 32 adjacent lanes of a wave (the next
+// power of two from its vector count) and a wave 64 / P rows, so short prompts
+// keep most lanes busy and every access is a 16-byte one.  A lane's history is
+// its left neighbour's last three inputs (wave shift) unless it holds the
+// first vector of its row; the rows of a wave belong to different channels, so
+// each lane loads its own taps.  Field use: nseg = P, chunk = log2(P),
+// ntasks = rows (B * C), nvec = vectors per row.
+// ---------------------------------------------------------------------------
+template <int DT, int W, bool MASK>
+__global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs a)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    const uint32_t shift = a.chunk, P = a.nseg;
+    const uint32_t first_row = wave * (64u >> shift);
+    if (first_row >= a.ntasks) return;
+    const uint32_t sub = lane & (P - 1u);
+    const uint32_t row = first_row + (lane >> shift);
+    const bool row_ok = row < a.ntasks;
+    const uint32_t rr = row_ok ? row : a.ntasks - 1u;            // idle lanes shadow the last row / vector:
+    const uint32_t v = sub < a.nvec ? sub : a.nvec - 1u;         // loads need no predicate
+    const bool active = row_ok && sub < a.nvec;
+    const uint32_t b = fdiv(rr, a.div_C);
+    const uint32_t c = rr - b * a.C;
+    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
+    char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
+
+    const uint4 X = load_vec<false>(xrow + (int64_t)v * 16);
+    RawTaps<1> raw;
+    fetch_taps<W, 1>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c, raw);
+    float M[1][E];
+    if constexpr (MASK) {
+        const int64_t mbase[1] = {(int64_t)b * a.m_sb + (int64_t)v * E * a.m_sl};
+        load_mask_vec<E, 1>(a.mask, mbase, a.m_sl, a.mask_dtype, a.m_vec != 0, M);
+    }
+    float w[1][W], bvv[1];
+    decode_taps<DT, W, 1>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bvv);
+    const float bv = bvv[0];
+
+    float xr[E], xm_store[MASK ? E : 1];
+    float *xm = MASK ? xm_store : xr;
+    unpack_vec<DT>(X, xr);
+    if constexpr (MASK) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) xm[j] = mul_round<DT>(xr[j], M[0][j]);
+    }
+    // seq[0..2] = the three masked inputs before this vector
+    float seq[E + 3];
+    seq[0] = wave_shift_up(xm[E - 3], 0.0f);
+    seq[1] = wave_shift_up(xm[E - 2], 0.0f);
+    seq[2] = wave_shift_up(xm[E - 1], 0.0f);
+    if (sub == 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            seq[j] = 0.0f;
+            if (j >= 3 - (W - 1) && a.init)
+                seq[j] = load1<DT>(a.init, b * a.i_sb + c * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < E; ++j) seq[3 + j] = xm[j];
+
+    float o[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+        float acc = bv;
+#pragma unroll
+        for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
+        o[j] = acc;
+    }
+    if (a.act) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) o[j] = silu_fast(o[j]);
+    }
+    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) o[j] += xr[j];
+    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) o[j] += xm[j];
+    }
+    if (active) store_vec<false>(orow + (int64_t)v * 16, pack_vec<DT>(o));
+
+    if (a.fin && row_ok)
+        for (uint32_t slot = sub; slot < (uint32_t)a.S_out; slot += P) capture_row_state<DT>(a, b, c, (int)slot);
+}
+
+// ---------------------------------------------------------------------------
 // prefill, channel-contiguous rows ([B, L, C] memory, x_stride_c == 1): the
 // layout CanonLayer hands over (a transposed view of [B, T, D]).
 //
@@ -691,7 +781,8 @@ template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, 
 
 template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
 {
-    if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
+    if (pl.kind == FWD_BCL_SHORT) hipLaunchKernelGGL((canon_fwd_bcl_short_kernel<DT, W, MASK>), dim3(pl.grid), dim3(256), 0, s, pl.args);
+    else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
     else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
 }
 

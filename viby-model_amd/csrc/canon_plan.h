@@ -150,7 +150,7 @@ constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 %
 constexpr int kBwdSlab = CANON_BWD_SLAB;    // time steps per wave and tile
 constexpr int kBwdWaves = 4;
 constexpr int kBwdMaxChunk = 32 * kBwdSlab * kBwdWaves;   // most time steps one block of the channel-contiguous backward walks
-enum FwdKind { FWD_BCL, FWD_BLC, FWD_GENERIC };
+enum FwdKind { FWD_BCL, FWD_BCL_SHORT, FWD_BLC, FWD_GENERIC };
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel

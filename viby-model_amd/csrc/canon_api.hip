@@ -153,16 +153,18 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
                         a.x_sb % EB == 0 && a.x_sl % EB == 0 && a.o_sb % EB == 0 && a.o_sl % EB == 0 &&
                         a.x_sl != 1;
 
-    // time-contiguous rows of at most 32 whole, aligned vectors share a wave (measured against one row per
-    // wave, the kernel below: 2.3x faster at 16 vectors per row, 1.3x at 32)
+    // Time-contiguous rows of at most 32 whole, aligned vectors share waves (canon_fwd_bcl_short_kernel):
+    // measured against one row per wave, the kernel below, 2.3x faster at 16 vectors per row, 1.3x at 32.
+    // (Longer rows packed back to back the same way lose to the kernel below even where it leaves half of its
+    // lanes idle: 4.4-4.6 against 5.1-5.7 TB/s.)
     const uint32_t kBclShortMaxVectors = 32;
     if (!p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && bcl_aligned && a.L / E >= 1 &&
         a.L / E <= kBclShortMaxVectors && rows < (1ull << 31)) {
         const uint32_t nvec = a.L / E;
         uint32_t shift = 0;
-        while ((1u << shift) < nvec) ++shift;            // lanes per row: the next power of two
-        const uint64_t rows_per_wave = 64u >> shift;
-        const uint64_t nwaves = (rows + rows_per_wave - 1) / rows_per_wave;
+        while ((1u << shift) < nvec) ++shift;                  // one group of lanes per row: the next power of two
+        const uint64_t groups_per_wave = 64u >> shift;
+        const uint64_t nwaves = (rows + groups_per_wave - 1) / groups_per_wave;
         plan->kind = FWD_BCL_SHORT;
         a.nvec = nvec; a.nseg = 1u << shift; a.chunk = shift; a.ntasks = (uint32_t)rows;
         a.div_C = make_fastdiv(a.C);
@@ -172,13 +174,19 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     }
     if (bcl_ok) {
         const uint32_t nvec = a.L / E;
-        // vectors per lane (1, 2 or 4): the largest that leaves no more lane slots idle than one vector
-        // per lane would and still keeps >= 2048 waves in flight
+        // vectors per lane (1, 2 or 4): the fewest that reach the smallest number of segments per row while
+        // >= 2048 waves stay in flight.  Every segment after a row's first re-reads its three inputs of history
+        // from memory after the wave's own loads, a second round trip: rows of 144..192 vectors as three
+        // segments of one vector per lane ran at 3.3-4.2 TB/s, as one segment of four (half of those idle) at
+        // 5+ TB/s.  Idle lane slots cost next to nothing here.
         int U = 1;
-        const uint64_t slots1 = (nvec + 63u) / 64u;
+        uint64_t best = (nvec + 63u) / 64u;
         for (int cand = 2; cand <= 4; cand *= 2) {
             const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
-            if (nseg * cand <= slots1 && rows * nseg >= 2048) U = cand;
+            if (nseg < best && rows * nseg >= 2048) {
+                U = cand;
+                best = nseg;
+            }
         }
         const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
         const uint64_t ntasks = rows * nseg;

@@ -105,6 +105,30 @@ def test_backward_blocks_that_walk_several_tiles(cc, dtype):
         check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_time_contiguous_rows_with_partly_idle_vector_slots(cc, dtype):
+    """Time-contiguous rows whose vector count is not a multiple of 64: the planner gives a lane 2 or 4 vectors
+    to keep a row in one segment, so some of a lane's slots lie past the end of the row (65, 144 vectors),
+    and rows that need two segments of four (300 vectors).  Forward and backward against the float64 oracle."""
+    g = torch.Generator().manual_seed(30)
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    for nvec in (65, 144, 300):
+        B, C, L = 2, 1024, nvec * E      # 2048 rows: enough for the planner to give a lane several vectors
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, 4, generator=g) * 0.5).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.2).to(dtype)
+        dout = torch.randn(B, C, L, generator=g).to(dtype)
+        mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+        for act, residual, m in [("silu", "masked", mask), (None, "unmasked", None)]:
+            dx, dw, db, out = gpu_grads(cc, x, w, b, dout, "bcl", m, act, residual)
+            rdx, rdw, rdb, rout = conv1d_grads(x, w, b, dout, m, act, residual)
+            what = f"{dtype} {nvec} vectors {act} {residual} mask{m is not None}"
+            check(out, rout, dtype, what + " out")
+            check(dx, rdx, dtype, what + " dx")
+            check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
+            check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
 def test_backward_finite_differences_like_the_reference_tests(cc):
     """causal-conv1d-mps/test.py:259-272 and :275-291: eps 1e-3, atol 1e-3, rtol 1e-2, loss = out.sum()."""
     torch.manual_seed(0)

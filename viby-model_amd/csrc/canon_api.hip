@@ -488,10 +488,15 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     if (rows) {
         const uint32_t nvec = a.L / E;
         const uint64_t nrows = (uint64_t)a.B * a.C;
+        // vectors per lane: the fewest that reach the smallest number of segments per row (see plan_fwd)
         int U = 1;
+        uint64_t best = (nvec + 63u) / 64u;
         for (int cand = 2; cand <= 4; cand *= 2) {
             const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
-            if (nvec >= 64u * cand && nrows * nseg >= 2048) U = cand;
+            if (nseg < best && nrows * nseg >= 2048) {
+                U = cand;
+                best = nseg;
+            }
         }
         const uint64_t nseg = (nvec + 64u * U - 1) / (64u * U);
         const uint64_t ntasks = nrows * nseg;

@@ -526,13 +526,21 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         const uint32_t nvec = a.C / E8;
         const uint32_t nct = (nvec + 63) / 64;
         // time steps per block: as long as possible (few partial sets to write and to add up, taps and
-        // chunk-end work amortised) while the grid still has one and a half blocks per CU
-        uint32_t chunk = tile;
-        for (uint32_t cand = 2 * tile; cand <= (uint32_t)kBwdMaxChunk; cand *= 2) {
-            const uint64_t blocks = (uint64_t)a.B * ((a.L + cand - 1) / cand) * nct;
-            if (2 * blocks >= 256ull * kBwdHalfBlocksPerCU) chunk = cand;
+        // chunk-end work amortised) while the grid still has one and a half blocks per CU.  The sequence is
+        // cut into the fewest equal chunks (whole tiles) that give such a grid: a block walks every tile of
+        // its chunk, so chunks of a fixed length would leave the last one mostly empty (L = 520 as 512 + 8).
+        const uint32_t max_chunks = (a.L + tile - 1) / tile;
+        uint32_t nchunk = max_chunks, chunk = tile;
+        for (uint32_t n = 1; n <= max_chunks; ++n) {
+            const uint32_t len = ((a.L + n - 1) / n + tile - 1) / tile * tile;
+            if (len > (uint32_t)kBwdMaxChunk) continue;
+            const uint32_t used = (a.L + len - 1) / len;               // chunks of that length that hold steps
+            if (2ull * a.B * used * nct >= 256ull * kBwdHalfBlocksPerCU || n == max_chunks) {
+                nchunk = used;
+                chunk = len;
+                break;
+            }
         }
-        const uint32_t nchunk = (a.L + chunk - 1) / chunk;
         const uint64_t blocks = (uint64_t)a.B * nchunk * nct;
         if (blocks < (1ull << 31)) {
             plan->kind = BWD_BLC_VEC;

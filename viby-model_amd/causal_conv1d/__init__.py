@@ -534,15 +534,16 @@ def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv
 def _part_array(xs, outs):
     arr = (_lib.Part * len(xs))()
     for i, (x, o) in enumerate(zip(xs, outs)):
-        arr[i].x = x.data_ptr()
-        arr[i].out = o.data_ptr()
-        arr[i].channels = x.shape[1]
+        p = arr[i]
+        p.x = x.data_ptr()
+        p.out = o.data_ptr()
+        p.channels = x.shape[1]
         if x.dim() == 3:
-            arr[i].x_stride_b, arr[i].x_stride_c, arr[i].x_stride_l = x.stride()
-            arr[i].out_stride_b, arr[i].out_stride_c, arr[i].out_stride_l = o.stride()
+            p.x_stride_b, p.x_stride_c, p.x_stride_l = x.stride()
+            p.out_stride_b, p.out_stride_c, p.out_stride_l = o.stride()
         else:
-            arr[i].x_stride_b, arr[i].x_stride_c = x.stride()
-            arr[i].out_stride_b, arr[i].out_stride_c = o.stride()
+            p.x_stride_b, p.x_stride_c = x.stride()
+            p.out_stride_b, p.out_stride_c = o.stride()
     return arr
 
 

@@ -260,8 +260,8 @@ def test_whole_model_with_canon_layers_and_caches_traces_as_one_graph(cc):
 
 
 def test_compiled_training_through_the_multi_part_call(cc):
-    """Traced training graphs take the differentiable single-tensor operator on the concatenation: same dx bits
-    as the eager per-part backward, dweight equal up to the order of summation."""
+    """Traced training graphs differentiate through the multi-part operator (one fused backward per part on
+    its rows of the weights, as the eager path): same bits."""
     torch.manual_seed(9)
     B, L, dims = 2, 128, (64, 32)
     C = sum(dims)
@@ -282,6 +282,5 @@ def test_compiled_training_through_the_multi_part_call(cc):
 
     outs_e, dx_e, dw_e = step(f)
     outs_c, dx_c, dw_c = step(torch.compile(f, backend="aot_eager", fullgraph=True))
-    for a, e in zip(outs_c + dx_c, outs_e + dx_e):
+    for a, e in zip(outs_c + dx_c + [dw_c], outs_e + dx_e + [dw_e]):
         assert torch.equal(bits(a), bits(e))
-    torch.testing.assert_close(dw_c, dw_e, rtol=1e-5, atol=1e-5)

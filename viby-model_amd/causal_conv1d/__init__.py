@@ -601,16 +601,10 @@ def causal_conv1d_fn_parts(
     if _wants_grad(*xs, weight, bias) and initial_states is not None:
         raise NotImplementedError("gradients through a call with initial_states are not implemented")
     if torch.compiler.is_compiling():
-        if _wants_grad(*xs, weight, bias):
-            # traced training graphs: the differentiable single-tensor operator on the concatenation
-            y, fin = torch.ops.canon_conv1d.fwd(torch.cat(xs, dim=1), weight, bias, attention_mask, None, None,
-                                                final_states.shape[2] if final_states is not None else 0, act, res, rnd)
-            outs = tuple(y.split(dims, dim=1))
-        else:
-            *outs, fin = torch.ops.canon_conv1d.fwd_parts(xs, weight, bias, attention_mask, initial_states,
-                                                          final_states.shape[2] if final_states is not None else 0,
-                                                          act, res, rnd)
-            outs = tuple(outs)
+        *outs, fin = torch.ops.canon_conv1d.fwd_parts(xs, weight, bias, attention_mask, initial_states,
+                                                      final_states.shape[2] if final_states is not None else 0,
+                                                      act, res, rnd)
+        outs = tuple(outs)
         if final_states is not None:
             final_states.copy_(fin)
     elif _wants_grad(*xs, weight, bias):
@@ -815,6 +809,30 @@ def _op_fwd_parts(xs: List[torch.Tensor], weight: torch.Tensor, bias: Optional[t
 def _(xs, weight, bias, mask, initial_states, state_len, act, res, rnd):
     channels = sum(x.shape[1] for x in xs)
     return [torch.empty_like(x) for x in xs] + [xs[0].new_empty((xs[0].shape[0], channels, state_len))]
+
+
+def _op_fwd_parts_setup(ctx, inputs, output):
+    xs, weight, bias, mask, _initial, _state_len, act, res, _rnd = inputs
+    ctx.save_for_backward(weight, bias, mask, *xs)
+    ctx.flags = (act, res, bias is not None)
+
+
+def _op_fwd_parts_backward(ctx, grads):
+    # one fused backward per part, on that part's rows of the weights (no cat here either)
+    weight, bias, mask, *xs = ctx.saved_tensors
+    act, res, has_bias = ctx.flags
+    dxs, dws, dbs, c0 = [], [], [], 0
+    for x, dout in zip(xs, grads):
+        c1 = c0 + x.shape[1]
+        dx, dw, db = torch.ops.canon_conv1d.bwd(x, dout, weight[c0:c1], bias[c0:c1] if has_bias else None, mask, act, res)
+        dxs.append(dx)
+        dws.append(dw)
+        dbs.append(db)
+        c0 = c1
+    return dxs, torch.cat(dws, dim=0), (torch.cat(dbs, dim=0) if has_bias else None), None, None, None, None, None, None
+
+
+_op_fwd_parts.register_autograd(_op_fwd_parts_backward, setup_context=_op_fwd_parts_setup)
 
 
 @torch.library.custom_op("canon_conv1d::update_parts", mutates_args=("conv_state",), device_types="cuda")

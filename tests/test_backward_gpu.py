@@ -287,3 +287,42 @@ def test_backward_randomised(cc):
         check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
         if b is not None:
             check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
+def test_forward_and_backward_inside_a_captured_graph(cc):
+    """A training step's Canon part (forward, backward with its reduction, scratch from torch's allocator)
+    captured once as a device graph and replayed with new data between eager work: every replay must give
+    what the eager call gives on the same data."""
+    torch.manual_seed(31)
+    B, L, C = 4, 256, 264
+    x = torch.randn(B, L, C, device=DEV).bfloat16().requires_grad_()
+    w = (torch.randn(C, 4, device=DEV) * 0.3).requires_grad_()
+    b = (torch.randn(C, device=DEV) * 0.1).requires_grad_()
+    mask = right_padded_mask([256, 100, 31, 200], L).to(DEV)
+    dout = torch.randn(B, L, C, device=DEV).bfloat16()
+
+    def step():
+        y = cc.causal_conv1d_fn(x.transpose(1, 2), w, b, activation="silu", attention_mask=mask, residual=True)
+        gx, gw, gb = torch.autograd.grad(y, (x, w, b), dout.transpose(1, 2))
+        return y.detach(), gx, gw, gb
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture (library handles, allocator)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for i in range(4):
+        with torch.no_grad():                    # new data in the captured tensors, eager work in between
+            x.copy_(torch.randn(B, L, C, device=DEV).bfloat16())
+            dout.copy_(torch.randn(B, L, C, device=DEV).bfloat16())
+            w.mul_(1.01)
+        want = [t.clone() for t in step()]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, exp in zip(("y", "dx", "dweight", "dbias"), outs, want):
+            assert torch.equal(bits(got), bits(exp)), (i, name)

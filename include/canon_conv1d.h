@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 2
+#define CANON_CONV1D_ABI_VERSION 3
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -181,6 +181,9 @@ typedef struct canon_conv1d_update_params {
  *   dxm[t] = sum_k weight[k] * dz[t + (W-1) - k]  (+ dout[t] for RESIDUAL_MASKED)
  *   dx[t]  = dxm[t] * mask[t]                     (+ dout[t] for RESIDUAL_UNMASKED)
  *   dweight[c,k] = sum_{b,t} dz[b,c,t] * xm[b,c,t-(W-1)+k],   dbias[c] = sum_{b,t} dz[b,c,t]
+ * With seq_idx, the terms that pair an output step with a tap step of another
+ * sequence index (the ones the forward left out) are left out of z, dxm and
+ * dweight alike.
  * All arithmetic in fp32; dx is rounded once to the storage type.  dweight and
  * dbias are fp32, OVERWRITTEN (not accumulated into), and reduced in a fixed
  * order in two stages through `workspace` (no float atomics: results are
@@ -211,6 +214,8 @@ typedef struct canon_conv1d_bwd_params {
     float *dbias;                   /* [channels] fp32, or NULL */
     void *workspace;                /* canon_conv1d_bwd_workspace_bytes() bytes, 16-byte aligned */
     int64_t workspace_bytes;
+    const int32_t *seq_idx;         /* [batch, seqlen] or NULL: the forward's packed-sequence indices */
+    int64_t seq_stride_b, seq_stride_l;
 } canon_conv1d_bwd_params;
 
 /*

@@ -308,6 +308,12 @@ def test_bwd_plan_and_workspace():
     assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl"))) == b"bwd_bcl_vec"
     assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(layout="bcl", L=1023))) == b"bwd_generic"
     assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(C=3457))) == b"bwd_generic"
+    # packed sequences: only the walk kernel gates taps by sequence index
+    for layout in ("blc", "bcl"):
+        q = bwd_params(layout=layout, seq_idx=FAKE_X + 0x400000, seq_stride_b=1024, seq_stride_l=1)
+        assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == b"bwd_generic"
+    assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(seq_idx=FAKE_X + 2))) == -1
+    assert "seq_idx must be 4-byte aligned" in last_error()
     assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(width=9))) == -1
     assert "width 9" in last_error()
     assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(B=0))) == 0
@@ -406,9 +412,9 @@ def test_torch_operators_for_traced_graphs_have_shape_only_twins():
     assert y.shape == x.shape and y.stride() == x.stride() and y.dtype == x.dtype
     assert tuple(fin.shape) == (2, 16, 8) and fin.dtype == x.dtype
     assert tuple(ops.fwd(x, w, None, None, None, None, 0, 0, 0, 0)[1].shape) == (2, 16, 0)
-    dx, dw, db = ops.bwd(x, x, w, b, None, 0, 1)
+    dx, dw, db = ops.bwd(x, x, w, b, None, None, 0, 1)
     assert dx.stride() == x.stride() and tuple(dw.shape) == (16, 4) and dw.dtype == w.dtype and tuple(db.shape) == (16,)
-    assert tuple(ops.bwd(x, x, w, None, None, 0, 1)[2].shape) == (0,)
+    assert tuple(ops.bwd(x, x, w, None, None, None, 0, 1)[2].shape) == (0,)
     st = torch.empty(2, 16, 4, device="meta", dtype=torch.bfloat16)
     assert tuple(ops.update(x[:, :, 0], st, w, None, None, None, None, 0, 0, 0).shape) == (2, 16)
     outs = ops.fwd_parts([x[:, :12], x[:, 12:]], w, None, None, None, 3, 0, 0, 0)

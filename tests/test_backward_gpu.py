@@ -20,7 +20,7 @@ def cc():
     return causal_conv1d
 
 
-def gpu_grads(cc, x_cpu, w, b, dout_cpu, layout, mask=None, act=None, residual=False):
+def gpu_grads(cc, x_cpu, w, b, dout_cpu, layout, mask=None, act=None, residual=False, seq_idx=None):
     xg = x_cpu.to(DEV)
     dg = dout_cpu.to(DEV)
     if layout == "blc":
@@ -30,7 +30,8 @@ def gpu_grads(cc, x_cpu, w, b, dout_cpu, layout, mask=None, act=None, residual=F
     wg = w.to(DEV).requires_grad_(True)
     bg = b.to(DEV).requires_grad_(True) if b is not None else None
     out = cc.causal_conv1d_fn(xg, wg, bg, activation=act,
-                              attention_mask=None if mask is None else mask.to(DEV), residual=residual)
+                              attention_mask=None if mask is None else mask.to(DEV), residual=residual,
+                              seq_idx=None if seq_idx is None else seq_idx.to(DEV))
     out.backward(dg)
     torch.cuda.synchronize()
     return xg.grad, wg.grad, (bg.grad if bg is not None else None), out.detach()
@@ -287,6 +288,70 @@ def test_backward_randomised(cc):
         check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
         if b is not None:
             check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
+def packed_seq_idx(B, L, g, max_len):
+    """[B, L] int32: each row cut into consecutive sequences of random lengths 1..max_len, numbered from 0."""
+    q = torch.empty(B, L, dtype=torch.int32)
+    for b in range(B):
+        t, n = 0, 0
+        while t < L:
+            step = int(torch.randint(1, max_len + 1, (1,), generator=g))
+            q[b, t:t + step] = n
+            t, n = t + step, n + 1
+    return q
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["bcl", "blc"])
+def test_backward_of_packed_sequences(cc, dtype, layout):
+    """Gradients of a call with seq_idx: no term may cross a sequence boundary, in dx (through the dz of
+    later steps), in dweight or in the recomputed pre-activation.  Sequences shorter than the kernel
+    width, boundaries next to chunk ends and a padding mask on top are all in the draw."""
+    g = torch.Generator().manual_seed(4242)
+    for case, (B, C, L, W, max_len) in enumerate([(2, 24, 97, 4, 9), (1, 7, 160, 3, 40), (3, 64, 33, 2, 3),
+                                                  (2, 130, 515, 4, 64), (1, 8, 1, 4, 1), (2, 16, 1024, 4, 300)]):
+        for act, res in ((None, False), ("silu", "masked"), ("silu", "unmasked")):
+            x = torch.randn(B, C, L, generator=g).to(dtype)
+            w = (torch.randn(C, W, generator=g) * 0.5).to(dtype)
+            b = (torch.randn(C, generator=g) * 0.2).to(dtype) if case % 2 == 0 else None
+            dout = torch.randn(B, C, L, generator=g).to(dtype)
+            seq = packed_seq_idx(B, L, g, max_len)
+            mask = right_padded_mask([max(1, L - 5 * i) for i in range(B)], L) if case % 3 == 0 else None
+            dx, dw, db, out = gpu_grads(cc, x, w, b, dout, layout, mask, act, res, seq_idx=seq)
+            rdx, rdw, rdb, rout = conv1d_grads(x, w, b, dout, mask, act, res, seq_idx=seq)
+            what = f"case {case} {dtype} {layout} {B}x{C}x{L} W{W} {act} {res}"
+            check(out, rout, dtype, what + " out")
+            check(dx, rdx, dtype, what + " dx")
+            check(dw, rdw, dtype, what + " dweight", sum_terms=B * L)
+            if b is not None:
+                check(db, rdb, dtype, what + " dbias", sum_terms=B * L)
+
+
+def test_backward_of_packed_sequences_equals_the_sequences_on_their_own(cc):
+    """Oracle-free: the gradients of a packed row are those of its sequences run as separate calls
+    (dx cut out per sequence, dweight / dbias summed over them)."""
+    g = torch.Generator().manual_seed(99)
+    C, W = 48, 4
+    lengths = [5, 1, 2, 40, 3, 77]
+    L = sum(lengths)
+    x = torch.randn(1, C, L, generator=g)
+    w = torch.randn(C, W, generator=g) * 0.5
+    b = torch.randn(C, generator=g) * 0.2
+    dout = torch.randn(1, C, L, generator=g)
+    seq = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, n in enumerate(lengths)]).unsqueeze(0)
+    dx, dw, db, out = gpu_grads(cc, x, w, b, dout, "bcl", None, "silu", "unmasked", seq_idx=seq)
+    dw_sum, db_sum, t = torch.zeros(C, W, dtype=torch.float64), torch.zeros(C, dtype=torch.float64), 0
+    for n in lengths:
+        sdx, sdw, sdb, sout = gpu_grads(cc, x[:, :, t:t + n].contiguous(), w, b, dout[:, :, t:t + n].contiguous(),
+                                        "bcl", None, "silu", "unmasked")
+        torch.testing.assert_close(out[:, :, t:t + n], sout, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(dx[:, :, t:t + n], sdx, rtol=1e-5, atol=1e-6)
+        dw_sum += sdw.cpu().double()
+        db_sum += sdb.cpu().double()
+        t += n
+    torch.testing.assert_close(dw.cpu().double(), dw_sum, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(db.cpu().double(), db_sum, rtol=1e-4, atol=1e-5)
 
 
 def test_forward_and_backward_inside_a_captured_graph(cc):

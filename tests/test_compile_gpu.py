@@ -102,6 +102,30 @@ def test_compiled_training_step_has_the_eager_gradients(cc, backend):
             assert torch.equal(bits(a), bits(e)), name
 
 
+def test_compiled_training_step_over_packed_sequences(cc):
+    """seq_idx travels through the traced forward into the traced backward."""
+    torch.manual_seed(11)
+    B, L, C = 2, 96, 64
+    x0 = torch.randn(B, L, C, device=DEV)
+    w0 = torch.randn(C, 4, device=DEV) * 0.3
+    seq = torch.tensor([[0] * 10 + [1] * 2 + [2] * 84, [0] * 50 + [1] * 46], dtype=torch.int32, device=DEV)
+    dout = torch.randn(B, L, C, device=DEV)
+
+    def step(fn):
+        x, w = x0.clone().requires_grad_(), w0.clone().requires_grad_()
+        y = fn(x, w)
+        y.backward(dout)
+        return y.detach(), x.grad, w.grad
+
+    def f(x, w):
+        return cc.causal_conv1d_fn(x.transpose(1, 2), w, None, activation="silu", seq_idx=seq).transpose(1, 2)
+
+    want = step(f)
+    got = step(torch.compile(f, backend="aot_eager", fullgraph=True))
+    for name, a, e in zip(("y", "dx", "dweight"), got, want):
+        assert torch.equal(bits(a), bits(e)), name
+
+
 def test_decode_step_traces_and_updates_the_state_in_place(cc):
     torch.manual_seed(2)
     B, C, S = 8, 264, 4

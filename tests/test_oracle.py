@@ -418,6 +418,38 @@ def test_seq_idx_oracle_brute_force_and_separate_sequences():
         assert torch.equal(a.view(torch.int16), b_.view(torch.int16))
 
 
+def test_gradient_oracle_of_packed_sequences_is_pinned():
+    """The float64 gradient oracle with seq_idx: its forward equals the C oracle of the packed forward,
+    and its gradients equal those of every sequence differentiated on its own with the plain conv1d
+    formulation (dx cut out per sequence, dweight / dbias summed)."""
+    from oracle.canon_grad import conv1d_grads
+    g = torch.Generator().manual_seed(5)
+    B, C, L = 2, 5, 23
+    x = torch.randn(B, C, L, generator=g)
+    dout = torch.randn(B, C, L, generator=g)
+    mask = (torch.rand(B, L, generator=g) > 0.2).float()
+    seq = torch.tensor([[0] * 7 + [1] * 3 + [2] * 1 + [3] * 12, [0] * 23], dtype=torch.int32)
+    for W in (2, 3, 4):
+        w = torch.randn(C, W, generator=g)
+        b = torch.randn(C, generator=g)
+        for act, res in itertools.product((None, "silu"), (0, 1, 2)):
+            dx, dw, db, out = conv1d_grads(x, w, b, dout, mask, act, res, seq_idx=seq)
+            want = co.conv1d_fwd_seq(x, w, b, seq, mask, act, res)
+            torch.testing.assert_close(out.float(), want, rtol=1e-5, atol=1e-5)
+            dx2, dw2, db2 = torch.zeros_like(dx), torch.zeros_like(dw), torch.zeros_like(db)
+            for bi in range(B):
+                cuts = [0] + [t for t in range(1, L) if seq[bi, t] != seq[bi, t - 1]] + [L]
+                for s0, s1 in zip(cuts[:-1], cuts[1:]):
+                    a, aw, ab, _ = conv1d_grads(x[bi:bi + 1, :, s0:s1], w, b, dout[bi:bi + 1, :, s0:s1],
+                                                mask[bi:bi + 1, s0:s1], act, res)
+                    dx2[bi, :, s0:s1] = a[0]
+                    dw2 += aw
+                    db2 += ab
+            torch.testing.assert_close(dx, dx2, rtol=1e-12, atol=1e-12)
+            torch.testing.assert_close(dw, dw2, rtol=1e-12, atol=1e-12)
+            torch.testing.assert_close(db, db2, rtol=1e-12, atol=1e-12)
+
+
 def test_ring_buffer_and_state_pool_update_equal_the_shift_register():
     g = torch.Generator().manual_seed(83)
     for dtype, W, S in itertools.product([torch.float32, torch.bfloat16], [2, 3, 4], [3, 4, 7, 8]):

@@ -395,8 +395,6 @@ def test_errors_surface(cc):
         cc.causal_conv1d_fn(x, torch.randn(8, 5, device=DEV))
     with pytest.raises(ValueError, match="int32"):
         cc.causal_conv1d_fn(x, w, seq_idx=torch.zeros(2, 16, dtype=torch.int64, device=DEV))
-    with pytest.raises(NotImplementedError, match="seq_idx"):
-        cc.causal_conv1d_fn(x.clone().requires_grad_(), w, seq_idx=torch.zeros(2, 16, dtype=torch.int32, device=DEV))
     with pytest.raises(ValueError, match="shorter than width-1"):
         cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 2, device=DEV), w)
     with pytest.raises(NotImplementedError, match="backward"):

@@ -292,8 +292,6 @@ def causal_conv1d_fn(
                              f"({x.shape[0]}, {x.shape[2]})")
         if seq_idx.dtype != torch.int32 or seq_idx.device != x.device:
             raise ValueError("seq_idx must be an int32 tensor on the device of x")
-        if _wants_grad(x, weight, bias):
-            raise NotImplementedError("gradients of a call with seq_idx are not implemented")
     bias, attention_mask, final_states = _check_fwd_args(
         x, tuple(x.shape), weight, bias, attention_mask, initial_states, return_final_states, final_states_out)
 
@@ -315,7 +313,7 @@ def causal_conv1d_fn(
         final_states.copy_(fin)
         return result, final_states
     if _wants_grad(x, weight, bias):
-        result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd)
+        result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd, seq_idx)
     else:
         result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd, seq_idx)
         if final_states is not None:
@@ -344,9 +342,9 @@ class _CanonConvFn(torch.autograd.Function):
     (causal_conv1d_mps/autograd.py:13-160, 162-338)."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd):
-        out = _launch_fwd(x, weight, bias, mask, None, final_states, act, res, rnd)
-        ctx.save_for_backward(x, weight, bias, mask)
+    def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd, seq_idx=None):
+        out = _launch_fwd(x, weight, bias, mask, None, final_states, act, res, rnd, seq_idx)
+        ctx.save_for_backward(x, weight, bias, mask, seq_idx)
         ctx.flags = (act, res)
         if final_states is not None:
             ctx.mark_non_differentiable(final_states)
@@ -355,17 +353,17 @@ class _CanonConvFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
-        x, weight, bias, mask = ctx.saved_tensors
+        x, weight, bias, mask, seq_idx = ctx.saved_tensors
         act, res = ctx.flags
         channels, width = weight.shape
         dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
         dbias = torch.empty(channels, dtype=torch.float32, device=x.device) if bias is not None else None
-        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res)
+        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx)
         return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
-                None, None, None, None, None)
+                None, None, None, None, None, None)
 
 
-def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res) -> torch.Tensor:
+def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=None) -> torch.Tensor:
     """One backward launch (+ the fixed-order reduction): returns dx with x's strides and fills the
     fp32 ``dweight`` (channels, W) / ``dbias`` (channels,) given (rows of larger tensors are fine)."""
     if dout.dtype != x.dtype:
@@ -394,6 +392,9 @@ def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res) -> torch.
         p.mask = mask.data_ptr()
         p.mask_dtype = _lib.MASK_CODE[mask.dtype]
         p.mask_stride_b, p.mask_stride_l = mask.stride()
+    if seq_idx is not None:
+        p.seq_idx = seq_idx.data_ptr()
+        p.seq_stride_b, p.seq_stride_l = seq_idx.stride()
     p.dweight = dweight.data_ptr()
     p.dbias = dbias.data_ptr() if dbias is not None else None
     L = _lib.lib()
@@ -751,31 +752,32 @@ def _(x, weight, bias, mask, initial_states, seq_idx, state_len, act, res, rnd):
 
 @torch.library.custom_op("canon_conv1d::bwd", mutates_args=(), device_types="cuda")
 def _op_bwd(x: torch.Tensor, dout: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-            mask: Optional[torch.Tensor], act: int, res: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+            mask: Optional[torch.Tensor], seq_idx: Optional[torch.Tensor], act: int, res: int
+            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     channels, width = weight.shape
     dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
     dbias = torch.empty(channels if bias is not None else 0, dtype=torch.float32, device=x.device)
-    dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias if bias is not None else None, act, res)
+    dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias if bias is not None else None, act, res, seq_idx)
     return dx, dweight.to(weight.dtype), dbias.to(bias.dtype if bias is not None else weight.dtype)
 
 
 @_op_bwd.register_fake
-def _(x, dout, weight, bias, mask, act, res):
+def _(x, dout, weight, bias, mask, seq_idx, act, res):
     return (torch.empty_like(x), torch.empty_like(weight, memory_format=torch.contiguous_format),
             weight.new_empty((weight.shape[0] if bias is not None else 0,),
                              dtype=bias.dtype if bias is not None else weight.dtype))
 
 
 def _op_fwd_setup(ctx, inputs, output):
-    x, weight, bias, mask, _initial, _seq, _state_len, act, res, _rnd = inputs
-    ctx.save_for_backward(x, weight, bias, mask)
+    x, weight, bias, mask, _initial, seq_idx, _state_len, act, res, _rnd = inputs
+    ctx.save_for_backward(x, weight, bias, mask, seq_idx)
     ctx.flags = (act, res, bias is not None)
 
 
 def _op_fwd_backward(ctx, dout, _dstate):
-    x, weight, bias, mask = ctx.saved_tensors
+    x, weight, bias, mask, seq_idx = ctx.saved_tensors
     act, res, has_bias = ctx.flags
-    dx, dweight, dbias = torch.ops.canon_conv1d.bwd(x, dout, weight, bias, mask, act, res)
+    dx, dweight, dbias = torch.ops.canon_conv1d.bwd(x, dout, weight, bias, mask, seq_idx, act, res)
     return dx, dweight, (dbias if has_bias else None), None, None, None, None, None, None, None
 
 
@@ -824,7 +826,8 @@ def _op_fwd_parts_backward(ctx, grads):
     dxs, dws, dbs, c0 = [], [], [], 0
     for x, dout in zip(xs, grads):
         c1 = c0 + x.shape[1]
-        dx, dw, db = torch.ops.canon_conv1d.bwd(x, dout, weight[c0:c1], bias[c0:c1] if has_bias else None, mask, act, res)
+        dx, dw, db = torch.ops.canon_conv1d.bwd(x, dout, weight[c0:c1], bias[c0:c1] if has_bias else None,
+                                                mask, None, act, res)
         dxs.append(dx)
         dws.append(dw)
         dbs.append(db)

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -76,6 +76,7 @@ class BwdParams(ctypes.Structure):
         ("mask", _vp), ("mask_stride_b", _i64), ("mask_stride_l", _i64),
         ("dweight", _vp), ("dbias", _vp),
         ("workspace", _vp), ("workspace_bytes", _i64),
+        ("seq_idx", _vp), ("seq_stride_b", _i64), ("seq_stride_l", _i64),
     ]
 
 

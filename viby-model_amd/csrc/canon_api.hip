@@ -448,6 +448,8 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         return fail(CANON_ERR_UNSUPPORTED, "batch*channels and seqlen must each be below 2^31");
     if (p->mask && !valid_mask_dtype(p->mask_dtype))
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    if (p->seq_idx && ((uintptr_t)p->seq_idx & 3u))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx must be 4-byte aligned");
     const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
     if (check_pointers) {
         if (p->channels > 0 && (!p->weight || !p->dweight))
@@ -468,6 +470,7 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.d_sb = p->dx_stride_b; a.d_sc = p->dx_stride_c; a.d_sl = p->dx_stride_l;
     a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
     a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
+    a.seq = p->seq_idx; a.q_sb = p->seq_stride_b; a.q_sl = p->seq_stride_l;
     a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
     a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode;
@@ -482,7 +485,8 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
-    const bool rows = ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
+    const bool packed = p->seq_idx != nullptr;   // packed sequences: only the walk kernel gates taps by sequence index
+    const bool rows = !packed && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
                       a.d_sb % E == 0 && a.d_sc % E == 0;
     if (rows) {
@@ -518,7 +522,7 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     // channel-contiguous tensors: 8-byte groups of channels per lane
     const int E8 = 8 / elem_bytes(p->x_dtype);
     const bool ptrs8 = !check_pointers || ((((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0);
-    const bool vec = a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
+    const bool vec = !packed && a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
                      a.x_sb % E8 == 0 && a.x_sl % E8 == 0 && a.g_sb % E8 == 0 && a.g_sl % E8 == 0 &&
                      a.d_sb % E8 == 0 && a.d_sl % E8 == 0 && ptrs8;
     if (vec) {

@@ -17,6 +17,11 @@ namespace canon {
 // carried in registers), z[t] needs xm[t-3 .. t] (a sliding window refilled
 // with one row per step, fetched R rows ahead).  The three dz values just past
 // the chunk are recomputed from memory.
+//
+// SEQ (packed sequences): the sequence index of every row travels with it
+// (window, carried dz values, look-ahead).  A product of a tap with a row of
+// another sequence index is dropped wherever it appears: in z, in dx (the dz
+// of a later step of another sequence) and in dweight.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float silu_grad(float z)
 {
@@ -24,7 +29,7 @@ __device__ __forceinline__ float silu_grad(float z)
     return s * (1.0f + z * (1.0f - s));
 }
 
-template <int DT, int W, bool MASK, int R>
+template <int DT, int W, bool MASK, int R, bool SEQ>
 __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 {
     constexpr int BY = Elem<DT>::bytes;
@@ -65,6 +70,8 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
         g3[j][0] = load1<DT>(gb + (t > Lm1 ? Lm1 : t) * gs, 0);
     }
     if constexpr (MASK) load_mask_rows<7>(a.mask, (int64_t)b * a.m_sb, t_end - 4, a.L, a.m_sl, a.mask_dtype, m7);
+    int32_t q7[7] = {0, 0, 0, 0, 0, 0, 0};   // sequence indices of the same seven rows
+    if constexpr (SEQ) load_seq_rows<7>(a.seq, (int64_t)b * a.q_sb, t_end - 4, a.L, a.q_sl, q7);
 
     float w[E][W], bias[E];
     decode_taps<DT, W, E>(raw, a.w_dtype, false, a.bias != nullptr, w, bias);
@@ -88,7 +95,11 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
         for (int e = 0; e < E; ++e) {
             float z = bias[e];
 #pragma unroll
-            for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xr7[j + 1 + (4 - W) + k][e], z);   // xm[t_end+j-(W-1)+k]
+            for (int k = 0; k < W; ++k) {
+                const int row = j + 1 + (4 - W) + k;                                   // xm[t_end+j-(W-1)+k]
+                const float v = (!SEQ || q7[row] == q7[j + 4]) ? xr7[row][e] : 0.0f;
+                z = fmaf(w[e][k], v, z);
+            }
             const float d = a.act ? g3[j][e] * silu_grad(z) : g3[j][e];
             dzf[j][e] = inside ? d : 0.0f;
         }
@@ -99,6 +110,9 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     for (int k = 0; k < 4; ++k)
 #pragma unroll
         for (int e = 0; e < E; ++e) xw[k][e] = xr7[k][e];
+    // qw[k]: sequence index of xw[k]'s row; qf[j]: of dzf[j]'s step
+    int32_t qw[4] = {q7[0], q7[1], q7[2], q7[3]};
+    int32_t qf[3] = {q7[4], q7[5], q7[6]};
 
     float dw[E][W], dbs[E];
 #pragma unroll
@@ -113,6 +127,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
         // Rows are kept as loaded (raw) until their step, to keep the register count down.
         float G[R], XN[R];
         float mk[R], mn[R];
+        int32_t QN[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t t = t_hi - r;
@@ -120,6 +135,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
             const int64_t tn = t - 4 < 0 ? 0 : t - 4;
             G[r] = load1<DT>(gb + tg * gs, 0);
             XN[r] = load1<DT>(xb + tn * xs, 0);
+            QN[r] = SEQ ? a.seq[(int64_t)b * a.q_sb + tn * a.q_sl] : 0;
             mk[r] = 1.0f;
             mn[r] = 1.0f;
         }
@@ -140,11 +156,17 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
             float g[E], xn[E], dz[E], o[E];
             g[0] = G[r];
             xn[0] = XN[r];
+            // the window as this step sees it: rows of other sequences read as zero
+            float xs_[4][E];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int e = 0; e < E; ++e) xs_[k][e] = (!SEQ || qw[k] == qw[3]) ? xw[k][e] : 0.0f;
 #pragma unroll
             for (int e = 0; e < E; ++e) {
                 float z = bias[e];
 #pragma unroll
-                for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xw[(4 - W) + k][e], z);
+                for (int k = 0; k < W; ++k) z = fmaf(w[e][k], xs_[(4 - W) + k][e], z);
                 dz[e] = z;
             }
             if (a.act) {
@@ -158,12 +180,12 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
             for (int e = 0; e < E; ++e) {
                 // dxm[t] = sum_k w[k] * dz[t + (W-1) - k]
                 float acc = w[e][W - 1] * dz[e];
-                acc = fmaf(w[e][W - 2], dzf[0][e], acc);
-                if constexpr (W >= 3) acc = fmaf(w[e][W - 3], dzf[1][e], acc);
-                if constexpr (W == 4) acc = fmaf(w[e][0], dzf[2][e], acc);
+                acc = fmaf(w[e][W - 2], (!SEQ || qf[0] == qw[3]) ? dzf[0][e] : 0.0f, acc);
+                if constexpr (W >= 3) acc = fmaf(w[e][W - 3], (!SEQ || qf[1] == qw[3]) ? dzf[1][e] : 0.0f, acc);
+                if constexpr (W == 4) acc = fmaf(w[e][0], (!SEQ || qf[2] == qw[3]) ? dzf[2][e] : 0.0f, acc);
                 o[e] = acc;
 #pragma unroll
-                for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xw[(4 - W) + k][e], dw[e][k]);
+                for (int k = 0; k < W; ++k) dw[e][k] = fmaf(dz[e], xs_[(4 - W) + k][e], dw[e][k]);
                 dbs[e] += dz[e];
                 dzf[2][e] = dzf[1][e];
                 dzf[1][e] = dzf[0][e];
@@ -191,6 +213,10 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
                 xw[2][e] = xw[1][e];
                 xw[1][e] = xw[0][e];
                 xw[0][e] = has_row ? v : 0.0f;
+            }
+            if constexpr (SEQ) {
+                qf[2] = qf[1]; qf[1] = qf[0]; qf[0] = qw[3];
+                qw[3] = qw[2]; qw[2] = qw[1]; qw[1] = qw[0]; qw[0] = QN[r];
             }
             store1<DT>(db_ + t * ds, 0, o[0]);
         }
@@ -922,8 +948,10 @@ template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStre
         if (pl.args.act) hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, true>), g, b, 0, s, pl.args);
         else hipLaunchKernelGGL((canon_bwd_blc_kernel<DT, W, MASK, false>), g, b, 0, s, pl.args);
     }
+    else if (pl.args.seq)
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, MASK, kBwdRows, true>), g, b, 0, s, pl.args);
     else
-        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, MASK, kBwdRows>), g, b, 0, s, pl.args);
+        hipLaunchKernelGGL((canon_bwd_walk_kernel<DT, W, MASK, kBwdRows, false>), g, b, 0, s, pl.args);
 }
 
 template <int DT> void launch_bwd(const BwdPlan &pl, hipStream_t s)

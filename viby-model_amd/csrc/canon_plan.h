@@ -110,6 +110,8 @@ struct BwdArgs {
     float *partial;
     float *dweight;
     float *dbias;
+    const int32_t *seq;   // packed-sequence indices [B, L] or nullptr (walk kernel only)
+    int64_t q_sb, q_sl;
     int64_t x_sb, x_sc, x_sl;
     int64_t g_sb, g_sc, g_sl;
     int64_t d_sb, d_sc, d_sl;

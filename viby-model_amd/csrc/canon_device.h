@@ -259,6 +259,22 @@ __device__ __forceinline__ void load_mask_rows(const void *p, int64_t row_base, 
     load_mask_entries<N, false>(p, 0, idx, dt, m);
 }
 
+// N (<= 64) mask entries of consecutive time steps t_first .. t_first+N-1 (clamped to [0, L-1]) of one batch
+// row, the same for every lane of the wave: lane j fetches entry j with one vector load, the values are then
+// broadcast lane by lane.  Against one scalar load per entry this keeps eleven 64-bit addresses out of the
+// scalar registers (the channel-contiguous kernel ran out of them and spilled) and puts the mask in the same
+// in-order queue as the rows.
+template <int N>
+__device__ __forceinline__ void load_mask_rows_wave(const void *p, int64_t row_base, int64_t t_first, int64_t L,
+                                                    int64_t stride, int dt, int lane, float *m)
+{
+    int64_t t = t_first + (lane < N ? lane : N - 1);
+    t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+    const float v = load_mask(p, row_base + t * stride, dt);
+#pragma unroll
+    for (int j = 0; j < N; ++j) m[j] = bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
+}
+
 // A lane's access unit in the channel-contiguous kernels: 16 bytes, or 8 bytes (half the registers
 // per lane, twice the waves in flight)
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));

@@ -468,7 +468,7 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
         if constexpr (MASK) {
             // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
             float mm[R + 3];
-            load_mask_rows<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, mm);
+            load_mask_rows_wave<R + 3>(a.mask, (int64_t)b * a.m_sb, t0 - 3, a.L, a.m_sl, a.mask_dtype, lane, mm);
 #pragma unroll
             for (int j = 0; j < 3; ++j) mh[j] = mm[j];
 #pragma unroll

@@ -275,6 +275,18 @@ __device__ __forceinline__ void load_mask_rows_wave(const void *p, int64_t row_b
     for (int j = 0; j < N; ++j) m[j] = bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
 }
 
+// The same for N sequence indices.
+template <int N>
+__device__ __forceinline__ void load_seq_rows_wave(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L,
+                                                   int64_t stride, int lane, int32_t *q)
+{
+    int64_t t = t_first + (lane < N ? lane : N - 1);
+    t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+    const int32_t v = p[row_base + t * stride];
+#pragma unroll
+    for (int j = 0; j < N; ++j) q[j] = __builtin_amdgcn_readlane(v, j);
+}
+
 // A lane's access unit in the channel-contiguous kernels: 16 bytes, or 8 bytes (half the registers
 // per lane, twice the waves in flight)
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));

@@ -464,7 +464,7 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
         // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
         if constexpr (MODE == TAPS_ANY)
             fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
-        if constexpr (SEQ) load_seq_rows<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, sq);
+        if constexpr (SEQ) load_seq_rows_wave<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, lane, sq);
         if constexpr (MASK) {
             // mask of the three rows before the slab and of the slab, last so that nothing is issued after its wait
             float mm[R + 3];

@@ -533,13 +533,25 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         // chunk-end work amortised) while the grid still has one and a half blocks per CU.  The sequence is
         // cut into the fewest equal chunks (whole tiles) that give such a grid: a block walks every tile of
         // its chunk, so chunks of a fixed length would leave the last one mostly empty (L = 520 as 512 + 8).
-        const uint32_t max_chunks = (a.L + tile - 1) / tile;
+        const uint32_t max_chunks = (a.L + tile - 1) / tile;   // = tiles per sequence
         uint32_t nchunk = max_chunks, chunk = tile;
+        bool found = false;
         for (uint32_t n = 1; n <= max_chunks; ++n) {
             const uint32_t len = ((a.L + n - 1) / n + tile - 1) / tile * tile;
             if (len > (uint32_t)kBwdMaxChunk) continue;
             const uint32_t used = (a.L + len - 1) / len;               // chunks of that length that hold steps
-            if (2ull * a.B * used * nct >= 256ull * kBwdHalfBlocksPerCU || n == max_chunks) {
+            const bool enough = 2ull * a.B * used * nct >= 256ull * kBwdHalfBlocksPerCU || n == max_chunks;
+            if (!found && enough) {
+                found = true;
+                nchunk = used;
+                chunk = len;
+                if (max_chunks % used == 0) break;
+                continue;
+            }
+            // the first count that is enough leaves a short last chunk: a slightly larger count that cuts the
+            // tiles evenly runs 5-10 % faster (B4 L1024: 8 chunks of 4 tiles 24.9 us, 7 of 5 tiles 27.1 us)
+            if (found && (n >= 2 * nchunk || len < 2 * tile)) break;
+            if (found && used == n && max_chunks % n == 0) {
                 nchunk = used;
                 chunk = len;
                 break;

@@ -7,6 +7,7 @@
  *   canon_conv1d_fwd     replaces  causal_conv1d_fn      (prefill)
  *   canon_conv1d_update  replaces  causal_conv1d_update  (one decode token)
  *   canon_conv1d_bwd     gradient of canon_conv1d_fwd    (training)
+ *   canon_conv1d_update_bwd  gradient of canon_conv1d_update
  *
  * Plain pointers, sizes and element strides only; no framework types.  Every
  * pointer is a DEVICE pointer owned by the caller.  Kernels are enqueued on
@@ -25,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 3
+#define CANON_CONV1D_ABI_VERSION 4
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -220,6 +221,61 @@ typedef struct canon_conv1d_bwd_params {
 } canon_conv1d_bwd_params;
 
 /*
+ * Backward of canon_conv1d_update (shift-register mode).  Same role as the
+ * reference's short_conv_update_bwd (causal_conv1d_mps/autograd.py:465-498,
+ * causal_conv1d.metal:1738-1850): dx, dconv_state, dweight, dbias from the
+ * token, the state AS IT WAS BEFORE the forward call (the caller keeps a
+ * copy, as causal_conv1d_mps/autograd.py:452 does: the forward overwrites
+ * it) and dout.  Unlike the reference it also takes the gradient that
+ * arrives through the UPDATED state, so that a chain of decode steps can be
+ * differentiated end to end.
+ *
+ * With xt = x * token_mask, z = bias + sum_{k<W-1} weight[k] * state[S-(W-1)+k] + weight[W-1] * xt,
+ * out = act(z) (+ xt | + x), state' = state[1:] ++ xt:
+ *   dz        = dout * act'(z)
+ *   dxt       = weight[W-1] * dz (+ dout for RESIDUAL_MASKED) + dstate_out[S-1]
+ *   dx        = dxt * token_mask (+ dout for RESIDUAL_UNMASKED)
+ *   dstate[j] = dstate_out[j-1]  (0 for j = 0)  + weight[j-(S-(W-1))] * dz  for j >= S-(W-1)
+ *   dweight[c,k] = sum_b dz[b,c] * (k < W-1 ? state[b,c,S-(W-1)+k] : xt[b,c]),   dbias[c] = sum_b dz[b,c]
+ * All arithmetic in fp32, dx and dstate rounded once to the storage type;
+ * dweight / dbias fp32, overwritten, summed over the batch in a fixed order in
+ * two stages through `workspace` (no float atomics).
+ */
+typedef struct canon_conv1d_update_bwd_params {
+    uint32_t struct_size;           /* sizeof(canon_conv1d_update_bwd_params) */
+    int32_t x_dtype;                /* x, conv_state, dout, dstate_out, dx, dstate */
+    int32_t w_dtype;                /* weight and bias as used by the forward */
+    int32_t mask_dtype;
+    int32_t width;
+    int32_t activation;
+    int32_t residual_mode;
+    int32_t state_len;
+    int64_t batch, channels;
+    const void *x;                  /* [batch, channels]: the token of the forward call */
+    int64_t x_stride_b, x_stride_c;
+    const void *conv_state;         /* [batch, channels, state_len]: the state BEFORE the forward call */
+    int64_t state_stride_b, state_stride_c, state_stride_s;
+    const void *weight;
+    int64_t w_stride_c, w_stride_k;
+    const void *bias;               /* or NULL */
+    const void *token_mask;         /* [batch], or NULL */
+    int64_t mask_stride_b;
+    const void *dout;               /* [batch, channels] */
+    int64_t dout_stride_b, dout_stride_c;
+    const void *dstate_out;         /* [batch, channels, state_len]: gradient w.r.t. the updated state, or NULL (zero) */
+    int64_t dstate_out_stride_b, dstate_out_stride_c, dstate_out_stride_s;
+    void *dx;                       /* [batch, channels] */
+    int64_t dx_stride_b, dx_stride_c;
+    void *dstate;                   /* [batch, channels, state_len]: gradient w.r.t. the state before, or NULL (not wanted);
+                                       must not alias dstate_out */
+    int64_t dstate_stride_b, dstate_stride_c, dstate_stride_s;
+    float *dweight;                 /* [channels, width] contiguous fp32, or NULL (no parameter gradients) */
+    float *dbias;                   /* [channels] fp32, or NULL; needs dweight */
+    void *workspace;                /* canon_conv1d_update_bwd_workspace_bytes() bytes, 16-byte aligned (unused when dweight == NULL) */
+    int64_t workspace_bytes;
+} canon_conv1d_update_bwd_params;
+
+/*
  * One channel range of a logical [batch, channels, seqlen] input that lives in
  * a tensor of its own.  Canon-B convolves cat(q, k, v) and Canon-D
  * cat(gate, up) along the channels (model/model.py:772-789, 962-971): with
@@ -246,6 +302,7 @@ const char *canon_conv1d_last_error(void);
 int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream);
 int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
 int canon_conv1d_bwd(const canon_conv1d_bwd_params *p, void *stream);
+int canon_conv1d_update_bwd(const canon_conv1d_update_bwd_params *p, void *stream);
 
 /*
  * The same operators with x / out given as 1..CANON_CONV1D_MAX_PARTS channel
@@ -262,6 +319,7 @@ int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_c
 /* Scratch bytes canon_conv1d_bwd needs for these sizes and strides (the
  * pointers in *p are not read); negative if the arguments are rejected. */
 int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
+int64_t canon_conv1d_update_bwd_workspace_bytes(const canon_conv1d_update_bwd_params *p);
 
 /*
  * Name of the kernel family the call above would launch for these arguments

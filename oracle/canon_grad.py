@@ -15,6 +15,16 @@ convolution is written as a sum of shifted, gated copies of ``xm``.  That
 form is pinned by the tests in two ways: its output against the C oracle of
 the packed forward, and its gradients against this same function run without
 ``seq_idx`` on every sequence cut out on its own.
+
+``update_grads`` does the same for one decode step in the formulation of
+the eager module's step (model/model.py:372-398): the window is the last
+W-1 state slots and the token, ``out = act(bias + sum_k w[k] * window[k])``
+plus the residual, and the new state is the old one shifted left by one with
+the token appended.  The loss whose gradient it returns is
+``sum(out * dout) + sum(new_state * dstate_out)``, so it covers the gradient
+that reaches a step through the state it hands to the next one.  Pinned by
+the tests through the prefill: a chain of such steps has the gradients of
+``conv1d_grads`` on the same tokens laid out along time.
 """
 from __future__ import annotations
 
@@ -54,3 +64,32 @@ def conv1d_grads(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
         y = y + x64
     y.backward(dout.detach().cpu().double())
     return x64.grad, w64.grad, (b64.grad if b64 is not None else None), y.detach()
+
+
+def update_grads(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                 dout: torch.Tensor, dstate_out: Optional[torch.Tensor] = None, token_mask: Optional[torch.Tensor] = None,
+                 activation=None, residual=0):
+    """x, dout [B, C]; conv_state, dstate_out [B, C, S] (the state BEFORE the step); weight [C, W] and
+    bias [C] are first rounded to x.dtype.  Returns (dx, dstate, dweight, dbias, out, new_state) in float64."""
+    C, W = weight.shape
+    x64 = x.detach().cpu().double().requires_grad_(True)
+    s64 = conv_state.detach().cpu().double().requires_grad_(True)
+    w64 = weight.detach().cpu().to(x.dtype).double().requires_grad_(True)
+    b64 = bias.detach().cpu().to(x.dtype).double().requires_grad_(True) if bias is not None else None
+    xt = x64 if token_mask is None else x64 * token_mask.detach().cpu().double().unsqueeze(1)
+    window = torch.cat([s64[:, :, s64.shape[2] - (W - 1):], xt.unsqueeze(-1)], dim=-1)      # [B, C, W]
+    z = (window * w64.unsqueeze(0)).sum(-1)
+    if b64 is not None:
+        z = z + b64
+    y = F.silu(z) if activation in ("silu", "swish", True, 1) else z
+    if residual in (True, 1, "masked"):
+        y = y + xt
+    elif residual in (2, "unmasked"):
+        y = y + x64
+    new_state = torch.cat([s64[:, :, 1:], xt.unsqueeze(-1)], dim=-1)
+    loss = (y * dout.detach().cpu().double()).sum()
+    if dstate_out is not None:
+        loss = loss + (new_state * dstate_out.detach().cpu().double()).sum()
+    loss.backward()
+    return (x64.grad, s64.grad if s64.grad is not None else torch.zeros_like(s64), w64.grad,
+            b64.grad if b64 is not None else None, y.detach(), new_state.detach())

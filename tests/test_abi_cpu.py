@@ -22,7 +22,7 @@ HEADER = os.path.join(ROOT, "include", "canon_conv1d.h")
 
 import causal_conv1d as cc                      # noqa: E402
 from causal_conv1d import _lib                  # noqa: E402
-from causal_conv1d._lib import BwdParams, FwdParams, Part, UpdateParams  # noqa: E402
+from causal_conv1d._lib import BwdParams, FwdParams, Part, UpdateBwdParams, UpdateParams  # noqa: E402
 
 
 def test_library_exports_every_declared_function():
@@ -40,7 +40,8 @@ def test_library_exports_every_declared_function():
 def test_ctypes_structs_match_the_header(tmp_path):
     lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){']
     structs = (("canon_conv1d_fwd_params", FwdParams), ("canon_conv1d_update_params", UpdateParams),
-               ("canon_conv1d_bwd_params", BwdParams), ("canon_conv1d_part", Part))
+               ("canon_conv1d_bwd_params", BwdParams), ("canon_conv1d_update_bwd_params", UpdateBwdParams),
+               ("canon_conv1d_part", Part))
     for cname, cls in structs:
         lines.append(f'printf("{cname} size %zu\\n", sizeof({cname}));')
         for fname, _ in cls._fields_:
@@ -322,6 +323,46 @@ def test_bwd_plan_and_workspace():
     assert "workspace" in last_error()
     assert L.canon_conv1d_bwd(ctypes.byref(bwd_params(dx=FAKE_X)), None) == _lib.ERR_INVALID_ARGUMENT
     assert "alias" in last_error()
+
+
+def update_bwd_params(B=256, C=3456, S=3, dtype=1, **over):
+    p = UpdateBwdParams()
+    p.struct_size = ctypes.sizeof(UpdateBwdParams)
+    p.x_dtype = p.w_dtype = dtype
+    p.width, p.state_len = 4, S
+    p.batch, p.channels = B, C
+    p.x, p.dout, p.dx, p.weight, p.conv_state = FAKE_X, FAKE_OUT, FAKE_OUT + 0x4000000, FAKE_W, FAKE_STATE
+    p.dweight, p.workspace, p.workspace_bytes = FAKE_W + 0x100000, FAKE_W + 0x200000, 1 << 30
+    for name in ("x", "dout", "dx"):
+        setattr(p, f"{name}_stride_b", C)
+        setattr(p, f"{name}_stride_c", 1)
+    for name in ("state", "dstate_out", "dstate"):
+        for s, v in zip(("b", "c", "s"), (C * S, S, 1)):
+            setattr(p, f"{name}_stride_{s}", v)
+    p.w_stride_c, p.w_stride_k = 4, 1
+    for k, v in over.items():
+        setattr(p, k, v)
+    return p
+
+
+def test_update_bwd_validation_and_workspace():
+    L = _lib.lib()
+    ws = L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(update_bwd_params()))
+    assert 0 < ws <= 8 << 20 and ws % (3456 * 5 * 4) == 0          # whole partial sets, one per batch group
+    assert L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(update_bwd_params(dweight=0))) == 0
+    assert L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(update_bwd_params(B=0))) == 0
+    assert L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(update_bwd_params(B=1, C=8))) == 8 * 5 * 4
+    for over, msg in [(dict(width=5), "width 5"), (dict(S=2), "shorter than width-1"), (dict(struct_size=4), "struct_size"),
+                      (dict(x_dtype=7), "x_dtype 7"), (dict(activation=3), "activation 3"),
+                      (dict(dweight=0, dbias=FAKE_W), "dbias needs dweight"),
+                      (dict(token_mask=FAKE_X, mask_dtype=9), "mask_dtype 9")]:
+        assert L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(update_bwd_params(**over))) == -1, over
+        assert msg in last_error(), (over, last_error())
+    # what only the launching call can check: pointers and the scratch
+    for over, msg in [(dict(dout=0), "NULL"), (dict(workspace=0), "workspace"), (dict(workspace_bytes=16), "workspace"),
+                      (dict(dstate=FAKE_X, dstate_out=FAKE_X), "alias")]:
+        assert L.canon_conv1d_update_bwd(ctypes.byref(update_bwd_params(**over)), None) == _lib.ERR_INVALID_ARGUMENT, over
+        assert msg in last_error(), (over, last_error())
 
 
 def make_parts(dims, B=8, L=1024, layout="blc", elem=2, row=None):

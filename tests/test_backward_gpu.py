@@ -225,7 +225,7 @@ def test_unsupported_gradients_raise(cc):
     with pytest.raises(NotImplementedError, match="initial_states"):
         cc.causal_conv1d_fn(x, w, initial_states=torch.zeros(2, 8, 3, device=DEV))
     with pytest.raises(NotImplementedError, match="backward of the decode step"):
-        cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 4, device=DEV), w)
+        cc.causal_conv1d_update_parts([x[:, :4, 0], x[:, 4:, 0]], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
     assert out.requires_grad and not fs.requires_grad
 

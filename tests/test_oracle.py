@@ -479,3 +479,34 @@ def test_ring_buffer_and_state_pool_update_equal_the_shift_register():
             assert torch.equal(pool[rows_of.long()], shift)
         others = [r for r in range(rows) if r not in rows_of.tolist()]
         assert torch.equal(pool[others], untouched[others])
+
+
+def test_update_gradient_oracle_chained_equals_the_prefill_gradient_oracle():
+    """oracle/canon_grad.update_grads, chained backwards through the state it hands on, must give the
+    gradients of conv1d_grads (torch autograd through F.conv1d) on the same tokens laid out along time;
+    a wrong slot, a dropped state term or a missing residual fails this."""
+    from oracle.canon_grad import conv1d_grads, update_grads
+    torch.manual_seed(0)
+    for (S, W), act, res, masked in itertools.product([(4, 4), (3, 4), (8, 4), (5, 3), (1, 2)], [None, "silu"],
+                                                      [0, 1, 2], [False, True]):
+        B, C, T = 2, 5, 6
+        x, w, b = torch.randn(B, C, T).double(), torch.randn(C, W).double(), torch.randn(C).double()
+        dout = torch.randn(B, C, T).double()
+        mask = (torch.rand(B, T) > 0.3).double() if masked else None
+        dx_ref, dw_ref, db_ref, out_ref = conv1d_grads(x, w, b, dout, mask=mask, activation=act, residual=res)
+        states = [torch.zeros(B, C, S, dtype=torch.float64)]
+        for t in range(T):
+            r = update_grads(x[:, :, t], states[-1], w, b, dout[:, :, t], None, None if mask is None else mask[:, t],
+                             act, res)
+            assert torch.allclose(r[4], out_ref[:, :, t], atol=1e-12)
+            states.append(r[5])
+        ds, dw, db = None, torch.zeros_like(w), torch.zeros_like(b)
+        dx = torch.zeros_like(x)
+        for t in reversed(range(T)):
+            r = update_grads(x[:, :, t], states[t], w, b, dout[:, :, t], ds, None if mask is None else mask[:, t],
+                             act, res)
+            dx[:, :, t], ds = r[0], r[1]
+            dw += r[2]
+            db += r[3]
+        for got, want in ((dx, dx_ref), (dw, dw_ref), (db, db_ref)):
+            assert torch.allclose(got, want, atol=1e-11), (S, W, act, res, masked)

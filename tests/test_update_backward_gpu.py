@@ -1,0 +1,195 @@
+"""Backward of the decode step (dx, dconv_state, dweight, dbias) against torch autograd of the eager
+step formulation (oracle/canon_grad.py, float64), by finite differences as the reference's own test
+does (causal-conv1d-mps/test.py:294-321), and as a chain of steps against the backward of the prefill."""
+import itertools
+
+import pytest
+import torch
+
+from oracle.canon_grad import conv1d_grads, update_grads
+from test_backward_gpu import check
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def cc():
+    import causal_conv1d
+    return causal_conv1d
+
+
+def quantised(shape, dtype, scale=1.0):
+    return (torch.randn(*shape) * scale).to(dtype)
+
+
+def run_step(cc, x, state, w, b, dout, dstate_out, mask, act, residual):
+    """One differentiable step on the GPU; the loss also reads the updated state when dstate_out is given."""
+    xg = x.to(DEV).requires_grad_(True)
+    s0 = state.to(DEV).requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True) if b is not None else None
+    s = s0.clone()                      # the in-place update needs a non-leaf tensor
+    out = cc.causal_conv1d_update(xg, s, wg, bg, activation=act, residual=residual,
+                                  token_mask=None if mask is None else mask.to(DEV))
+    loss = (out.float() * dout.to(DEV).float()).sum()
+    if dstate_out is not None:
+        loss = loss + (s.float() * dstate_out.to(DEV).float()).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    return xg.grad, s0.grad, wg.grad, (bg.grad if bg is not None else None), out.detach(), s.detach()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("S,W", [(3, 4), (4, 4), (8, 4), (2, 3), (5, 2)])
+def test_update_backward_matches_autograd_of_the_eager_step(cc, dtype, S, W):
+    torch.manual_seed(S * 10 + W)
+    B, C = 5, 200
+    for act, residual, use_mask, use_bias, through_state in itertools.product(
+            [None, "silu"], [False, True, "unmasked"], [False, True], [True, False], [False, True]):
+        if use_mask != (residual is not False) and act is None:
+            continue                                   # thin the grid: 28 of the 48 combinations per shape
+        x, st = quantised((B, C), dtype), quantised((B, C, S), dtype)
+        w, b = quantised((C, W), dtype, 0.5), quantised((C,), dtype, 0.1) if use_bias else None
+        dout = quantised((B, C), dtype)
+        dso = quantised((B, C, S), dtype) if through_state else None
+        mask = torch.tensor([1, 0, 1, 1, 0], dtype=torch.int64) if use_mask else None
+        got = run_step(cc, x, st, w, b, dout, dso, mask, act, residual)
+        want = update_grads(x, st, w, b, dout, dso, mask, act, residual)
+        tag = f"{dtype} S{S} W{W} act={act} res={residual} mask={use_mask} bias={use_bias} state={through_state}"
+        check(got[0], want[0], dtype, "dx " + tag)
+        check(got[1], want[1], dtype, "dstate " + tag)
+        check(got[2], want[2], dtype, "dweight " + tag, sum_terms=B)
+        if use_bias:
+            check(got[3], want[3], dtype, "dbias " + tag, sum_terms=B)
+        # the state handed on is bit-exactly the shifted state with the (masked) token appended
+        assert torch.equal(got[5].cpu().double(), want[5]), "state " + tag
+
+
+def test_update_backward_finite_differences_like_the_reference_test(cc):
+    """causal-conv1d-mps/test.py:294-321: batch 2, dim 8, width 4, state_len 8, SiLU, residual; eps 1e-3,
+    atol 1e-3, rtol 1e-2, loss = out.sum() (test.py:8-80).  The state gradient is checked as well."""
+    torch.manual_seed(0)
+    B, C, W, S = 2, 8, 4, 8
+    x = torch.randn(B, C, device=DEV, requires_grad=True)
+    state = torch.randn(B, C, S, device=DEV, requires_grad=True)
+    w = torch.randn(C, W, device=DEV, requires_grad=True)
+    b = torch.randn(C, device=DEV, requires_grad=True)
+    params = [x, state, w, b]
+
+    def f():
+        return cc.causal_conv1d_update(x, state.clone(), w, b, activation="silu", residual=True)
+
+    f().sum().backward()
+    analytic = [p.grad.clone() for p in params]
+    eps = 1e-3
+    with torch.no_grad():
+        for p, a in zip(params, analytic):
+            num = torch.zeros_like(p)
+            for i in itertools.product(*[range(s) for s in p.shape]):
+                old = p[i].item()
+                p[i] = old + eps
+                lp = f().double().sum().item()
+                p[i] = old - eps
+                lm = f().double().sum().item()
+                p[i] = old
+                num[i] = (lp - lm) / (2 * eps)
+            assert torch.allclose(a, num, atol=1e-3, rtol=1e-2), (tuple(p.shape), (a - num).abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chain_of_steps_has_the_gradients_of_the_prefill(cc, dtype):
+    """T decode steps from a zero state, differentiated end to end through the carried state, against the
+    float64 gradient of the prefill over the same tokens, and against this library's own prefill backward."""
+    torch.manual_seed(3)
+    B, C, T, S, W = 3, 264, 7, 4, 4
+    x, w, b = quantised((B, C, T), dtype), quantised((C, W), dtype, 0.5), quantised((C,), dtype, 0.1)
+    dout = quantised((B, C, T), dtype)
+    xg = x.to(DEV).requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True)
+    state = torch.zeros(B, C, S, dtype=dtype, device=DEV)
+    outs = []
+    for t in range(T):
+        outs.append(cc.causal_conv1d_update(xg[:, :, t], state, wg, bg, activation="silu", residual=True))
+    out = torch.stack(outs, dim=-1)
+    out.backward(dout.to(DEV))
+    torch.cuda.synchronize()
+    want = conv1d_grads(x, w, b, dout, activation="silu", residual=1)
+    if dtype == torch.float32:
+        check(xg.grad, want[0], dtype, "dx chain")
+    else:
+        # every step rounds the gradient it hands back through the state to the storage type (up to three
+        # roundings on the way to a token): three ulps of the tensor's scale
+        scale = want[0].abs().max().item()
+        assert (xg.grad.cpu().double() - want[0]).abs().max().item() <= 3 * 2.0 ** -8 * scale
+    if dtype == torch.float32:
+        check(wg.grad, want[1], dtype, "dweight chain", sum_terms=B * T)
+        check(bg.grad, want[2], dtype, "dbias chain", sum_terms=B * T)
+    else:
+        # autograd adds the T per-step parameter gradients in the parameters' 16-bit type: T roundings
+        for got, ref in ((wg.grad, want[1]), (bg.grad, want[2])):
+            assert (got.cpu().double() - ref).abs().max().item() <= T * 2.0 ** -8 * scale_of(ref)
+    assert torch.equal(state[:, :, 1:].cpu(), x[:, :, T - 3:])       # and the state is the last tokens, bit for bit
+    if dtype == torch.float32:
+        x2 = x.to(DEV).requires_grad_(True)
+        w2 = w.to(DEV).requires_grad_(True)
+        cc.causal_conv1d_fn(x2, w2, b.to(DEV), activation="silu", residual=True).backward(dout.to(DEV))
+        assert (x2.grad - xg.grad).abs().max().item() <= 2e-5 * scale_of(x2.grad)
+        assert (w2.grad - wg.grad).abs().max().item() <= 1e-4 * scale_of(w2.grad)
+
+
+def scale_of(t):
+    return t.abs().max().item() + 1e-30
+
+
+def test_update_backward_at_decode_shape_is_deterministic(cc):
+    """B 256, C 3456, S 3 bf16 (the decode configuration): same bits on every run (fixed-order reduction,
+    no float atomics), gradients within the bar of the float64 oracle; strided token and dout."""
+    torch.manual_seed(5)
+    B, C, S, W = 256, 3456, 3, 4
+    dtype = torch.bfloat16
+    x3 = quantised((B, C, 1), dtype)                       # the (batch, dim, 1) form: the token is a view
+    st, w, b = quantised((B, C, S), dtype), quantised((C, W), dtype, 0.5), quantised((C,), dtype, 0.1)
+    dout = quantised((B, C), dtype)
+    runs = []
+    for _ in range(2):
+        xg = x3.to(DEV).requires_grad_(True)
+        s0 = st.to(DEV).requires_grad_(True)
+        wg = w.to(DEV).requires_grad_(True)
+        bg = b.to(DEV).requires_grad_(True)
+        out = cc.causal_conv1d_update(xg, s0.clone(), wg, bg, activation="silu")
+        assert out.shape == (B, C, 1)
+        out.backward(dout.to(DEV).unsqueeze(-1))
+        torch.cuda.synchronize()
+        runs.append((xg.grad[:, :, 0], s0.grad, wg.grad, bg.grad))
+    for a, b_ in zip(*runs):
+        assert torch.equal(a, b_)
+    want = update_grads(x3[:, :, 0], st, w, b, dout, None, None, "silu", 0)
+    check(runs[0][0], want[0], dtype, "dx")
+    check(runs[0][1], want[1], dtype, "dstate")
+    check(runs[0][2], want[2], dtype, "dweight", sum_terms=B)
+    check(runs[0][3], want[3], dtype, "dbias", sum_terms=B)
+
+
+def test_update_backward_argument_handling(cc):
+    x = torch.randn(2, 8, device=DEV, requires_grad=True)
+    w = torch.randn(8, 4, device=DEV)
+    with pytest.raises(NotImplementedError, match="shift-register mode"):
+        cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV), w,
+                                cache_seqlens=torch.zeros(2, dtype=torch.int32, device=DEV))
+    with pytest.raises(NotImplementedError, match="shift-register mode"):
+        cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV), w, rounding="eager")
+    # a state that is a leaf requiring grad cannot be updated in place: torch says so itself
+    with pytest.raises(RuntimeError, match="leaf"):
+        cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV, requires_grad=True), w)
+    # only the token needs a gradient: no parameter gradients are formed, the cache tensor is updated in place
+    state = torch.randn(2, 8, 4, device=DEV)
+    before = state.clone()
+    out = cc.causal_conv1d_update(x, state, w)
+    out.sum().backward()
+    assert torch.equal(state[:, :, :3], before[:, :, 1:]) and torch.equal(state[:, :, 3], x.detach())
+    assert torch.allclose(x.grad, w[:, 3].expand(2, 8))
+    # under no_grad nothing is recorded and no copy of the state is made
+    with torch.no_grad():
+        assert not cc.causal_conv1d_update(x, state, w).requires_grad

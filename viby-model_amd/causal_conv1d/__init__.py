@@ -77,8 +77,8 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
 def _no_grad_needed(*tensors) -> None:
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
         raise NotImplementedError(
-            "causal_conv1d_update (gfx950): backward of the decode step is not implemented; call under "
-            "torch.no_grad() or detach the inputs")
+            "causal_conv1d_update_parts (gfx950): backward of the decode step is implemented for the single-tensor "
+            "call only; call under torch.no_grad() or detach the inputs")
 
 
 def _check_shapes(x_dim: int, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
@@ -500,7 +500,13 @@ def causal_conv1d_update(
     _check_devices(weight, bias, x.device)
     if conv_state.shape[2] < weight.shape[1] - 1:
         raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
-    _no_grad_needed(x, weight, bias, conv_state)
+    wants_grad = _wants_grad(x, weight, bias, conv_state)
+    if wants_grad and (cache_seqlens is not None or conv_state_indices is not None or rnd != 0
+                       or torch.compiler.is_compiling()):
+        raise NotImplementedError(
+            "causal_conv1d_update (gfx950): the backward of the decode step covers the shift-register mode with "
+            "rounding='fused' outside torch.compile (no cache_seqlens / conv_state_indices); call under "
+            "torch.no_grad() or detach the inputs")
     bias = _prep_bias(weight, bias)
     if token_mask is not None:
         if token_mask.dim() != 1 or token_mask.shape[0] != batch:
@@ -508,7 +514,9 @@ def causal_conv1d_update(
         if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x.device:
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
 
-    if torch.compiler.is_compiling():
+    if wants_grad:
+        out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res)
+    elif torch.compiler.is_compiling():
         out = torch.ops.canon_conv1d.update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices,
                                             act, res, rnd)
     else:
@@ -527,6 +535,95 @@ def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv
         rc = _call(_lib.lib().canon_conv1d_update, x2.device, ctypes.byref(p))
         _lib.check(rc, "causal_conv1d_update")
     return out
+
+
+class _CanonUpdateFn(torch.autograd.Function):
+    """Autograd node of one decode step.  The forward overwrites ``conv_state``, so a copy of the
+    state as it was is kept for the backward (as ShortConvUpdateMPSFunction does,
+    causal_conv1d_mps/autograd.py:452-453); ``conv_state`` is declared modified in place and
+    returned, so a gradient that arrives through the updated state (the next decode step reading
+    it) flows back into this step's token and into the state before it."""
+
+    @staticmethod
+    def forward(ctx, x2, conv_state, weight, bias, token_mask, act, res):
+        before = conv_state.detach().clone()
+        out = _launch_update(x2, conv_state, weight, bias, token_mask, None, None, act, res, 0)
+        ctx.mark_dirty(conv_state)
+        ctx.set_materialize_grads(False)
+        ctx.save_for_backward(x2, before, weight, bias, token_mask)
+        ctx.flags = (act, res)
+        return out, conv_state
+
+    @staticmethod
+    def backward(ctx, dout, dstate_out):
+        x2, before, weight, bias, token_mask = ctx.saved_tensors
+        act, res = ctx.flags
+        if dout is None:
+            dout = torch.zeros_like(x2)
+        want_state = ctx.needs_input_grad[1]
+        want_params = ctx.needs_input_grad[2] or (bias is not None and ctx.needs_input_grad[3])
+        dx, dstate, dweight, dbias = _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res,
+                                                        want_state, want_params)
+        return (dx, dstate, dweight.to(weight.dtype) if dweight is not None else None,
+                dbias.to(bias.dtype) if dbias is not None else None, None, None, None)
+
+
+def _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res, want_state=True,
+                       want_params=True):
+    """One launch (+ the fixed-order reduction over the batch): (dx, dstate | None, dweight | None, dbias | None),
+    the parameter gradients in fp32."""
+    if dout.dtype != x2.dtype:
+        dout = dout.to(x2.dtype)
+    if dstate_out is not None and dstate_out.dtype != x2.dtype:
+        dstate_out = dstate_out.to(x2.dtype)
+    batch, channels = x2.shape
+    width = weight.shape[1]
+    dev = x2.device
+    dx = torch.empty(batch, channels, dtype=x2.dtype, device=dev)
+    dstate = torch.empty(tuple(before.shape), dtype=x2.dtype, device=dev) if want_state else None
+    dweight = torch.empty(channels, width, dtype=torch.float32, device=dev) if want_params else None
+    dbias = torch.empty(channels, dtype=torch.float32, device=dev) if want_params and bias is not None else None
+    p = _lib.UpdateBwdParams()
+    p.struct_size = ctypes.sizeof(_lib.UpdateBwdParams)
+    p.x_dtype = _lib.DTYPE_CODE[x2.dtype]
+    p.w_dtype = _lib.DTYPE_CODE[weight.dtype]
+    p.width = width
+    p.activation, p.residual_mode = act, res
+    p.state_len = before.shape[2]
+    p.batch, p.channels = batch, channels
+    p.x = x2.data_ptr()
+    p.x_stride_b, p.x_stride_c = x2.stride()
+    p.conv_state = before.data_ptr()
+    p.state_stride_b, p.state_stride_c, p.state_stride_s = before.stride()
+    p.weight = weight.data_ptr()
+    p.w_stride_c, p.w_stride_k = weight.stride()
+    p.bias = bias.data_ptr() if bias is not None else None
+    if token_mask is not None:
+        p.token_mask = token_mask.data_ptr()
+        p.mask_dtype = _lib.MASK_CODE[token_mask.dtype]
+        p.mask_stride_b = token_mask.stride(0)
+    p.dout = dout.data_ptr()
+    p.dout_stride_b, p.dout_stride_c = dout.stride()
+    if dstate_out is not None:
+        p.dstate_out = dstate_out.data_ptr()
+        p.dstate_out_stride_b, p.dstate_out_stride_c, p.dstate_out_stride_s = dstate_out.stride()
+    p.dx = dx.data_ptr()
+    p.dx_stride_b, p.dx_stride_c = dx.stride()
+    if dstate is not None:
+        p.dstate = dstate.data_ptr()
+        p.dstate_stride_b, p.dstate_stride_c, p.dstate_stride_s = dstate.stride()
+    p.dweight = dweight.data_ptr() if dweight is not None else None
+    p.dbias = dbias.data_ptr() if dbias is not None else None
+    L = _lib.lib()
+    nbytes = L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(p))
+    if nbytes < 0:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "causal_conv1d_update backward")
+    workspace = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=dev)
+    p.workspace = workspace.data_ptr()
+    p.workspace_bytes = workspace.numel()
+    rc = _call(L.canon_conv1d_update_bwd, dev, ctypes.byref(p))
+    _lib.check(rc, "causal_conv1d_update backward")
+    return dx, dstate, dweight, dbias
 
 
 # ---------------------------------------------------------------------------

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -80,6 +80,26 @@ class BwdParams(ctypes.Structure):
     ]
 
 
+class UpdateBwdParams(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", _u32),
+        ("x_dtype", _i32), ("w_dtype", _i32), ("mask_dtype", _i32),
+        ("width", _i32), ("activation", _i32), ("residual_mode", _i32), ("state_len", _i32),
+        ("batch", _i64), ("channels", _i64),
+        ("x", _vp), ("x_stride_b", _i64), ("x_stride_c", _i64),
+        ("conv_state", _vp), ("state_stride_b", _i64), ("state_stride_c", _i64), ("state_stride_s", _i64),
+        ("weight", _vp), ("w_stride_c", _i64), ("w_stride_k", _i64),
+        ("bias", _vp),
+        ("token_mask", _vp), ("mask_stride_b", _i64),
+        ("dout", _vp), ("dout_stride_b", _i64), ("dout_stride_c", _i64),
+        ("dstate_out", _vp), ("dstate_out_stride_b", _i64), ("dstate_out_stride_c", _i64), ("dstate_out_stride_s", _i64),
+        ("dx", _vp), ("dx_stride_b", _i64), ("dx_stride_c", _i64),
+        ("dstate", _vp), ("dstate_stride_b", _i64), ("dstate_stride_c", _i64), ("dstate_stride_s", _i64),
+        ("dweight", _vp), ("dbias", _vp),
+        ("workspace", _vp), ("workspace_bytes", _i64),
+    ]
+
+
 class Part(ctypes.Structure):
     _fields_ = [
         ("x", _vp), ("x_stride_b", _i64), ("x_stride_c", _i64), ("x_stride_l", _i64),
@@ -100,6 +120,8 @@ EXPORTS = (
     "canon_conv1d_bwd",
     "canon_conv1d_bwd_workspace_bytes",
     "canon_conv1d_bwd_plan",
+    "canon_conv1d_update_bwd",
+    "canon_conv1d_update_bwd_workspace_bytes",
     "canon_conv1d_fwd_parts",
     "canon_conv1d_update_parts",
     "canon_conv1d_fwd_parts_plan",
@@ -136,6 +158,10 @@ def lib() -> ctypes.CDLL:
         L.canon_conv1d_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdParams)]
         L.canon_conv1d_bwd_plan.restype = ctypes.c_char_p
         L.canon_conv1d_bwd_plan.argtypes = [ctypes.POINTER(BwdParams)]
+        L.canon_conv1d_update_bwd.restype = ctypes.c_int
+        L.canon_conv1d_update_bwd.argtypes = [ctypes.POINTER(UpdateBwdParams), _vp]
+        L.canon_conv1d_update_bwd_workspace_bytes.restype = ctypes.c_int64
+        L.canon_conv1d_update_bwd_workspace_bytes.argtypes = [ctypes.POINTER(UpdateBwdParams)]
         L.canon_conv1d_fwd_parts.restype = ctypes.c_int
         L.canon_conv1d_fwd_parts.argtypes = [ctypes.POINTER(FwdParams), ctypes.POINTER(Part), _i32, _vp]
         L.canon_conv1d_update_parts.restype = ctypes.c_int

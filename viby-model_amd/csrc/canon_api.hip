@@ -601,6 +601,76 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     return CANON_OK;
 }
 
+int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, bool check_pointers)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_update_bwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT,
+                    "struct_size %u does not match this library's canon_conv1d_update_bwd_params (%zu)", p->struct_size,
+                    sizeof(canon_conv1d_update_bwd_params));
+    if (!valid_dtype(p->x_dtype) || !valid_dtype(p->w_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown x_dtype %d or w_dtype %d", p->x_dtype, p->w_dtype);
+    if (p->width < CANON_CONV1D_MIN_WIDTH || p->width > CANON_CONV1D_MAX_WIDTH)
+        return fail(CANON_ERR_UNSUPPORTED, "width %d not supported (only widths 2..4)", p->width);
+    if (p->activation != CANON_ACT_NONE && p->activation != CANON_ACT_SILU)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown activation %d", p->activation);
+    if (p->residual_mode < CANON_RESIDUAL_NONE || p->residual_mode > CANON_RESIDUAL_UNMASKED)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown residual_mode %d", p->residual_mode);
+    if (p->batch < 0 || p->channels < 0)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "negative size (batch %lld, channels %lld)", (long long)p->batch,
+                    (long long)p->channels);
+    if (p->batch >= (1ll << 31) || p->channels >= (1ll << 29) || p->batch * p->channels >= (1ll << 31))
+        return fail(CANON_ERR_UNSUPPORTED, "batch*channels must be below 2^31 and channels below 2^29");
+    if (p->state_len < 1 || p->state_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_len %d is shorter than width-1 = %d", p->state_len, p->width - 1);
+    if (p->token_mask && !valid_mask_dtype(p->mask_dtype))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    if (p->dbias && !p->dweight) return fail(CANON_ERR_INVALID_ARGUMENT, "dbias needs dweight");
+    const bool empty = p->batch == 0 || p->channels == 0;
+    if (check_pointers && !empty) {
+        if (!p->x || !p->conv_state || !p->weight || !p->dout || !p->dx)
+            return fail(CANON_ERR_INVALID_ARGUMENT, "x, conv_state, weight, dout and dx must not be NULL");
+        if (p->dstate && p->dstate == p->dstate_out)
+            return fail(CANON_ERR_INVALID_ARGUMENT, "dstate must not alias dstate_out");
+    }
+
+    UpdBwdArgs &a = plan->args;
+    memset(&a, 0, sizeof(a));
+    a.x = (const char *)p->x; a.state = (const char *)p->conv_state; a.dy = (const char *)p->dout;
+    a.dso = (const char *)p->dstate_out; a.dx = (char *)p->dx; a.ds = (char *)p->dstate;
+    a.weight = p->weight; a.bias = p->bias; a.tmask = p->token_mask;
+    a.dweight = p->dweight; a.dbias = p->dbias;
+    a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.g_sb = p->dout_stride_b; a.g_sc = p->dout_stride_c;
+    a.d_sb = p->dx_stride_b; a.d_sc = p->dx_stride_c;
+    a.s_sb = p->state_stride_b; a.s_sc = p->state_stride_c; a.s_ss = p->state_stride_s;
+    a.q_sb = p->dstate_out_stride_b; a.q_sc = p->dstate_out_stride_c; a.q_ss = p->dstate_out_stride_s;
+    a.r_sb = p->dstate_stride_b; a.r_sc = p->dstate_stride_c; a.r_ss = p->dstate_stride_s;
+    a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k; a.m_sb = p->mask_stride_b;
+    a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels;
+    a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
+    a.act = p->activation; a.res_mode = p->residual_mode;
+    plan->grid_c = 0;
+    plan->workspace_bytes = 0;
+    if (empty) return CANON_OK;
+
+    // batch entries per thread: enough groups for about four blocks per compute unit, at most 1024 groups
+    const uint32_t grid_c = (a.C + 255u) / 256u;
+    uint32_t want = (1024u + grid_c - 1u) / grid_c;
+    if (want > 1024u) want = 1024u;
+    if (want > a.B) want = a.B;
+    a.group = (a.B + want - 1u) / want;
+    a.ngroups = (a.B + a.group - 1u) / a.group;
+    plan->grid_c = grid_c;
+    if (p->dweight) {
+        plan->workspace_bytes = (int64_t)a.ngroups * a.C * 5 * (int64_t)sizeof(float);
+        a.partial = (float *)p->workspace;
+        if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",
+                        (long long)plan->workspace_bytes, (long long)p->workspace_bytes);
+    }
+    return CANON_OK;
+}
+
 int check_launch(const char *what)
 {
     const hipError_t e = hipGetLastError();
@@ -664,6 +734,32 @@ CANON_API int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params
 {
     BwdPlan pl;
     if (plan_bwd(p, &pl, false) != CANON_OK) return -1;
+    return pl.workspace_bytes;
+}
+
+CANON_API int canon_conv1d_update_bwd(const canon_conv1d_update_bwd_params *p, void *stream)
+{
+    UpdBwdPlan pl;
+    const int rc = plan_update_bwd(p, &pl, true);
+    if (rc != CANON_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (pl.grid_c == 0) {
+        // an empty batch: the parameter gradients are zero (fill kernels, so that the call can be captured)
+        if (p->channels > 0 && p->dweight) {
+            launch_zero(p->dweight, (uint32_t)(p->channels * p->width), s);
+            if (p->dbias) launch_zero(p->dbias, (uint32_t)p->channels, s);
+            return check_launch("canon_conv1d_update_bwd");
+        }
+        return CANON_OK;
+    }
+    launch_update_bwd(pl, p->x_dtype, s);
+    return check_launch("canon_conv1d_update_bwd");
+}
+
+CANON_API int64_t canon_conv1d_update_bwd_workspace_bytes(const canon_conv1d_update_bwd_params *p)
+{
+    UpdBwdPlan pl;
+    if (plan_update_bwd(p, &pl, false) != CANON_OK) return -1;
     return pl.workspace_bytes;
 }
 

@@ -930,6 +930,87 @@ __global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *part
 }
 
 // ---------------------------------------------------------------------------
+// backward of one decode step (shift-register state).  A thread owns one
+// channel and walks the batch entries of its group in order, so a wave reads
+// dense stretches of x / dout / the state and the partial sums of dweight /
+// dbias it leaves per group are formed in a fixed order; canon_bwd_reduce_kernel
+// then sums the groups.  z is recomputed from the saved state and the token.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs a)
+{
+    constexpr int NB = 4;                   // batch entries whose loads are requested together
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= a.C) return;
+    const uint32_t g = blockIdx.y;
+    const int W = a.W, S = a.S;
+    const int first = S - (W - 1);          // state slot read by tap 0
+    float w[4] = {0, 0, 0, 0};
+    for (int k = 0; k < W; ++k) w[k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
+    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+    float dw[4] = {0, 0, 0, 0}, db = 0.0f;
+    const uint32_t b_begin = g * a.group;
+    const uint32_t b_stop = b_begin + a.group < a.B ? b_begin + a.group : a.B;
+    for (uint32_t b0 = b_begin; b0 < b_stop; b0 += NB) {
+        // every load of the NB entries first (nothing is stored in between, so they are in flight together)
+        float xr[NB], go[NB], m[NB], win[NB][4], q[NB][4];
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = b0 + n < b_stop ? b0 + n : b_stop - 1u;
+            xr[n] = load1<DT>(a.x, (int64_t)b * a.x_sb + (int64_t)c * a.x_sc);
+            go[n] = load1<DT>(a.dy, (int64_t)b * a.g_sb + (int64_t)c * a.g_sc);
+            m[n] = a.tmask ? load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype) : 1.0f;
+            const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
+            const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                win[n][k] = k < W - 1 ? load1<DT>(a.state, so + (int64_t)(first + k) * a.s_ss) : 0.0f;
+                // q[k]: gradient of the updated state at slot first-1+k (what shifts into slot first+k, and the
+                // token's own slot S-1 for k = W-1)
+                const int j = first - 1 + k;
+                q[n][k] = (a.dso && k < W && j >= 0) ? load1<DT>(a.dso, qo + (int64_t)j * a.q_ss) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = b0 + n;
+            if (b >= b_stop) break;
+            const float xt = a.tmask ? mul_round<DT>(xr[n], m[n]) : xr[n];
+            float dz = go[n];
+            if (a.act) {
+                float z = bv;
+                for (int k = 0; k < W - 1; ++k) z = fmaf(w[k], win[n][k], z);
+                z = fmaf(w[W - 1], xt, z);
+                dz = go[n] * silu_grad(z);
+            }
+            for (int k = 0; k < W - 1; ++k) dw[k] = fmaf(dz, win[n][k], dw[k]);
+            dw[W - 1] = fmaf(dz, xt, dw[W - 1]);
+            db += dz;
+            float dxt = w[W - 1] * dz;
+            if (a.res_mode == CANON_RESIDUAL_MASKED) dxt += go[n];
+            dxt += q[n][W - 1];
+            float dxv = a.tmask ? dxt * m[n] : dxt;
+            if (a.res_mode == CANON_RESIDUAL_UNMASKED) dxv += go[n];
+            store1<DT>(a.dx, (int64_t)b * a.d_sb + (int64_t)c * a.d_sc, dxv);
+            if (a.ds) {
+                const int64_t ro = (int64_t)b * a.r_sb + (int64_t)c * a.r_sc;
+                const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
+                // slots no tap reads: the gradient of the updated state shifted by one
+                for (int j = 0; j < first; ++j)
+                    store1<DT>(a.ds, ro + (int64_t)j * a.r_ss,
+                               (a.dso && j >= 1) ? load1<DT>(a.dso, qo + (int64_t)(j - 1) * a.q_ss) : 0.0f);
+                for (int k = 0; k < W - 1; ++k)
+                    store1<DT>(a.ds, ro + (int64_t)(first + k) * a.r_ss, fmaf(w[k], dz, q[n][k]));
+            }
+        }
+    }
+    if (a.partial) {
+        float *pp = a.partial + ((int64_t)g * a.C + c) * 5;
+        pp[0] = dw[0]; pp[1] = dw[1]; pp[2] = dw[2]; pp[3] = dw[3]; pp[4] = db;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------
 namespace {
@@ -975,6 +1056,19 @@ void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s)
     }
     hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 31u) / 32u), dim3(256), 0, s,
                        pl.args.partial, pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.nsets, pl.args.W);
+}
+
+void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s)
+{
+    const dim3 g(pl.grid_c, pl.args.ngroups), b(256);
+    switch (x_dtype) {
+    case CANON_DTYPE_F32: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F32>), g, b, 0, s, pl.args); break;
+    case CANON_DTYPE_BF16: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_BF16>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F16>), g, b, 0, s, pl.args); break;
+    }
+    if (pl.args.partial)
+        hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 31u) / 32u), dim3(256), 0, s, pl.args.partial,
+                           pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.ngroups, pl.args.W);
 }
 
 void launch_zero(float *p, uint32_t n, hipStream_t s)

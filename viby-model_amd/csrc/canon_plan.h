@@ -128,6 +128,29 @@ struct BwdArgs {
     FastDiv div_nvec, div_nchunk, div_nct;
 };
 
+// backward of one decode step: a thread owns a channel and walks the batch entries of its group
+struct UpdBwdArgs {
+    const char *x;
+    const char *state;     // the state before the step
+    const char *dy;
+    const char *dso;       // gradient w.r.t. the updated state, or nullptr
+    char *dx;
+    char *ds;              // gradient w.r.t. the state before, or nullptr
+    const void *weight;
+    const void *bias;
+    const void *tmask;
+    float *partial;        // [ngroups][C][5] partial sums of dweight / dbias, or nullptr
+    float *dweight;
+    float *dbias;
+    int64_t x_sb, x_sc, g_sb, g_sc, d_sb, d_sc;
+    int64_t s_sb, s_sc, s_ss, q_sb, q_sc, q_ss, r_sb, r_sc, r_ss;   // state, dstate_out, dstate
+    int64_t w_sc, w_sk, m_sb;
+    uint32_t B, C;
+    uint32_t group;        // batch entries per group
+    uint32_t ngroups;
+    int32_t W, S, w_dtype, mask_dtype, act, res_mode;
+};
+
 // Several channel ranges of one logical [B, C, L] problem that live in separate
 // tensors (q / k / v or gate / up projections), one launch: every block belongs
 // to one part and runs the single-tensor code on that part's argument block.
@@ -205,12 +228,19 @@ struct BwdPlan {
     int64_t workspace_bytes;
 };
 
+struct UpdBwdPlan {
+    UpdBwdArgs args;
+    uint32_t grid_c;        // blocks along the channels (0: nothing to launch)
+    int64_t workspace_bytes;
+};
+
 // Launchers (x_dtype is a CANON_DTYPE_* code; nothing here synchronises)
 void launch_fwd(const FwdPlan &pl, int x_dtype, hipStream_t s);
 void launch_fwd_parts(const FwdPartsPlan &pp, int x_dtype, hipStream_t s);
 void launch_update(const UpdPlan &pl, int x_dtype, hipStream_t s);
 void launch_update_parts(const UpdPartsPlan &pp, int x_dtype, hipStream_t s);
 void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s);          // dx + partial sets, then the reduction
+void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s);   // dx, dstate + partial sets, then the reduction
 void launch_zero(float *p, uint32_t n, hipStream_t s);                    // fill kernel (graph-capture safe)
 
 }  // namespace canon

@@ -193,3 +193,30 @@ def test_update_backward_argument_handling(cc):
     # under no_grad nothing is recorded and no copy of the state is made
     with torch.no_grad():
         assert not cc.causal_conv1d_update(x, state, w).requires_grad
+
+
+def test_canon_layer_trains_through_single_token_steps(cc):
+    """The drop-in CanonLayer fed token by token through its cache (model/model.py:270-317) has the
+    parameter and input gradients of the same layer called once on the whole block (:587-675)."""
+    import types
+    from causal_conv1d.canon import CanonLayer
+    torch.manual_seed(11)
+    B, T, D = 3, 6, 192
+    cfg = types.SimpleNamespace(canon_kernel=4, canon_bias=True, canon_activation=True)
+    layer = CanonLayer(D, cfg, "a").to(DEV)
+    layer.reset_parameters()
+    x = torch.randn(B, T, D, device=DEV)
+    dout = torch.randn(B, T, D, device=DEV)
+
+    xb = x.clone().requires_grad_(True)
+    layer(xb).backward(dout)
+    want = (xb.grad.clone(), layer.weight.grad.clone(), layer.bias_param.grad.clone())
+    layer.zero_grad()
+
+    xs = x.clone().requires_grad_(True)
+    cache = types.SimpleNamespace()
+    ys = [layer(xs[:, t:t + 1], cache=cache, layer_idx=0) for t in range(T)]
+    torch.cat(ys, dim=1).backward(dout)
+    torch.cuda.synchronize()
+    for got, ref, tol in zip((xs.grad, layer.weight.grad, layer.bias_param.grad), want, (2e-5, 1e-4, 1e-4)):
+        assert (got - ref).abs().max().item() <= tol * scale_of(ref)

@@ -32,9 +32,11 @@ Canon-B, gate and up for Canon-D) and returns one output per part, so the
 is not needed; the state on the cache is the same single tensor either way.
 
 Training: a block call without a cache is differentiable (fused backward
-kernel); the cached paths (prefill with state capture continues to work, the
-single-token step does not) are inference paths: run them under
-``torch.no_grad()`` / ``torch.inference_mode()``.
+kernel), and so are a prefill with state capture and the single-token step
+of ``forward`` (its own backward kernel; the cache tensor then carries the
+graph from step to step).  The chunked continuation (``initial_states``) and
+the single-token step of ``forward_parts`` are inference paths: run them
+under ``torch.no_grad()`` / ``torch.inference_mode()``.
 """
 from __future__ import annotations
 

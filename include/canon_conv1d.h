@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 4
+#define CANON_CONV1D_ABI_VERSION 5
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -171,7 +171,7 @@ typedef struct canon_conv1d_update_params {
 } canon_conv1d_update_params;
 
 /*
- * Backward of canon_conv1d_fwd (no initial/final state): the gradient a
+ * Backward of canon_conv1d_fwd (final_state carries no gradient): the gradient a
  * training step needs so that the fused forward can stay on the accelerated
  * path (trainer/base_trainer.py:274 calls backward through every Canon
  * layer).  Same role as the reference's own backward kernels
@@ -218,6 +218,16 @@ typedef struct canon_conv1d_bwd_params {
     int64_t workspace_bytes;
     const int32_t *seq_idx;         /* [batch, seqlen] or NULL: the forward's packed-sequence indices */
     int64_t seq_stride_b, seq_stride_l;
+    const void *initial_state;      /* [batch, channels, initial_len] or NULL: the forward's initial_state (the chunked
+                                       continuation of model/model.py:647-659 as one differentiable call); its last
+                                       W-1 entries enter z as the inputs before t = 0 and dweight with them.  Not with
+                                       seq_idx.  Such calls take the strided kernel. */
+    int64_t init_stride_b, init_stride_c, init_stride_s;
+    int32_t initial_len;            /* >= W-1 when initial_state != NULL */
+    int32_t reserved1;
+    void *dinitial_state;           /* [batch, channels, initial_len] in x_dtype, or NULL: receives the gradient w.r.t.
+                                       initial_state (zero for entries older than W-1); needs initial_state */
+    int64_t dinit_stride_b, dinit_stride_c, dinit_stride_s;
 } canon_conv1d_bwd_params;
 
 /*

@@ -16,6 +16,11 @@ form is pinned by the tests in two ways: its output against the C oracle of
 the packed forward, and its gradients against this same function run without
 ``seq_idx`` on every sequence cut out on its own.
 
+With ``initial_states`` the zero padding is replaced by their last W-1
+entries (``torch.cat`` instead of ``F.pad``); pinned by the tests through the
+split property: a block cut in two, the second half continued from the first
+half's last inputs, has the gradients of the block convolved in one go.
+
 ``update_grads`` does the same for one decode step in the formulation of
 the eager module's step (model/model.py:372-398): the window is the last
 W-1 state slots and the token, ``out = act(bias + sum_k w[k] * window[k])``
@@ -36,16 +41,22 @@ import torch.nn.functional as F
 
 def conv1d_grads(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], dout: torch.Tensor,
                  mask: Optional[torch.Tensor] = None, activation=None, residual=0,
-                 seq_idx: Optional[torch.Tensor] = None
-                 ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
+                 seq_idx: Optional[torch.Tensor] = None, initial_states: Optional[torch.Tensor] = None):
     """x, dout logical [B, C, L]; weight [C, W] and bias [C] are first rounded to x.dtype, as the
-    forward does.  Returns (dx, dweight, dbias, out) in float64."""
+    forward does.  Returns (dx, dweight, dbias, out) in float64; with ``initial_states`` [B, C, S >= W-1]
+    (the inputs before t = 0 instead of the zero padding, unmasked: the chunked continuation of
+    model/model.py:647-659) also their gradient as a fifth entry."""
     C, W = weight.shape
     x64 = x.detach().cpu().double().requires_grad_(True)
     w64 = weight.detach().cpu().to(x.dtype).double().requires_grad_(True)
     b64 = bias.detach().cpu().to(x.dtype).double().requires_grad_(True) if bias is not None else None
     xm = x64 if mask is None else x64 * mask.detach().cpu().double().unsqueeze(1)
-    if seq_idx is None:
+    h64 = None
+    if initial_states is not None:
+        assert seq_idx is None
+        h64 = initial_states.detach().cpu().double().requires_grad_(True)
+        z = F.conv1d(torch.cat([h64[:, :, h64.shape[2] - (W - 1):], xm], dim=2), w64.unsqueeze(1), b64, groups=C)
+    elif seq_idx is None:
         z = F.conv1d(F.pad(xm, (W - 1, 0)), w64.unsqueeze(1), b64, groups=C)
     else:
         L = x64.shape[2]
@@ -63,6 +74,8 @@ def conv1d_grads(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     elif residual in (2, "unmasked"):
         y = y + x64
     y.backward(dout.detach().cpu().double())
+    if h64 is not None:
+        return x64.grad, w64.grad, (b64.grad if b64 is not None else None), y.detach(), h64.grad
     return x64.grad, w64.grad, (b64.grad if b64 is not None else None), y.detach()
 
 

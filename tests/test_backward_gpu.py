@@ -223,7 +223,7 @@ def test_unsupported_gradients_raise(cc):
     x = torch.randn(2, 8, 16, device=DEV, requires_grad=True)
     w = torch.randn(8, 4, device=DEV)
     with pytest.raises(NotImplementedError, match="initial_states"):
-        cc.causal_conv1d_fn(x, w, initial_states=torch.zeros(2, 8, 3, device=DEV))
+        cc.causal_conv1d_fn_parts([x[:, :4], x[:, 4:]], w, initial_states=torch.zeros(2, 8, 3, device=DEV))
     with pytest.raises(NotImplementedError, match="backward of the decode step"):
         cc.causal_conv1d_update_parts([x[:, :4, 0], x[:, 4:, 0]], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
@@ -391,3 +391,43 @@ def test_forward_and_backward_inside_a_captured_graph(cc):
         torch.cuda.synchronize()
         for name, got, exp in zip(("y", "dx", "dweight", "dbias"), outs, want):
             assert torch.equal(bits(got), bits(exp)), (i, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["bcl", "blc"])
+def test_backward_through_initial_states(cc, dtype, layout):
+    """A call continued from an initial state (the chunked continuation of model/model.py:647-659): dx, dweight,
+    dbias and the gradient of the state itself against float64 autograd; rows shorter and longer than the
+    history, several time chunks per row, all widths."""
+    torch.manual_seed(17)
+    for (B, C, L, S, W), act, residual, masked in itertools.product(
+            [(2, 24, 1, 3, 4), (2, 24, 2, 4, 4), (3, 40, 5, 8, 4), (2, 16, 700, 3, 4), (2, 24, 37, 2, 3), (2, 24, 9, 4, 2)],
+            [None, "silu"], [False, True, "unmasked"], [False, True]):
+        x = torch.randn(B, C, L).to(dtype)
+        w, b = (torch.randn(C, W) * 0.5).to(dtype), (torch.randn(C) * 0.1).to(dtype)
+        init = torch.randn(B, C, S).to(dtype)
+        dout = torch.randn(B, C, L).to(dtype)
+        mask = (torch.rand(B, L) > 0.3).to(torch.int64) if masked else None
+        xg, dg = x.to(DEV), dout.to(DEV)
+        if layout == "blc":
+            xg = xg.transpose(1, 2).contiguous().transpose(1, 2)
+            dg = dg.transpose(1, 2).contiguous().transpose(1, 2)
+        xg.requires_grad_(True)
+        wg, bg = w.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+        ig = init.to(DEV).requires_grad_(True)
+        out = cc.causal_conv1d_fn(xg, wg, bg, activation=act, initial_states=ig, residual=residual,
+                                  attention_mask=None if mask is None else mask.to(DEV))
+        out.backward(dg)
+        torch.cuda.synchronize()
+        want = conv1d_grads(x, w, b, dout, mask=mask, activation=act, residual=residual, initial_states=init)
+        tag = f"{dtype} {layout} B{B} C{C} L{L} S{S} W{W} act={act} res={residual} mask={masked}"
+        check(xg.grad, want[0], dtype, "dx " + tag)
+        check(ig.grad, want[4], dtype, "dinit " + tag)
+        check(wg.grad, want[1], dtype, "dweight " + tag, sum_terms=B * L)
+        check(bg.grad, want[2], dtype, "dbias " + tag, sum_terms=B * L)
+    # only the state needs a gradient
+    ig = torch.randn(2, 8, 3, device=DEV, requires_grad=True)
+    w = torch.randn(8, 4, device=DEV)
+    cc.causal_conv1d_fn(torch.randn(2, 8, 6, device=DEV), w, initial_states=ig).sum().backward()
+    want = torch.stack([w[:, 0], w[:, 0] + w[:, 1], w[:, 0] + w[:, 1] + w[:, 2]], dim=1).expand(2, 8, 3)
+    assert torch.allclose(ig.grad, want, atol=1e-6)

@@ -510,3 +510,35 @@ def test_update_gradient_oracle_chained_equals_the_prefill_gradient_oracle():
             db += r[3]
         for got, want in ((dx, dx_ref), (dw, dw_ref), (db, db_ref)):
             assert torch.allclose(got, want, atol=1e-11), (S, W, act, res, masked)
+
+
+def test_gradient_oracle_with_initial_states_equals_the_block_in_one_go():
+    """conv1d_grads(initial_states=...) on the second half of a block, continued from the (masked) last inputs
+    of the first half, plus conv1d_grads on the first half, must add up to conv1d_grads on the whole block."""
+    from oracle.canon_grad import conv1d_grads
+    torch.manual_seed(1)
+    for W, S, act, res, masked, L1 in itertools.product([2, 3, 4], [3, 5], [None, "silu"], [0, 1, 2], [False, True],
+                                                        [1, 2, 7]):
+        if S < W - 1:
+            continue
+        B, C, L2 = 2, 3, 5
+        x = torch.randn(B, C, L1 + L2).double()
+        w, b, dout = torch.randn(C, W).double(), torch.randn(C).double(), torch.randn(B, C, L1 + L2).double()
+        mask = (torch.rand(B, L1 + L2) > 0.3).double() if masked else None
+        m1, m2 = (None, None) if mask is None else (mask[:, :L1], mask[:, L1:])
+        whole = conv1d_grads(x, w, b, dout, mask=mask, activation=act, residual=res)
+        # state after the first half: its last S masked inputs, zero filled on the left
+        xm1 = x[:, :, :L1] if m1 is None else x[:, :, :L1] * m1.unsqueeze(1)
+        state = F.pad(xm1, (S, 0))[:, :, -S:]
+        second = conv1d_grads(x[:, :, L1:], w, b, dout[:, :, L1:], mask=m2, activation=act, residual=res,
+                              initial_states=state)
+        first = conv1d_grads(x[:, :, :L1], w, b, dout[:, :, :L1], mask=m1, activation=act, residual=res)
+        assert torch.allclose(torch.cat([first[3], second[3]], dim=2), whole[3], atol=1e-12)
+        # the state's gradient flows back into the inputs it copied (times their mask)
+        n = min(S, L1)
+        back = torch.zeros_like(first[0])
+        back[:, :, L1 - n:] = second[4][:, :, S - n:] * (1.0 if m1 is None else m1[:, L1 - n:].unsqueeze(1))
+        assert torch.allclose(torch.cat([first[0] + back, second[0]], dim=2), whole[0], atol=1e-11), (W, S, act, res)
+        assert torch.allclose(first[1] + second[1], whole[1], atol=1e-11)
+        assert torch.allclose(first[2] + second[2], whole[2], atol=1e-11)
+        assert float(second[4][:, :, :S - (W - 1)].abs().max()) == 0.0 if S > W - 1 else True

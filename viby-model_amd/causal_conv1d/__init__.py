@@ -263,7 +263,7 @@ def causal_conv1d_fn(
                      with different values do not see each other (the slot the
                      reference leaves at None, ``model/model.py:465``).  Inference
                      only, without initial / final states.
-    initial_states   (batch, dim, >= W-1): history before t = 0 instead of zeros.
+    initial_states   (batch, dim, >= W-1): history before t = 0 instead of zeros (differentiable).
     return_final_states / final_states_out (batch, dim, S): receives the last S
                      inputs (S = W-1 when allocated here; any S >= 1 when
                      given, e.g. the 4- or 8-slot conv_state of CanonLayer,
@@ -300,9 +300,10 @@ def causal_conv1d_fn(
     if x.numel() == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
-    if _wants_grad(x, weight, bias) and initial_states is not None:
-        raise NotImplementedError("gradients through a call with initial_states are not implemented")
     if torch.compiler.is_compiling():
+        if initial_states is not None and _wants_grad(x, weight, bias, initial_states):
+            raise NotImplementedError("gradients through a call with initial_states are not implemented under "
+                                      "torch.compile")
         # under torch.compile the launch is one opaque operator of the traced graph (trainer/train_pretrain.py:39
         # and eval_model.py:157 compile the whole model, the latter with fullgraph=True)
         result, fin = torch.ops.canon_conv1d.fwd(x, weight, bias, attention_mask, initial_states, seq_idx,
@@ -312,8 +313,9 @@ def causal_conv1d_fn(
             return result
         final_states.copy_(fin)
         return result, final_states
-    if _wants_grad(x, weight, bias):
-        result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd, seq_idx)
+    if _wants_grad(x, weight, bias, initial_states):
+        result = _CanonConvFn.apply(x, weight, bias, attention_mask, final_states, act, res, rnd, seq_idx,
+                                    initial_states)
     else:
         result = _launch_fwd(x, weight, bias, attention_mask, initial_states, final_states, act, res, rnd, seq_idx)
         if final_states is not None:
@@ -342,9 +344,9 @@ class _CanonConvFn(torch.autograd.Function):
     (causal_conv1d_mps/autograd.py:13-160, 162-338)."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd, seq_idx=None):
-        out = _launch_fwd(x, weight, bias, mask, None, final_states, act, res, rnd, seq_idx)
-        ctx.save_for_backward(x, weight, bias, mask, seq_idx)
+    def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd, seq_idx=None, initial_states=None):
+        out = _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx)
+        ctx.save_for_backward(x, weight, bias, mask, seq_idx, initial_states)
         ctx.flags = (act, res)
         if final_states is not None:
             ctx.mark_non_differentiable(final_states)
@@ -353,17 +355,21 @@ class _CanonConvFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout, *unused):
-        x, weight, bias, mask, seq_idx = ctx.saved_tensors
+        x, weight, bias, mask, seq_idx, initial_states = ctx.saved_tensors
         act, res = ctx.flags
         channels, width = weight.shape
         dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
         dbias = torch.empty(channels, dtype=torch.float32, device=x.device) if bias is not None else None
-        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx)
+        dinit = None
+        if initial_states is not None and ctx.needs_input_grad[9]:
+            dinit = torch.empty_like(initial_states)
+        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx, initial_states, dinit)
         return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
-                None, None, None, None, None, None)
+                None, None, None, None, None, None, dinit)
 
 
-def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=None) -> torch.Tensor:
+def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=None, initial_states=None,
+                dinit=None) -> torch.Tensor:
     """One backward launch (+ the fixed-order reduction): returns dx with x's strides and fills the
     fp32 ``dweight`` (channels, W) / ``dbias`` (channels,) given (rows of larger tensors are fine)."""
     if dout.dtype != x.dtype:
@@ -395,6 +401,16 @@ def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=N
     if seq_idx is not None:
         p.seq_idx = seq_idx.data_ptr()
         p.seq_stride_b, p.seq_stride_l = seq_idx.stride()
+    if initial_states is not None:
+        p.initial_state = initial_states.data_ptr()
+        p.init_stride_b, p.init_stride_c, p.init_stride_s = initial_states.stride()
+        p.initial_len = initial_states.shape[2]
+        if dinit is not None:
+            if x.numel() == 0:
+                dinit.zero_()
+            else:
+                p.dinitial_state = dinit.data_ptr()
+                p.dinit_stride_b, p.dinit_stride_c, p.dinit_stride_s = dinit.stride()
     p.dweight = dweight.data_ptr()
     p.dbias = dbias.data_ptr() if dbias is not None else None
     L = _lib.lib()

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -77,6 +77,9 @@ class BwdParams(ctypes.Structure):
         ("dweight", _vp), ("dbias", _vp),
         ("workspace", _vp), ("workspace_bytes", _i64),
         ("seq_idx", _vp), ("seq_stride_b", _i64), ("seq_stride_l", _i64),
+        ("initial_state", _vp), ("init_stride_b", _i64), ("init_stride_c", _i64), ("init_stride_s", _i64),
+        ("initial_len", _i32), ("reserved1", _i32),
+        ("dinitial_state", _vp), ("dinit_stride_b", _i64), ("dinit_stride_c", _i64), ("dinit_stride_s", _i64),
     ]
 
 

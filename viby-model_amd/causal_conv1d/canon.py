@@ -34,9 +34,11 @@ is not needed; the state on the cache is the same single tensor either way.
 Training: a block call without a cache is differentiable (fused backward
 kernel), and so are a prefill with state capture and the single-token step
 of ``forward`` (its own backward kernel; the cache tensor then carries the
-graph from step to step).  The chunked continuation (``initial_states``) and
-the single-token step of ``forward_parts`` are inference paths: run them
-under ``torch.no_grad()`` / ``torch.inference_mode()``.
+graph from step to step) and the chunked continuation of ``forward``
+(``initial_states``; the captured state itself carries no gradient, so the
+graph is cut at chunk boundaries).  The cached paths of ``forward_parts`` are
+inference paths: run them under ``torch.no_grad()`` /
+``torch.inference_mode()``.
 """
 from __future__ import annotations
 

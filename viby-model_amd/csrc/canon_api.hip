@@ -450,7 +450,15 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
     if (p->seq_idx && ((uintptr_t)p->seq_idx & 3u))
         return fail(CANON_ERR_INVALID_ARGUMENT, "seq_idx must be 4-byte aligned");
+    if (p->initial_state && p->seq_idx)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "initial_state cannot be combined with seq_idx");
+    if (p->initial_state && p->initial_len < p->width - 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "initial_len %d is shorter than width-1 = %d", p->initial_len, p->width - 1);
+    if (p->dinitial_state && !p->initial_state)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "dinitial_state needs initial_state");
     const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
+    if (empty && p->dinitial_state && p->batch > 0 && p->channels > 0)
+        return fail(CANON_ERR_UNSUPPORTED, "dinitial_state of an empty input (it is all zeros) is left to the caller");
     if (check_pointers) {
         if (p->channels > 0 && (!p->weight || !p->dweight))
             return fail(CANON_ERR_INVALID_ARGUMENT, "weight and dweight must not be NULL");
@@ -471,6 +479,10 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k;
     a.m_sb = p->mask_stride_b; a.m_sl = p->mask_stride_l;
     a.seq = p->seq_idx; a.q_sb = p->seq_stride_b; a.q_sl = p->seq_stride_l;
+    a.init = (const char *)p->initial_state; a.dinit = (char *)p->dinitial_state;
+    a.i_sb = p->init_stride_b; a.i_sc = p->init_stride_c; a.i_ss = p->init_stride_s;
+    a.j_sb = p->dinit_stride_b; a.j_sc = p->dinit_stride_c; a.j_ss = p->dinit_stride_s;
+    a.S_in = p->initial_state ? p->initial_len : 0;
     a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
     a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode;
@@ -485,7 +497,8 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
-    const bool packed = p->seq_idx != nullptr;   // packed sequences: only the walk kernel gates taps by sequence index
+    // packed sequences and an initial state: only the walk kernel gates taps by sequence index / reads the history
+    const bool packed = p->seq_idx != nullptr || p->initial_state != nullptr;
     const bool rows = !packed && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
                       a.d_sb % E == 0 && a.d_sc % E == 0;

@@ -18,6 +18,11 @@ namespace canon {
 // with one row per step, fetched R rows ahead).  The three dz values just past
 // the chunk are recomputed from memory.
 //
+// With an initial state (a.init) the rows before t = 0 are its last entries
+// instead of zeros: they enter the windows (z and dweight) like any other row,
+// and the lane that ends at t = 0 also forms their gradient from the three dz
+// values it carries out of the loop.
+//
 // SEQ (packed sequences): the sequence index of every row travels with it
 // (window, carried dz values, look-ahead).  A product of a tap with a row of
 // another sequence index is dropped wherever it appears: in z, in dx (the dz
@@ -70,6 +75,17 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
         g3[j][0] = load1<DT>(gb + (t > Lm1 ? Lm1 : t) * gs, 0);
     }
     if constexpr (MASK) load_mask_rows<7>(a.mask, (int64_t)b * a.m_sb, t_end - 4, a.L, a.m_sl, a.mask_dtype, m7);
+    // rows before t = 0: entries of the initial state (not masked), zeros without one
+    const char *ib = a.init ? a.init + ((int64_t)b * a.i_sb + (int64_t)c0 * a.i_sc + (int64_t)a.S_in * a.i_ss) * BY : nullptr;
+    const int64_t is = a.i_ss * BY;
+    float h7[7] = {0, 0, 0, 0, 0, 0, 0};
+    if (ib && t_end < 4) {
+#pragma unroll
+        for (int j = 0; j < 7; ++j) {
+            const int64_t t = t_end - 4 + j;
+            if (t < 0 && t >= -(int64_t)a.S_in) h7[j] = load1<DT>(ib + t * is, 0);
+        }
+    }
     int32_t q7[7] = {0, 0, 0, 0, 0, 0, 0};   // sequence indices of the same seven rows
     if constexpr (SEQ) load_seq_rows<7>(a.seq, (int64_t)b * a.q_sb, t_end - 4, a.L, a.q_sl, q7);
 
@@ -83,7 +99,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             float v = MASK ? mul_round<DT>(xr7[j][e], m7[j]) : xr7[j][e];
-            xr7[j][e] = inside ? v : 0.0f;
+            xr7[j][e] = inside ? v : (t < 0 ? h7[j] : 0.0f);
         }
     }
     // dzf[j] = dz[t_end + j]
@@ -125,7 +141,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
     for (int64_t t_hi = t_end - 1; t_hi >= t_begin; t_hi -= R) {
         // this batch: steps t_hi, t_hi-1, .., t_hi-R+1; needs dout of those steps and x rows t-4.
         // Rows are kept as loaded (raw) until their step, to keep the register count down.
-        float G[R], XN[R];
+        float G[R], XN[R], HN[R];
         float mk[R], mn[R];
         int32_t QN[R];
 #pragma unroll
@@ -135,6 +151,7 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
             const int64_t tn = t - 4 < 0 ? 0 : t - 4;
             G[r] = load1<DT>(gb + tg * gs, 0);
             XN[r] = load1<DT>(xb + tn * xs, 0);
+            HN[r] = (ib && t - 4 < 0 && t - 4 >= -(int64_t)a.S_in) ? load1<DT>(ib + (t - 4) * is, 0) : 0.0f;
             QN[r] = SEQ ? a.seq[(int64_t)b * a.q_sb + tn * a.q_sl] : 0;
             mk[r] = 1.0f;
             mn[r] = 1.0f;
@@ -212,13 +229,29 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
                 xw[3][e] = xw[2][e];
                 xw[2][e] = xw[1][e];
                 xw[1][e] = xw[0][e];
-                xw[0][e] = has_row ? v : 0.0f;
+                xw[0][e] = has_row ? v : HN[r];
             }
             if constexpr (SEQ) {
                 qf[2] = qf[1]; qf[1] = qf[0]; qf[0] = qw[3];
                 qw[3] = qw[2]; qw[2] = qw[1]; qw[1] = qw[0]; qw[0] = QN[r];
             }
             store1<DT>(db_ + t * ds, 0, o[0]);
+        }
+    }
+
+    if (a.dinit && ch == 0) {
+        // here dzf[i] = dz[i] (zero past the end of the row).  Entry s is the input at t = s - S_in = -d:
+        // its gradient is sum_i w[W-1-d-i] * dz[i] over the taps that exist
+        char *jb = a.dinit + ((int64_t)b * a.j_sb + (int64_t)c0 * a.j_sc) * BY;
+        for (int s = 0; s < a.S_in; ++s) {
+            const int d = a.S_in - s;
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                const int k = W - 1 - d - i;
+                if (k >= 0) acc = fmaf(w[0][k], dzf[i][0], acc);
+            }
+            store1<DT>(jb + (int64_t)s * a.j_ss * BY, 0, acc);
         }
     }
 

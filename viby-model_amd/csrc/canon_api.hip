@@ -664,11 +664,27 @@ int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, b
     a.act = p->activation; a.res_mode = p->residual_mode;
     plan->grid_c = 0;
     plan->workspace_bytes = 0;
+    plan->vec = false;
     if (empty) return CANON_OK;
 
+    const int S = p->state_len;
+    const int BY = elem_bytes(p->x_dtype);
+    const int E = upd_lane_channels(BY, S);
+    auto dense_state = [&](const void *ptr, int64_t sb, int64_t sc, int64_t ss) {
+        return !ptr || ((uintptr_t)ptr % 4 == 0 && ss == 1 && sc == S && sb * BY % 4 == 0);
+    };
+    auto dense_token = [&](const void *ptr, int64_t sb, int64_t sc) {
+        return (uintptr_t)ptr % 4 == 0 && sc == 1 && sb * BY % 4 == 0;
+    };
+    plan->vec = (S == 3 || S == 4) && a.C % E == 0 && (!check_pointers || (
+                    dense_token(p->x, a.x_sb, a.x_sc) && dense_token(p->dout, a.g_sb, a.g_sc) &&
+                    dense_token(p->dx, a.d_sb, a.d_sc) && dense_state(p->conv_state, a.s_sb, a.s_sc, a.s_ss) &&
+                    dense_state(p->dstate_out, a.q_sb, a.q_sc, a.q_ss) && dense_state(p->dstate, a.r_sb, a.r_sc, a.r_ss)));
     // batch entries per thread: enough groups for about four blocks per compute unit, at most 1024 groups
-    const uint32_t grid_c = (a.C + 255u) / 256u;
-    uint32_t want = (1024u + grid_c - 1u) / grid_c;
+    // (counted on the channels alone, so that the scratch size does not depend on the kernel chosen)
+    const uint32_t grid_c = (plan->vec ? a.C / E + 255u : a.C + 255u) / 256u;
+    const uint32_t cblocks = (a.C + 255u) / 256u;
+    uint32_t want = (1024u + cblocks - 1u) / cblocks;
     if (want > 1024u) want = 1024u;
     if (want > a.B) want = a.B;
     a.group = (a.B + want - 1u) / want;

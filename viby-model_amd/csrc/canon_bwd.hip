@@ -969,6 +969,59 @@ __global__ __launch_bounds__(256) void canon_bwd_reduce_kernel(const float *part
 // dbias it leaves per group are formed in a fixed order; canon_bwd_reduce_kernel
 // then sums the groups.  z is recomputed from the saved state and the token.
 // ---------------------------------------------------------------------------
+// Taps, window and sums are kept right-aligned in arrays of four (tap k of a width-W filter at index
+// 4-W+k, the token's tap always at 3, window entry i = state slot S-3+i), so every register array is
+// indexed by compile-time constants whatever W is.
+template <int DT>
+__device__ __forceinline__ void load_taps_right(const UpdBwdArgs &a, uint32_t c, float *wr, float &bv)
+{
+    const int lead = 4 - a.W;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        wr[i] = i >= lead ? round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + (i - lead) * a.w_sk, a.w_dtype)) : 0.0f;
+    bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
+}
+
+// one (batch entry, channel): wn[i] = state slot S-3+i (0 where no tap reads it), qr[i] = gradient of the updated
+// state at slot S-4+i (qr[3]: the token's own slot).  Returns dz; dx in dxv; adds to the sums.
+__device__ __forceinline__ float update_bwd_point(const UpdBwdArgs &a, const float *wr, float bv, const float *wn,
+                                                  const float *qr, float xr, float xt, float go, float m, float *dwr,
+                                                  float &db, float &dxv)
+{
+    float dz = go;
+    if (a.act) {
+        float z = bv;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) z = fmaf(wr[i], wn[i], z);
+        z = fmaf(wr[3], xt, z);
+        dz = go * silu_grad(z);
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) dwr[i] = fmaf(dz, wn[i], dwr[i]);
+    dwr[3] = fmaf(dz, xt, dwr[3]);
+    db += dz;
+    float dxt = wr[3] * dz;
+    if (a.res_mode == CANON_RESIDUAL_MASKED) dxt += go;
+    dxt += qr[3];
+    dxv = a.tmask ? dxt * m : dxt;
+    if (a.res_mode == CANON_RESIDUAL_UNMASKED) dxv += go;
+    return dz;
+}
+
+__device__ __forceinline__ void store_partial_right(const UpdBwdArgs &a, float *pp, const float *dwr, float db)
+{
+    const int lead = 4 - a.W;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float v = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (i - lead == k) v = dwr[i];
+        pp[k] = v;
+    }
+    pp[4] = db;
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs a)
 {
@@ -976,17 +1029,16 @@ __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs 
     const uint32_t c = blockIdx.x * 256u + threadIdx.x;
     if (c >= a.C) return;
     const uint32_t g = blockIdx.y;
-    const int W = a.W, S = a.S;
-    const int first = S - (W - 1);          // state slot read by tap 0
-    float w[4] = {0, 0, 0, 0};
-    for (int k = 0; k < W; ++k) w[k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
-    const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
-    float dw[4] = {0, 0, 0, 0}, db = 0.0f;
+    const int S = a.S;
+    const int lead = 4 - a.W;               // window entries / taps below this index do not exist
+    float wr[4], bv;
+    load_taps_right<DT>(a, c, wr, bv);
+    float dwr[4] = {0, 0, 0, 0}, db = 0.0f;
     const uint32_t b_begin = g * a.group;
     const uint32_t b_stop = b_begin + a.group < a.B ? b_begin + a.group : a.B;
     for (uint32_t b0 = b_begin; b0 < b_stop; b0 += NB) {
         // every load of the NB entries first (nothing is stored in between, so they are in flight together)
-        float xr[NB], go[NB], m[NB], win[NB][4], q[NB][4];
+        float xr[NB], go[NB], m[NB], wn[NB][3], qr[NB][4];
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
             const uint32_t b = b0 + n < b_stop ? b0 + n : b_stop - 1u;
@@ -996,12 +1048,9 @@ __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs 
             const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
             const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                win[n][k] = k < W - 1 ? load1<DT>(a.state, so + (int64_t)(first + k) * a.s_ss) : 0.0f;
-                // q[k]: gradient of the updated state at slot first-1+k (what shifts into slot first+k, and the
-                // token's own slot S-1 for k = W-1)
-                const int j = first - 1 + k;
-                q[n][k] = (a.dso && k < W && j >= 0) ? load1<DT>(a.dso, qo + (int64_t)j * a.q_ss) : 0.0f;
+            for (int i = 0; i < 4; ++i) {
+                if (i < 3) wn[n][i] = i >= lead ? load1<DT>(a.state, so + (int64_t)(S - 3 + i) * a.s_ss) : 0.0f;
+                qr[n][i] = (a.dso && i >= lead && S - 4 + i >= 0) ? load1<DT>(a.dso, qo + (int64_t)(S - 4 + i) * a.q_ss) : 0.0f;
             }
         }
 #pragma unroll
@@ -1009,37 +1058,106 @@ __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs 
             const uint32_t b = b0 + n;
             if (b >= b_stop) break;
             const float xt = a.tmask ? mul_round<DT>(xr[n], m[n]) : xr[n];
-            float dz = go[n];
-            if (a.act) {
-                float z = bv;
-                for (int k = 0; k < W - 1; ++k) z = fmaf(w[k], win[n][k], z);
-                z = fmaf(w[W - 1], xt, z);
-                dz = go[n] * silu_grad(z);
-            }
-            for (int k = 0; k < W - 1; ++k) dw[k] = fmaf(dz, win[n][k], dw[k]);
-            dw[W - 1] = fmaf(dz, xt, dw[W - 1]);
-            db += dz;
-            float dxt = w[W - 1] * dz;
-            if (a.res_mode == CANON_RESIDUAL_MASKED) dxt += go[n];
-            dxt += q[n][W - 1];
-            float dxv = a.tmask ? dxt * m[n] : dxt;
-            if (a.res_mode == CANON_RESIDUAL_UNMASKED) dxv += go[n];
+            float dxv;
+            const float dz = update_bwd_point(a, wr, bv, wn[n], qr[n], xr[n], xt, go[n], m[n], dwr, db, dxv);
             store1<DT>(a.dx, (int64_t)b * a.d_sb + (int64_t)c * a.d_sc, dxv);
             if (a.ds) {
                 const int64_t ro = (int64_t)b * a.r_sb + (int64_t)c * a.r_sc;
                 const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
                 // slots no tap reads: the gradient of the updated state shifted by one
-                for (int j = 0; j < first; ++j)
+                for (int j = 0; j < S - 3 + lead; ++j)
                     store1<DT>(a.ds, ro + (int64_t)j * a.r_ss,
                                (a.dso && j >= 1) ? load1<DT>(a.dso, qo + (int64_t)(j - 1) * a.q_ss) : 0.0f);
-                for (int k = 0; k < W - 1; ++k)
-                    store1<DT>(a.ds, ro + (int64_t)(first + k) * a.r_ss, fmaf(w[k], dz, q[n][k]));
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    if (i >= lead) store1<DT>(a.ds, ro + (int64_t)(S - 3 + i) * a.r_ss, fmaf(wr[i], dz, qr[n][i]));
             }
         }
     }
+    if (a.partial) store_partial_right(a, a.partial + ((int64_t)g * a.C + c) * 5, dwr, db);
+}
+
+// The same for a contiguous [B, C, S] state (and state gradients), S = 3 or 4, channel-contiguous token / dout /
+// dx: a lane owns E adjacent channels (two of a 16-bit type, one fp32) whose state rows are ONE run of 12 or
+// 16 bytes, as in the forward kernel, so every access of a wave is a dense stretch read or written whole.
+template <int DT, int S>
+__global__ __launch_bounds__(256) void canon_update_bwd_vec_kernel(const UpdBwdArgs a)
+{
+    constexpr int NB = 4;                   // batch entries whose loads are requested together
+    constexpr int BY = Elem<DT>::bytes;
+    constexpr int E = upd_lane_channels(BY, S);
+    constexpr int ND = E * S * BY / 4;      // words of state per lane and batch entry
+    static_assert(E * BY == 4 && (S == 3 || S == 4), "one word of token / dout / dx per lane");
+    const uint32_t cv = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t c0 = cv * E;
+    if (c0 >= a.C) return;
+    const uint32_t g = blockIdx.y;
+    const int lead = 4 - a.W;
+    float wr[E][4], bv[E], dwr[E][4], db[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        load_taps_right<DT>(a, c0 + e, wr[e], bv[e]);
+        db[e] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dwr[e][i] = 0.0f;
+    }
+    const uint32_t b_begin = g * a.group;
+    const uint32_t b_stop = b_begin + a.group < a.B ? b_begin + a.group : a.B;
+    for (uint32_t b0 = b_begin; b0 < b_stop; b0 += NB) {
+        uint32_t X[NB], G[NB], ST[NB][ND], Q[NB][ND];
+        float m[NB];
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = b0 + n < b_stop ? b0 + n : b_stop - 1u;
+            X[n] = *(const uint32_t *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
+            G[n] = *(const uint32_t *)(a.dy + ((int64_t)b * a.g_sb + c0) * BY);
+            load_words<ND>(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
+            if (a.dso) {
+                load_words<ND>(a.dso + ((int64_t)b * a.q_sb + (int64_t)c0 * S) * BY, Q[n]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < ND; ++i) Q[n][i] = 0u;
+            }
+            m[n] = a.tmask ? load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype) : 1.0f;
+        }
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = b0 + n;
+            if (b >= b_stop) break;
+            uint32_t ox = 0u, DS[ND];
+#pragma unroll
+            for (int i = 0; i < ND; ++i) DS[i] = 0u;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const float xr = Packed<DT>::as_float(Packed<DT>::get(&X[n], e));
+                const float go = Packed<DT>::as_float(Packed<DT>::get(&G[n], e));
+                const float xt = a.tmask ? mul_round<DT>(xr, m[n]) : xr;
+                float wn[3], qr[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (i < 3) wn[i] = i >= lead ? Packed<DT>::as_float(Packed<DT>::get(ST[n], e * S + S - 3 + i)) : 0.0f;
+                    qr[i] = (i >= lead && S - 4 + i >= 0) ? Packed<DT>::as_float(Packed<DT>::get(Q[n], e * S + (S - 4 + i >= 0 ? S - 4 + i : 0))) : 0.0f;
+                }
+                float dxv;
+                const float dz = update_bwd_point(a, wr[e], bv[e], wn, qr, xr, xt, go, m[n], dwr[e], db[e], dxv);
+                Packed<DT>::put(&ox, e, Packed<DT>::raw_of(dxv));
+                // slots no tap reads: the gradient of the updated state shifted by one (raw bits); the others
+                // add their tap's share
+#pragma unroll
+                for (int j = 0; j < S; ++j) {
+                    const int i = j - (S - 3);
+                    uint32_t raw = j >= 1 ? Packed<DT>::get(Q[n], e * S + (j >= 1 ? j - 1 : 0)) : 0u;
+                    if (i >= 0 && i >= lead) raw = Packed<DT>::raw_of(fmaf(wr[e][i >= 0 ? i : 0], dz, qr[i >= 0 ? i : 0]));
+                    Packed<DT>::put(DS, e * S + j, raw);
+                }
+            }
+            *(uint32_t *)(a.dx + ((int64_t)b * a.d_sb + c0) * BY) = ox;
+            if (a.ds) store_words<ND>(a.ds + ((int64_t)b * a.r_sb + (int64_t)c0 * S) * BY, DS);
+        }
+    }
     if (a.partial) {
-        float *pp = a.partial + ((int64_t)g * a.C + c) * 5;
-        pp[0] = dw[0]; pp[1] = dw[1]; pp[2] = dw[2]; pp[3] = dw[3]; pp[4] = db;
+#pragma unroll
+        for (int e = 0; e < E; ++e) store_partial_right(a, a.partial + ((int64_t)g * a.C + c0 + e) * 5, dwr[e], db[e]);
     }
 }
 
@@ -1094,10 +1212,28 @@ void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s)
 void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s)
 {
     const dim3 g(pl.grid_c, pl.args.ngroups), b(256);
-    switch (x_dtype) {
-    case CANON_DTYPE_F32: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F32>), g, b, 0, s, pl.args); break;
-    case CANON_DTYPE_BF16: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_BF16>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F16>), g, b, 0, s, pl.args); break;
+    if (pl.vec) {
+        const bool s3 = pl.args.S == 3;
+        switch (x_dtype) {
+        case CANON_DTYPE_F32:
+            if (s3) hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_F32, 3>), g, b, 0, s, pl.args);
+            else hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_F32, 4>), g, b, 0, s, pl.args);
+            break;
+        case CANON_DTYPE_BF16:
+            if (s3) hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_BF16, 3>), g, b, 0, s, pl.args);
+            else hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_BF16, 4>), g, b, 0, s, pl.args);
+            break;
+        default:
+            if (s3) hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_F16, 3>), g, b, 0, s, pl.args);
+            else hipLaunchKernelGGL((canon_update_bwd_vec_kernel<CANON_DTYPE_F16, 4>), g, b, 0, s, pl.args);
+            break;
+        }
+    } else {
+        switch (x_dtype) {
+        case CANON_DTYPE_F32: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F32>), g, b, 0, s, pl.args); break;
+        case CANON_DTYPE_BF16: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_BF16>), g, b, 0, s, pl.args); break;
+        default: hipLaunchKernelGGL((canon_update_bwd_kernel<CANON_DTYPE_F16>), g, b, 0, s, pl.args); break;
+        }
     }
     if (pl.args.partial)
         hipLaunchKernelGGL(canon_bwd_reduce_kernel, dim3((pl.args.C * 5u + 31u) / 32u), dim3(256), 0, s, pl.args.partial,

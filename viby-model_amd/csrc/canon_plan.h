@@ -233,6 +233,7 @@ struct BwdPlan {
 };
 
 struct UpdBwdPlan {
+    bool vec;               // contiguous states of 3 or 4 slots, channel-contiguous token: dense 4 / 12 / 16-byte lanes
     UpdBwdArgs args;
     uint32_t grid_c;        // blocks along the channels (0: nothing to launch)
     int64_t workspace_bytes;

@@ -106,6 +106,42 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True):
     return ms, plan
 
 
+def bench_ragged(layout, steps, warmup, nbuf, batch=32):
+    """configs[2]: right-padded batch of 32, valid lengths uniform in [128, 1024], the padding mask multiplied
+    in before the conv and the masked residual added (out = m*x + conv(m*x) + bias).  The mask is what the
+    Python wrapper hands the kernel for a trainer's int64 mask on a problem of this size: narrowed to bf16."""
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(4)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    lens = torch.randint(128, L + 1, (batch,), generator=g, device=dev)
+    mask = (torch.arange(L, device=dev)[None, :] < lens[:, None]).to(torch.bfloat16)
+    keep, refs = [], []
+    for _ in range(nbuf):
+        if layout == "bcl":
+            x = torch.randn(batch, C, L, generator=g, device=dev).bfloat16()
+        else:
+            x = torch.randn(batch, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        o = torch.empty_like(x)
+        p = cc._fill_fwd(x, o, w, bias, mask, None, None, 0, 1, 0)
+        keep.append((x, o, p))
+        refs.append(ctypes.byref(p))
+    fwd = _lib.lib().canon_conv1d_fwd
+    plan = _lib.lib().canon_conv1d_fwd_plan(refs[0]).decode()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step(i):
+        rc = fwd(refs[i % nbuf], stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_fwd")
+
+    ms = time_region(step, steps, warmup)
+    return ms, plan, prefill_bytes(batch, C, L) + batch * L * 2
+
+
 def bench_copy(steps, warmup, nbuf):
     """What the runtime's own device-to-device copy of one x-sized buffer reaches on this GPU with the
     same buffer rotation: the same bytes as a kernel that reads x once and writes out once."""
@@ -328,6 +364,9 @@ def main():
     ms_copy = bench_copy(args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
     ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
+    rag_steps, rag_warm = max(20, args.steps // 4), max(4, args.warmup // 4)
+    ms_rag, plan_rag, rag_bytes = bench_ragged("blc", rag_steps, rag_warm, 3)     # 3 x 453 MB between reuses
+    ms_rag_t, plan_rag_t, _ = bench_ragged("bcl", rag_steps, rag_warm, 3)
     dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
@@ -353,6 +392,13 @@ def main():
         "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",
                                        "kernel": plan_parts, "ms_per_step": round(ms_parts, 6),
                                        "GB/s": round(nbytes / (ms_parts * 1e-3) / 1e9, 1)},
+        "ragged_prefill_B32": {"workload": "configs[2]: bf16 x[32,3456,1024] right-padded, lengths U[128,1024], bf16 "
+                                           "padding mask multiplied in, masked residual fused; rate over all "
+                                           "B*C*L elements (the padded ones are read and written too)",
+                               "channel_last": {"kernel": plan_rag, "ms_per_step": round(ms_rag, 6),
+                                                "GB/s": round(rag_bytes / (ms_rag * 1e-3) / 1e9, 1)},
+                               "time_contiguous": {"kernel": plan_rag_t, "ms_per_step": round(ms_rag_t, 6),
+                                                   "GB/s": round(rag_bytes / (ms_rag_t * 1e-3) / 1e9, 1)}},
         "decode": {"workload": f"configs[3]: bf16 state[{DEC_B},{C},{DEC_S}], {DEC_STEPS} carried steps",
                    "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
                    "us_per_step_hipgraph": round(dec_graph_us, 3),

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 5
+#define CANON_CONV1D_ABI_VERSION 6
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -171,7 +171,7 @@ typedef struct canon_conv1d_update_params {
 } canon_conv1d_update_params;
 
 /*
- * Backward of canon_conv1d_fwd (final_state carries no gradient): the gradient a
+ * Backward of canon_conv1d_fwd: the gradient a
  * training step needs so that the fused forward can stay on the accelerated
  * path (trainer/base_trainer.py:274 calls backward through every Canon
  * layer).  Same role as the reference's own backward kernels
@@ -228,6 +228,13 @@ typedef struct canon_conv1d_bwd_params {
     void *dinitial_state;           /* [batch, channels, initial_len] in x_dtype, or NULL: receives the gradient w.r.t.
                                        initial_state (zero for entries older than W-1); needs initial_state */
     int64_t dinit_stride_b, dinit_stride_c, dinit_stride_s;
+    const void *dfinal_state;       /* [batch, channels, final_len] in x_dtype, or NULL: the gradient that arrives through
+                                       the forward's final_state (the last final_len entries of initial_state ++ xm):
+                                       added to dxm of the last steps and, where the state reaches back before t = 0,
+                                       to dinitial_state.  Such calls take the strided kernel. */
+    int64_t dfinal_stride_b, dfinal_stride_c, dfinal_stride_s;
+    int32_t final_len;              /* >= 1 when dfinal_state != NULL */
+    int32_t reserved2;
 } canon_conv1d_bwd_params;
 
 /*

@@ -41,11 +41,14 @@ import torch.nn.functional as F
 
 def conv1d_grads(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], dout: torch.Tensor,
                  mask: Optional[torch.Tensor] = None, activation=None, residual=0,
-                 seq_idx: Optional[torch.Tensor] = None, initial_states: Optional[torch.Tensor] = None):
+                 seq_idx: Optional[torch.Tensor] = None, initial_states: Optional[torch.Tensor] = None,
+                 dfinal: Optional[torch.Tensor] = None):
     """x, dout logical [B, C, L]; weight [C, W] and bias [C] are first rounded to x.dtype, as the
     forward does.  Returns (dx, dweight, dbias, out) in float64; with ``initial_states`` [B, C, S >= W-1]
     (the inputs before t = 0 instead of the zero padding, unmasked: the chunked continuation of
-    model/model.py:647-659) also their gradient as a fifth entry."""
+    model/model.py:647-659) also their gradient as a fifth entry.  ``dfinal`` [B, C, S_out]: a gradient arriving
+    through the captured state (the last S_out entries of initial_states ++ xm, zero filled on the left,
+    model/model.py:470-489); the loss differentiated is then sum(out * dout) + sum(final * dfinal)."""
     C, W = weight.shape
     x64 = x.detach().cpu().double().requires_grad_(True)
     w64 = weight.detach().cpu().to(x.dtype).double().requires_grad_(True)
@@ -73,7 +76,14 @@ def conv1d_grads(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
         y = y + xm
     elif residual in (2, "unmasked"):
         y = y + x64
-    y.backward(dout.detach().cpu().double())
+    loss = (y * dout.detach().cpu().double()).sum()
+    if dfinal is not None:
+        assert seq_idx is None
+        S_out = dfinal.shape[2]
+        hist = xm if h64 is None else torch.cat([h64, xm], dim=2)
+        final = F.pad(hist, (S_out, 0))[:, :, -S_out:]
+        loss = loss + (final * dfinal.detach().cpu().double()).sum()
+    loss.backward()
     if h64 is not None:
         return x64.grad, w64.grad, (b64.grad if b64 is not None else None), y.detach(), h64.grad
     return x64.grad, w64.grad, (b64.grad if b64 is not None else None), y.detach()

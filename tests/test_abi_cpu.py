@@ -318,8 +318,11 @@ def test_bwd_plan_and_workspace():
     # an initial state: the walk kernel reads the history; its checks
     q = bwd_params(initial_state=FAKE_X + 0x800000, initial_len=3, init_stride_b=3456 * 3, init_stride_c=3, init_stride_s=1)
     assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == b"bwd_generic"
+    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(dfinal_state=FAKE_X + 0x900000, final_len=4))) == b"bwd_generic"
     for over, msg in [(dict(initial_state=FAKE_X, initial_len=2), "shorter than width-1"),
                       (dict(dinitial_state=FAKE_X), "needs initial_state"),
+                      (dict(dfinal_state=FAKE_X, final_len=0), "final_len 0"),
+                      (dict(dfinal_state=FAKE_X, final_len=4, seq_idx=FAKE_X + 0x400000), "seq_idx"),
                       (dict(initial_state=FAKE_X, initial_len=3, seq_idx=FAKE_X + 0x400000), "seq_idx")]:
         assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(**over))) == -1, over
         assert msg in last_error(), (over, last_error())

@@ -227,7 +227,7 @@ def test_unsupported_gradients_raise(cc):
     with pytest.raises(NotImplementedError, match="backward of the decode step"):
         cc.causal_conv1d_update_parts([x[:, :4, 0], x[:, 4:, 0]], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
-    assert out.requires_grad and not fs.requires_grad
+    assert out.requires_grad and fs.requires_grad          # the captured state is differentiable
 
 
 def test_backward_more_than_2_31_elements(cc):
@@ -431,3 +431,64 @@ def test_backward_through_initial_states(cc, dtype, layout):
     cc.causal_conv1d_fn(torch.randn(2, 8, 6, device=DEV), w, initial_states=ig).sum().backward()
     want = torch.stack([w[:, 0], w[:, 0] + w[:, 1], w[:, 0] + w[:, 1] + w[:, 2]], dim=1).expand(2, 8, 3)
     assert torch.allclose(ig.grad, want, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layout", ["bcl", "blc"])
+def test_backward_through_final_states(cc, dtype, layout):
+    """A gradient that arrives through the captured final state (model/model.py:470-489 keeps the last
+    inputs for the next call) reaches x, and initial_states where the state is longer than the row."""
+    torch.manual_seed(23)
+    for (B, C, L, S_in, S_out), act, residual, masked in itertools.product(
+            [(2, 24, 40, 0, 4), (2, 24, 2, 3, 8), (3, 16, 5, 4, 3), (2, 16, 300, 0, 8), (2, 24, 1, 8, 4)],
+            [None, "silu"], [False, True], [False, True]):
+        W = 4
+        x = torch.randn(B, C, L).to(dtype)
+        w, b = (torch.randn(C, W) * 0.5).to(dtype), (torch.randn(C) * 0.1).to(dtype)
+        init = torch.randn(B, C, S_in).to(dtype) if S_in else None
+        dout, dfin = torch.randn(B, C, L).to(dtype), torch.randn(B, C, S_out).to(dtype)
+        mask = (torch.rand(B, L) > 0.3).to(torch.int64) if masked else None
+        xg, dg = x.to(DEV), dout.to(DEV)
+        if layout == "blc":
+            xg = xg.transpose(1, 2).contiguous().transpose(1, 2)
+            dg = dg.transpose(1, 2).contiguous().transpose(1, 2)
+        xg.requires_grad_(True)
+        wg, bg = w.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+        ig = init.to(DEV).requires_grad_(True) if S_in else None
+        out, fs = cc.causal_conv1d_fn(xg, wg, bg, activation=act, initial_states=ig, residual=residual,
+                                      attention_mask=None if mask is None else mask.to(DEV),
+                                      final_states_out=torch.empty(B, C, S_out, dtype=dtype, device=DEV))
+        ((out.float() * dg.float()).sum() + (fs.float() * dfin.to(DEV).float()).sum()).backward()
+        torch.cuda.synchronize()
+        want = conv1d_grads(x, w, b, dout, mask=mask, activation=act, residual=residual, initial_states=init,
+                            dfinal=dfin)
+        tag = f"{dtype} {layout} B{B} C{C} L{L} S_in{S_in} S_out{S_out} act={act} res={residual} mask={masked}"
+        check(xg.grad, want[0], dtype, "dx " + tag)
+        if S_in:
+            check(ig.grad, want[4], dtype, "dinit " + tag)
+        check(wg.grad, want[1], dtype, "dweight " + tag, sum_terms=B * L)
+        check(bg.grad, want[2], dtype, "dbias " + tag, sum_terms=B * L)
+
+
+def test_block_in_two_chunks_trains_like_the_block_in_one_go(cc):
+    """Prefill of a first chunk with state capture, the second chunk continued from that state: the gradient
+    flows through the state, so x, weight and bias get the gradients of the single call over both chunks."""
+    torch.manual_seed(29)
+    B, C, L1, L2, S = 2, 48, 37, 21, 4
+    x = torch.randn(B, C, L1 + L2, device=DEV)
+    w, b = torch.randn(C, 4, device=DEV) * 0.5, torch.randn(C, device=DEV) * 0.1
+    dout = torch.randn(B, C, L1 + L2, device=DEV)
+    mask = (torch.rand(B, L1 + L2, device=DEV) > 0.2).to(torch.int64)
+
+    x1, w1, b1 = x.clone().requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    cc.causal_conv1d_fn(x1, w1, b1, activation="silu", attention_mask=mask, residual=True).backward(dout)
+
+    x2, w2, b2 = x.clone().requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    o1, state = cc.causal_conv1d_fn(x2[:, :, :L1], w2, b2, activation="silu", attention_mask=mask[:, :L1],
+                                    residual=True, final_states_out=torch.empty(B, C, S, device=DEV))
+    o2 = cc.causal_conv1d_fn(x2[:, :, L1:], w2, b2, activation="silu", attention_mask=mask[:, L1:], residual=True,
+                             initial_states=state)
+    torch.cat([o1, o2], dim=2).backward(dout)
+    torch.cuda.synchronize()
+    for got, ref, tol in ((x2.grad, x1.grad, 2e-5), (w2.grad, w1.grad, 1e-4), (b2.grad, b1.grad, 1e-4)):
+        assert (got - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1e-30)

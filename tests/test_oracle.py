@@ -539,6 +539,10 @@ def test_gradient_oracle_with_initial_states_equals_the_block_in_one_go():
         back = torch.zeros_like(first[0])
         back[:, :, L1 - n:] = second[4][:, :, S - n:] * (1.0 if m1 is None else m1[:, L1 - n:].unsqueeze(1))
         assert torch.allclose(torch.cat([first[0] + back, second[0]], dim=2), whole[0], atol=1e-11), (W, S, act, res)
+        # ... which is what the oracle does itself when handed the state's gradient as dfinal
+        chained = conv1d_grads(x[:, :, :L1], w, b, dout[:, :, :L1], mask=m1, activation=act, residual=res, dfinal=second[4])
+        assert torch.allclose(chained[0], first[0] + back, atol=1e-11), (W, S, act, res, "dfinal")
+        assert torch.allclose(chained[1], first[1], atol=1e-11) and torch.allclose(chained[3], first[3], atol=1e-12)
         assert torch.allclose(first[1] + second[1], whole[1], atol=1e-11)
         assert torch.allclose(first[2] + second[2], whole[2], atol=1e-11)
         assert float(second[4][:, :, :S - (W - 1)].abs().max()) == 0.0 if S > W - 1 else True

@@ -348,14 +348,19 @@ class _CanonConvFn(torch.autograd.Function):
         out = _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx)
         ctx.save_for_backward(x, weight, bias, mask, seq_idx, initial_states)
         ctx.flags = (act, res)
+        ctx.set_materialize_grads(False)
         if final_states is not None:
-            ctx.mark_non_differentiable(final_states)
+            # filled in place and differentiable: a gradient that arrives through the captured state (the next
+            # chunk's initial_states, a decode step reading the cache) flows back into this call's inputs
+            ctx.mark_dirty(final_states)
             return out, final_states
         return out
 
     @staticmethod
-    def backward(ctx, dout, *unused):
+    def backward(ctx, dout, dfinal=None):
         x, weight, bias, mask, seq_idx, initial_states = ctx.saved_tensors
+        if dout is None:
+            dout = torch.zeros_like(x)
         act, res = ctx.flags
         channels, width = weight.shape
         dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
@@ -363,13 +368,13 @@ class _CanonConvFn(torch.autograd.Function):
         dinit = None
         if initial_states is not None and ctx.needs_input_grad[9]:
             dinit = torch.empty_like(initial_states)
-        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx, initial_states, dinit)
+        dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx, initial_states, dinit, dfinal)
         return (dx, dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
                 None, None, None, None, None, None, dinit)
 
 
 def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=None, initial_states=None,
-                dinit=None) -> torch.Tensor:
+                dinit=None, dfinal=None) -> torch.Tensor:
     """One backward launch (+ the fixed-order reduction): returns dx with x's strides and fills the
     fp32 ``dweight`` (channels, W) / ``dbias`` (channels,) given (rows of larger tensors are fine)."""
     if dout.dtype != x.dtype:
@@ -411,6 +416,12 @@ def _launch_bwd(x, dout, weight, bias, mask, dweight, dbias, act, res, seq_idx=N
             else:
                 p.dinitial_state = dinit.data_ptr()
                 p.dinit_stride_b, p.dinit_stride_c, p.dinit_stride_s = dinit.stride()
+    if dfinal is not None and x.numel():
+        if dfinal.dtype != x.dtype:
+            dfinal = dfinal.to(x.dtype)
+        p.dfinal_state = dfinal.data_ptr()
+        p.dfinal_stride_b, p.dfinal_stride_c, p.dfinal_stride_s = dfinal.stride()
+        p.final_len = dfinal.shape[2]
     p.dweight = dweight.data_ptr()
     p.dbias = dbias.data_ptr() if dbias is not None else None
     L = _lib.lib()

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -80,6 +80,8 @@ class BwdParams(ctypes.Structure):
         ("initial_state", _vp), ("init_stride_b", _i64), ("init_stride_c", _i64), ("init_stride_s", _i64),
         ("initial_len", _i32), ("reserved1", _i32),
         ("dinitial_state", _vp), ("dinit_stride_b", _i64), ("dinit_stride_c", _i64), ("dinit_stride_s", _i64),
+        ("dfinal_state", _vp), ("dfinal_stride_b", _i64), ("dfinal_stride_c", _i64), ("dfinal_stride_s", _i64),
+        ("final_len", _i32), ("reserved2", _i32),
     ]
 
 

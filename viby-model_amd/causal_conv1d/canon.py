@@ -35,8 +35,8 @@ Training: a block call without a cache is differentiable (fused backward
 kernel), and so are a prefill with state capture and the single-token step
 of ``forward`` (its own backward kernel; the cache tensor then carries the
 graph from step to step) and the chunked continuation of ``forward``
-(``initial_states``; the captured state itself carries no gradient, so the
-graph is cut at chunk boundaries).  The cached paths of ``forward_parts`` are
+(``initial_states``; the captured state is differentiable, so the graph
+continues across chunk boundaries and into the decode steps).  The cached paths of ``forward_parts`` are
 inference paths: run them under ``torch.no_grad()`` /
 ``torch.inference_mode()``.
 """

@@ -456,6 +456,10 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
         return fail(CANON_ERR_INVALID_ARGUMENT, "initial_len %d is shorter than width-1 = %d", p->initial_len, p->width - 1);
     if (p->dinitial_state && !p->initial_state)
         return fail(CANON_ERR_INVALID_ARGUMENT, "dinitial_state needs initial_state");
+    if (p->dfinal_state && p->seq_idx)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "dfinal_state cannot be combined with seq_idx");
+    if (p->dfinal_state && p->final_len < 1)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "final_len %d must be at least 1 with dfinal_state", p->final_len);
     const bool empty = p->batch == 0 || p->channels == 0 || p->seqlen == 0;
     if (empty && p->dinitial_state && p->batch > 0 && p->channels > 0)
         return fail(CANON_ERR_UNSUPPORTED, "dinitial_state of an empty input (it is all zeros) is left to the caller");
@@ -483,6 +487,8 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.i_sb = p->init_stride_b; a.i_sc = p->init_stride_c; a.i_ss = p->init_stride_s;
     a.j_sb = p->dinit_stride_b; a.j_sc = p->dinit_stride_c; a.j_ss = p->dinit_stride_s;
     a.S_in = p->initial_state ? p->initial_len : 0;
+    a.dfin = (const char *)p->dfinal_state; a.S_out = p->dfinal_state ? p->final_len : 0;
+    a.k_sb = p->dfinal_stride_b; a.k_sc = p->dfinal_stride_c; a.k_ss = p->dfinal_stride_s;
     a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels; a.L = (uint32_t)p->seqlen;
     a.W = p->width; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode;
@@ -498,7 +504,7 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
     // packed sequences and an initial state: only the walk kernel gates taps by sequence index / reads the history
-    const bool packed = p->seq_idx != nullptr || p->initial_state != nullptr;
+    const bool packed = p->seq_idx != nullptr || p->initial_state != nullptr || p->dfinal_state != nullptr;
     const bool rows = !packed && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
                       a.d_sb % E == 0 && a.d_sc % E == 0;

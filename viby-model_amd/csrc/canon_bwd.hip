@@ -212,6 +212,10 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 #pragma unroll
                 for (int e = 0; e < E; ++e) o[e] += g[e];
             }
+            if (a.dfin && t >= (int64_t)a.L - a.S_out) {
+                // this step's masked input was captured into slot t - (L - S_out) of the final state
+                o[0] += load1<DT>(a.dfin + ((int64_t)b * a.k_sb + (int64_t)c0 * a.k_sc + (t - ((int64_t)a.L - a.S_out)) * a.k_ss) * BY, 0);
+            }
             if constexpr (MASK) {
 #pragma unroll
                 for (int e = 0; e < E; ++e) o[e] *= mk[r];
@@ -251,6 +255,10 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
                 const int k = W - 1 - d - i;
                 if (k >= 0) acc = fmaf(w[0][k], dzf[i][0], acc);
             }
+            // a final state longer than the row also captured this entry (input at t = -d) in slot S_out - L - d
+            const int64_t slot = (int64_t)a.S_out - (int64_t)a.L - d;
+            if (a.dfin && slot >= 0)
+                acc += load1<DT>(a.dfin + ((int64_t)b * a.k_sb + (int64_t)c0 * a.k_sc + slot * a.k_ss) * BY, 0);
             store1<DT>(jb + (int64_t)s * a.j_ss * BY, 0, acc);
         }
     }

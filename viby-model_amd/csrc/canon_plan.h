@@ -114,8 +114,9 @@ struct BwdArgs {
     int64_t q_sb, q_sl;
     const char *init;     // inputs before t = 0, [B, C, S_in], or nullptr (walk kernel only)
     char *dinit;          // their gradient, or nullptr
-    int64_t i_sb, i_sc, i_ss, j_sb, j_sc, j_ss;
-    int32_t S_in;
+    const char *dfin;     // gradient of the captured final state [B, C, S_out], or nullptr (walk kernel only)
+    int64_t i_sb, i_sc, i_ss, j_sb, j_sc, j_ss, k_sb, k_sc, k_ss;
+    int32_t S_in, S_out;
     int64_t x_sb, x_sc, x_sl;
     int64_t g_sb, g_sc, g_sl;
     int64_t d_sb, d_sc, d_sl;

@@ -686,18 +686,31 @@ int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, b
                     dense_token(p->x, a.x_sb, a.x_sc) && dense_token(p->dout, a.g_sb, a.g_sc) &&
                     dense_token(p->dx, a.d_sb, a.d_sc) && dense_state(p->conv_state, a.s_sb, a.s_sc, a.s_ss) &&
                     dense_state(p->dstate_out, a.q_sb, a.q_sc, a.q_ss) && dense_state(p->dstate, a.r_sb, a.r_sc, a.r_ss)));
-    // batch entries per thread: enough groups for about four blocks per compute unit, at most 1024 groups
-    // (counted on the channels alone, so that the scratch size does not depend on the kernel chosen)
-    const uint32_t grid_c = (plan->vec ? a.C / E + 255u : a.C + 255u) / 256u;
+    // Batch groups.  One channel per thread: enough groups for about four blocks per compute unit, at most 1024.
+    // Vector kernel: the four waves of a block split a group, four entries each per round, so a group is 16
+    // entries unless that leaves fewer blocks than compute units (measured at B256 C3456 bf16: groups of 16 / 8 / 4
+    // entries 8.4 / 9.6 / 13.4 us).  The scratch is sized for whichever needs more, so
+    // that its size does not depend on the pointers' alignment.
     const uint32_t cblocks = (a.C + 255u) / 256u;
     uint32_t want = (1024u + cblocks - 1u) / cblocks;
     if (want > 1024u) want = 1024u;
     if (want > a.B) want = a.B;
-    a.group = (a.B + want - 1u) / want;
-    a.ngroups = (a.B + a.group - 1u) / a.group;
-    plan->grid_c = grid_c;
+    const uint32_t group_s = (a.B + want - 1u) / want;
+    const uint32_t ngroups_s = (a.B + group_s - 1u) / group_s;
+    const uint32_t vblocks = (a.C / E + 63u) / 64u;
+    uint32_t group_v = 16u;
+    while (group_v > 4u && (uint64_t)vblocks * ((a.B + group_v - 1u) / group_v) < 256u) group_v /= 2u;
+    while ((a.B + group_v - 1u) / group_v > 65535u) group_v *= 2u;
+    const uint32_t ngroups_v = (a.B + group_v - 1u) / group_v;
+    if (plan->vec) {
+        a.group = group_v; a.ngroups = ngroups_v; plan->grid_c = vblocks;
+    } else {
+        a.group = group_s; a.ngroups = ngroups_s; plan->grid_c = cblocks;
+    }
+    if (a.ngroups > 65535u) return fail(CANON_ERR_UNSUPPORTED, "batch too large for the decode backward");
     if (p->dweight) {
-        plan->workspace_bytes = (int64_t)a.ngroups * a.C * 5 * (int64_t)sizeof(float);
+        const uint32_t most = ngroups_v > ngroups_s ? ngroups_v : ngroups_s;
+        plan->workspace_bytes = (int64_t)most * a.C * 5 * (int64_t)sizeof(float);
         a.partial = (float *)p->workspace;
         if (check_pointers && (!p->workspace || !aligned16(p->workspace) || p->workspace_bytes < plan->workspace_bytes))
             return fail(CANON_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned and at least %lld bytes (got %lld)",

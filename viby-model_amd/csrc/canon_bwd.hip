@@ -1088,6 +1088,9 @@ __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs 
 // The same for a contiguous [B, C, S] state (and state gradients), S = 3 or 4, channel-contiguous token / dout /
 // dx: a lane owns E adjacent channels (two of a 16-bit type, one fp32) whose state rows are ONE run of 12 or
 // 16 bytes, as in the forward kernel, so every access of a wave is a dense stretch read or written whole.
+// The four waves of a block share a 64-lane channel tile and take every fourth batch entry of the block's
+// group; their sums are added in wave order through LDS, so a group is 4 x as many entries (a quarter of the
+// partial sets) for the same work per wave.
 template <int DT, int S>
 __global__ __launch_bounds__(256) void canon_update_bwd_vec_kernel(const UpdBwdArgs a)
 {
@@ -1096,27 +1099,31 @@ __global__ __launch_bounds__(256) void canon_update_bwd_vec_kernel(const UpdBwdA
     constexpr int E = upd_lane_channels(BY, S);
     constexpr int ND = E * S * BY / 4;      // words of state per lane and batch entry
     static_assert(E * BY == 4 && (S == 3 || S == 4), "one word of token / dout / dx per lane");
-    const uint32_t cv = blockIdx.x * 256u + threadIdx.x;
+    __shared__ float sums[3][64][E * 5 + 1];   // waves 1..3 hand their sums to wave 0 (+1: no bank conflicts)
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    const uint32_t cv = blockIdx.x * 64u + lane;
     const uint32_t c0 = cv * E;
-    if (c0 >= a.C) return;
+    const bool live = c0 < a.C;
     const uint32_t g = blockIdx.y;
     const int lead = 4 - a.W;
     float wr[E][4], bv[E], dwr[E][4], db[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        load_taps_right<DT>(a, c0 + e, wr[e], bv[e]);
+        if (live) load_taps_right<DT>(a, c0 + e, wr[e], bv[e]);
         db[e] = 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) dwr[e][i] = 0.0f;
     }
     const uint32_t b_begin = g * a.group;
     const uint32_t b_stop = b_begin + a.group < a.B ? b_begin + a.group : a.B;
-    for (uint32_t b0 = b_begin; b0 < b_stop; b0 += NB) {
+    // this wave's entries: b_begin + wv, + 4, + 8, ...
+    for (uint32_t b0 = b_begin + wv; live && b0 < b_stop; b0 += 4u * NB) {
         uint32_t X[NB], G[NB], ST[NB][ND], Q[NB][ND];
         float m[NB];
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
-            const uint32_t b = b0 + n < b_stop ? b0 + n : b_stop - 1u;
+            const uint32_t bn = b0 + 4u * n;
+            const uint32_t b = bn < b_stop ? bn : b0;
             X[n] = *(const uint32_t *)(a.x + ((int64_t)b * a.x_sb + c0) * BY);
             G[n] = *(const uint32_t *)(a.dy + ((int64_t)b * a.g_sb + c0) * BY);
             load_words<ND>(a.state + ((int64_t)b * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
@@ -1130,7 +1137,7 @@ __global__ __launch_bounds__(256) void canon_update_bwd_vec_kernel(const UpdBwdA
         }
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
-            const uint32_t b = b0 + n;
+            const uint32_t b = b0 + 4u * n;
             if (b >= b_stop) break;
             uint32_t ox = 0u, DS[ND];
 #pragma unroll
@@ -1163,10 +1170,28 @@ __global__ __launch_bounds__(256) void canon_update_bwd_vec_kernel(const UpdBwdA
             if (a.ds) store_words<ND>(a.ds + ((int64_t)b * a.r_sb + (int64_t)c0 * S) * BY, DS);
         }
     }
-    if (a.partial) {
+    if (!a.partial) return;                 // uniform over the block
+    if (wv != 0) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) store_partial_right(a, a.partial + ((int64_t)g * a.C + c0 + e) * 5, dwr[e], db[e]);
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sums[wv - 1][lane][e * 5 + i] = dwr[e][i];
+            sums[wv - 1][lane][e * 5 + 4] = db[e];
+        }
     }
+    __syncthreads();
+    if (wv != 0 || !live) return;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {           // wave order: a fixed order of additions
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dwr[e][i] += sums[k][lane][e * 5 + i];
+            db[e] += sums[k][lane][e * 5 + 4];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) store_partial_right(a, a.partial + ((int64_t)g * a.C + c0 + e) * 5, dwr[e], db[e]);
 }
 
 // ---------------------------------------------------------------------------
@@ -1219,7 +1244,7 @@ void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s)
 
 void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s)
 {
-    const dim3 g(pl.grid_c, pl.args.ngroups), b(256);
+    const dim3 g(pl.grid_c, pl.args.ngroups), b(256);   // vec: 64 lanes of channels per block, else 256 channels
     if (pl.vec) {
         const bool s3 = pl.args.S == 3;
         switch (x_dtype) {

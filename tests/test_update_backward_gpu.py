@@ -220,3 +220,33 @@ def test_canon_layer_trains_through_single_token_steps(cc):
     torch.cuda.synchronize()
     for got, ref, tol in zip((xs.grad, layer.weight.grad, layer.bias_param.grad), want, (2e-5, 1e-4, 1e-4)):
         assert (got - ref).abs().max().item() <= tol * scale_of(ref)
+
+
+def test_canon_layer_prefill_then_steps_trains_like_the_block(cc):
+    """Prefill with state capture, a continued chunk, then single-token steps, all through the layer's cache
+    (model/model.py:470-489, 647-659, 270-317): the graph runs through the cached state, so inputs and
+    parameters get the gradients of one call over the whole block."""
+    import types
+    from causal_conv1d.canon import CanonLayer
+    torch.manual_seed(13)
+    B, D, T1, T2, T3 = 2, 128, 9, 5, 3
+    T = T1 + T2 + T3
+    cfg = types.SimpleNamespace(canon_kernel=4, canon_bias=True, canon_activation=True)
+    layer = CanonLayer(D, cfg, "a").to(DEV)
+    layer.reset_parameters()
+    x = torch.randn(B, T, D, device=DEV)
+    dout = torch.randn(B, T, D, device=DEV)
+
+    xb = x.clone().requires_grad_(True)
+    layer(xb).backward(dout)
+    want = (xb.grad.clone(), layer.weight.grad.clone(), layer.bias_param.grad.clone())
+    layer.zero_grad()
+
+    xs = x.clone().requires_grad_(True)
+    cache = types.SimpleNamespace()
+    ys = [layer(xs[:, :T1], cache=cache, layer_idx=0), layer(xs[:, T1:T1 + T2], cache=cache, layer_idx=0)]
+    ys += [layer(xs[:, t:t + 1], cache=cache, layer_idx=0) for t in range(T1 + T2, T)]
+    torch.cat(ys, dim=1).backward(dout)
+    torch.cuda.synchronize()
+    for got, ref, tol in zip((xs.grad, layer.weight.grad, layer.bias_param.grad), want, (2e-5, 1e-4, 1e-4)):
+        assert (got - ref).abs().max().item() <= tol * scale_of(ref)

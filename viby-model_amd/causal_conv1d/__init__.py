@@ -346,7 +346,10 @@ class _CanonConvFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, mask, final_states, act, res, rnd, seq_idx=None, initial_states=None):
         out = _launch_fwd(x, weight, bias, mask, initial_states, final_states, act, res, rnd, seq_idx)
-        ctx.save_for_backward(x, weight, bias, mask, seq_idx, initial_states)
+        # a copy of the (small) initial state: callers keep it in a cache tensor they overwrite right after
+        # the call (CanonLayer copies the new state into it, decode steps shift it in place)
+        ctx.save_for_backward(x, weight, bias, mask, seq_idx,
+                              initial_states.detach().clone() if initial_states is not None else None)
         ctx.flags = (act, res)
         ctx.set_materialize_grads(False)
         if final_states is not None:

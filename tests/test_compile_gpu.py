@@ -308,3 +308,34 @@ def test_compiled_training_through_the_multi_part_call(cc):
     outs_c, dx_c, dw_c = step(torch.compile(f, backend="aot_eager", fullgraph=True))
     for a, e in zip(outs_c + dx_c + [dw_c], outs_e + dx_e + [dw_e]):
         assert torch.equal(bits(a), bits(e))
+
+
+def test_compiled_training_through_the_captured_state(cc):
+    """A block processed as two chunks inside one traced function, the second continued from the state the
+    first captured: the traced operators pass the state's gradient on, as the eager calls do."""
+    torch.manual_seed(7)
+    B, C, L1, L2, S = 2, 64, 40, 24, 4
+    x0 = torch.randn(B, C, L1 + L2, device=DEV)
+    w0, b0 = torch.randn(C, 4, device=DEV) * 0.3, torch.randn(C, device=DEV) * 0.1
+    dout = torch.randn(B, C, L1 + L2, device=DEV)
+
+    def whole(x, w, b):
+        return cc.causal_conv1d_fn(x, w, b, activation="silu", residual=True)
+
+    def chunked(x, w, b):
+        o1, state = cc.causal_conv1d_fn(x[:, :, :L1], w, b, activation="silu", residual=True,
+                                        final_states_out=torch.empty(B, C, S, device=DEV))
+        o2 = cc.causal_conv1d_fn(x[:, :, L1:], w, b, activation="silu", residual=True, initial_states=state)
+        return torch.cat([o1, o2], dim=2)
+
+    def step(fn):
+        x, w, b = x0.clone().requires_grad_(), w0.clone().requires_grad_(), b0.clone().requires_grad_()
+        y = fn(x, w, b)
+        y.backward(dout)
+        return y.detach(), x.grad, w.grad, b.grad
+
+    want = step(whole)
+    for fn in (chunked, torch.compile(chunked, backend="aot_eager", fullgraph=True)):
+        got = step(fn)
+        for name, a, e, tol in zip(("y", "dx", "dweight", "dbias"), got, want, (1e-6, 2e-5, 1e-4, 1e-4)):
+            assert (a - e).abs().max().item() <= tol * (e.abs().max().item() + 1e-30), name

@@ -301,9 +301,6 @@ def causal_conv1d_fn(
         raise ValueError("cannot produce final states from an empty input")
 
     if torch.compiler.is_compiling():
-        if initial_states is not None and _wants_grad(x, weight, bias, initial_states):
-            raise NotImplementedError("gradients through a call with initial_states are not implemented under "
-                                      "torch.compile")
         # under torch.compile the launch is one opaque operator of the traced graph (trainer/train_pretrain.py:39
         # and eval_model.py:157 compile the whole model, the latter with fullgraph=True)
         result, fin = torch.ops.canon_conv1d.fwd(x, weight, bias, attention_mask, initial_states, seq_idx,
@@ -879,33 +876,43 @@ def _(x, weight, bias, mask, initial_states, seq_idx, state_len, act, res, rnd):
 
 @torch.library.custom_op("canon_conv1d::bwd", mutates_args=(), device_types="cuda")
 def _op_bwd(x: torch.Tensor, dout: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-            mask: Optional[torch.Tensor], seq_idx: Optional[torch.Tensor], act: int, res: int
-            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+            mask: Optional[torch.Tensor], seq_idx: Optional[torch.Tensor], initial_states: Optional[torch.Tensor],
+            dfinal: Optional[torch.Tensor], act: int, res: int
+            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     channels, width = weight.shape
     dweight = torch.empty(channels, width, dtype=torch.float32, device=x.device)
     dbias = torch.empty(channels if bias is not None else 0, dtype=torch.float32, device=x.device)
-    dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias if bias is not None else None, act, res, seq_idx)
-    return dx, dweight.to(weight.dtype), dbias.to(bias.dtype if bias is not None else weight.dtype)
+    dinit = torch.empty_like(initial_states) if initial_states is not None else x.new_empty((x.shape[0], channels, 0))
+    dx = _launch_bwd(x, dout, weight, bias, mask, dweight, dbias if bias is not None else None, act, res, seq_idx,
+                     initial_states, dinit if initial_states is not None else None, dfinal)
+    return dx, dweight.to(weight.dtype), dbias.to(bias.dtype if bias is not None else weight.dtype), dinit
 
 
 @_op_bwd.register_fake
-def _(x, dout, weight, bias, mask, seq_idx, act, res):
+def _(x, dout, weight, bias, mask, seq_idx, initial_states, dfinal, act, res):
     return (torch.empty_like(x), torch.empty_like(weight, memory_format=torch.contiguous_format),
             weight.new_empty((weight.shape[0] if bias is not None else 0,),
-                             dtype=bias.dtype if bias is not None else weight.dtype))
+                             dtype=bias.dtype if bias is not None else weight.dtype),
+            torch.empty_like(initial_states) if initial_states is not None
+            else x.new_empty((x.shape[0], weight.shape[0], 0)))
 
 
 def _op_fwd_setup(ctx, inputs, output):
-    x, weight, bias, mask, _initial, seq_idx, _state_len, act, res, _rnd = inputs
-    ctx.save_for_backward(x, weight, bias, mask, seq_idx)
-    ctx.flags = (act, res, bias is not None)
+    x, weight, bias, mask, initial, seq_idx, state_len, act, res, _rnd = inputs
+    ctx.save_for_backward(x, weight, bias, mask, seq_idx, initial)
+    ctx.flags = (act, res, bias is not None, state_len)
 
 
-def _op_fwd_backward(ctx, dout, _dstate):
-    x, weight, bias, mask, seq_idx = ctx.saved_tensors
-    act, res, has_bias = ctx.flags
-    dx, dweight, dbias = torch.ops.canon_conv1d.bwd(x, dout, weight, bias, mask, seq_idx, act, res)
-    return dx, dweight, (dbias if has_bias else None), None, None, None, None, None, None, None
+def _op_fwd_backward(ctx, dout, dstate):
+    x, weight, bias, mask, seq_idx, initial = ctx.saved_tensors
+    act, res, has_bias, state_len = ctx.flags
+    # the captured state is a result of the operator: whatever gradient reaches it is passed on (a traced graph
+    # cannot tell an unused state from one whose gradient happens to be zero)
+    dfinal = dstate if state_len > 0 else None
+    dx, dweight, dbias, dinit = torch.ops.canon_conv1d.bwd(x, dout, weight, bias, mask, seq_idx, initial, dfinal,
+                                                           act, res)
+    return (dx, dweight, (dbias if has_bias else None), None, (dinit if initial is not None else None),
+            None, None, None, None, None)
 
 
 _op_fwd.register_autograd(_op_fwd_backward, setup_context=_op_fwd_setup)
@@ -953,8 +960,8 @@ def _op_fwd_parts_backward(ctx, grads):
     dxs, dws, dbs, c0 = [], [], [], 0
     for x, dout in zip(xs, grads):
         c1 = c0 + x.shape[1]
-        dx, dw, db = torch.ops.canon_conv1d.bwd(x, dout, weight[c0:c1], bias[c0:c1] if has_bias else None,
-                                                mask, None, act, res)
+        dx, dw, db, _ = torch.ops.canon_conv1d.bwd(x, dout, weight[c0:c1], bias[c0:c1] if has_bias else None,
+                                                   mask, None, None, None, act, res)
         dxs.append(dx)
         dws.append(dw)
         dbs.append(db)

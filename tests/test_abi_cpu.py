@@ -464,9 +464,12 @@ def test_torch_operators_for_traced_graphs_have_shape_only_twins():
     assert y.shape == x.shape and y.stride() == x.stride() and y.dtype == x.dtype
     assert tuple(fin.shape) == (2, 16, 8) and fin.dtype == x.dtype
     assert tuple(ops.fwd(x, w, None, None, None, None, 0, 0, 0, 0)[1].shape) == (2, 16, 0)
-    dx, dw, db = ops.bwd(x, x, w, b, None, None, 0, 1)
+    dx, dw, db, di = ops.bwd(x, x, w, b, None, None, None, None, 0, 1)
+    assert tuple(di.shape) == (2, 16, 0)
+    init = torch.empty(2, 16, 3, dtype=x.dtype, device="meta")
+    assert tuple(ops.bwd(x, x, w, b, None, None, init, init, 0, 1)[3].shape) == (2, 16, 3)
     assert dx.stride() == x.stride() and tuple(dw.shape) == (16, 4) and dw.dtype == w.dtype and tuple(db.shape) == (16,)
-    assert tuple(ops.bwd(x, x, w, None, None, None, 0, 1)[2].shape) == (0,)
+    assert tuple(ops.bwd(x, x, w, None, None, None, None, None, 0, 1)[2].shape) == (0,)
     st = torch.empty(2, 16, 4, device="meta", dtype=torch.bfloat16)
     assert tuple(ops.update(x[:, :, 0], st, w, None, None, None, None, 0, 0, 0).shape) == (2, 16)
     outs = ops.fwd_parts([x[:, :12], x[:, 12:]], w, None, None, None, 3, 0, 0, 0)

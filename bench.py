@@ -230,6 +230,59 @@ def bench_decode(reps, warmup):
     return ms_eager * 1e3, ms_graph * 1e3, plan
 
 
+def bench_decode_backward(steps, warmup, nbuf=8):
+    """Backward of one decode step at the decode configuration (with SiLU, state gradients both ways):
+    token, saved state, dout and the updated state's gradient read; dx and the state's gradient written."""
+    import torch
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(5)
+    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
+    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    dw = torch.empty(C, W, dtype=torch.float32, device=dev)
+    db = torch.empty(C, dtype=torch.float32, device=dev)
+    L_ = _lib.lib()
+    keep, refs, ws = [], [], None
+    for _ in range(nbuf):
+        def t(*shape):
+            return torch.randn(*shape, generator=g, device=dev).bfloat16()
+        x, dout, dx = t(DEC_B, C), t(DEC_B, C), torch.empty(DEC_B, C, dtype=torch.bfloat16, device=dev)
+        st, dso = t(DEC_B, C, DEC_S), t(DEC_B, C, DEC_S)
+        ds = torch.empty_like(st)
+        p = _lib.UpdateBwdParams()
+        p.struct_size = ctypes.sizeof(_lib.UpdateBwdParams)
+        p.x_dtype = p.w_dtype = 1
+        p.width, p.activation, p.state_len = W, 1, DEC_S
+        p.batch, p.channels = DEC_B, C
+        for name, ten in (("x", x), ("dout", dout), ("dx", dx)):
+            setattr(p, name, ten.data_ptr())
+            setattr(p, name + "_stride_b", ten.stride(0))
+            setattr(p, name + "_stride_c", ten.stride(1))
+        p.conv_state = st.data_ptr()
+        p.state_stride_b, p.state_stride_c, p.state_stride_s = st.stride()
+        p.dstate_out = dso.data_ptr()
+        p.dstate_out_stride_b, p.dstate_out_stride_c, p.dstate_out_stride_s = dso.stride()
+        p.dstate = ds.data_ptr()
+        p.dstate_stride_b, p.dstate_stride_c, p.dstate_stride_s = ds.stride()
+        p.weight, p.w_stride_c, p.w_stride_k = w.data_ptr(), W, 1
+        p.bias, p.dweight, p.dbias = bias.data_ptr(), dw.data_ptr(), db.data_ptr()
+        if ws is None:
+            ws = torch.empty(L_.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(p)), dtype=torch.uint8, device=dev)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+        keep.append((x, dout, dx, st, dso, ds, p))
+        refs.append(ctypes.byref(p))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step(i):
+        rc = L_.canon_conv1d_update_bwd(refs[i % nbuf], stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_update_bwd")
+
+    ms = time_region(step, steps, warmup)
+    elems = DEC_B * C
+    return ms * 1e3, (3 * DEC_S + 3) * elems * 2, ws.numel()
+
+
 def bench_backward(steps, warmup, nbuf):
     """Backward of the same prefill step (channel-contiguous, as a training step through the model
     produces it): reads x and dout, writes dx, reduces dweight / dbias."""
@@ -370,6 +423,8 @@ def main():
     dec_us, dec_graph_us, dec_plan = bench_decode(max(4, args.steps // 20), 2)
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
+    us_dbwd, dbwd_bytes, ws_dbwd = bench_decode_backward(max(50, args.steps), max(5, args.warmup))
+
     nbytes = prefill_bytes(B, C, L)
     gbps = nbytes / (ms * 1e-3) / 1e9
     out = {
@@ -407,6 +462,10 @@ def main():
                                   "GB/s": round(1.5 * nbytes / (ms_bwd * 1e-3) / 1e9, 1),
                                   "bytes": "x and dout read, dx written (3 tensor passes)",
                                   "scratch_bytes": ws_bwd},
+        "decode_backward": {"workload": f"backward of one decode step, bf16 state[{DEC_B},{C},{DEC_S}], SiLU, state "
+                                        "gradients in and out; two launches (step kernel + fixed-order reduction)",
+                            "us_per_step": round(us_dbwd, 3),
+                            "GB/s": round(dbwd_bytes / (us_dbwd * 1e-6) / 1e9, 1), "scratch_bytes": ws_dbwd},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
     }

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 6
+#define CANON_CONV1D_ABI_VERSION 7
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -149,7 +149,7 @@ typedef struct canon_conv1d_update_params {
     int32_t residual_mode;
     int32_t round_mode;
     int32_t state_len;
-    int32_t reserved0;
+    int32_t state_rows;             /* with conv_state_indices: rows of the conv_state pool, or 0 (not stated) */
     int64_t batch, channels;
     const void *x;
     int64_t x_stride_b, x_stride_c;
@@ -166,8 +166,11 @@ typedef struct canon_conv1d_update_params {
                                             shifted; the token is written to slot cache_seqlens[b] % state_len and
                                             the W-1 slots before it (cyclically) are the history.  Strided kernel. */
     const int32_t *conv_state_indices;   /* [batch] or NULL.  Upstream's batch indirection: batch entry b uses row
-                                            conv_state_indices[b] of conv_state (a state pool of any number of rows;
-                                            the caller guarantees the indices are valid and distinct). */
+                                            conv_state_indices[b] of conv_state (a state pool of state_rows rows; the
+                                            caller guarantees that the indices are distinct).  An entry whose index is
+                                            negative, or not below state_rows when that is stated, is skipped: neither
+                                            its state row nor its row of out is read or written (upstream's padding
+                                            slots). */
 } canon_conv1d_update_params;
 
 /*

@@ -28,7 +28,10 @@ def assert_parity(got: torch.Tensor, want: torch.Tensor, exact: bool, what: str 
     got, want = got.detach().cpu(), want.detach().cpu()
     assert got.shape == want.shape and got.dtype == want.dtype, (what, got.shape, want.shape)
     if exact:
-        assert torch.equal(bits(got), bits(want)), f"{what}: not bit exact"
+        diff = (bits(got) != bits(want)).nonzero()
+        first = tuple(diff[0].tolist()) if len(diff) else None
+        assert len(diff) == 0, (f"{what}: not bit exact: {len(diff)} of {got.numel()} elements differ, first at {first}: "
+                                f"got {got[first].item()!r}, want {want[first].item()!r}")
     elif got.dtype == torch.float32:
         scale = want.abs() if res is None else torch.maximum(want.abs(), res.detach().cpu().float().abs())
         err = (got - want).abs() / scale.clamp_min(1e-3)

@@ -102,10 +102,12 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     # as long as x and out share their strides
     assert plan(fwd_params(L=1023)) == "bcl_vec"
     assert plan(fwd_params(L=1023, out_stride_c=1024, out_stride_b=3456 * 1024)) == "generic"
-    # ragged channel counts, misaligned base pointers, eager rounding -> strided kernel
+    # ragged channel counts, misaligned base pointers -> strided kernel
     assert plan(fwd_params(C=3457, layout="blc")) == "generic"
     assert plan(fwd_params(x=FAKE_X + 2)) == "generic"
-    assert plan(fwd_params(round_mode=1)) == "generic"
+    # the eager module's rounding points are register arithmetic: the same kernels
+    assert plan(fwd_params(round_mode=1)) == "bcl_vec"
+    assert plan(fwd_params(round_mode=1, layout="blc")) == "blc_vec"
     # rows too short for a wave of their own: several rows per wave, as long as they are whole aligned vectors
     assert plan(fwd_params(L=64)) == "bcl_vec_short"
     assert plan(fwd_params(L=8)) == "bcl_vec_short"
@@ -115,7 +117,7 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     assert plan(fwd_params(L=255)) == "bcl_vec"                            # ... not whole vectors, but long enough
     assert plan(fwd_params(L=60)) == "generic"                             # ... not whole vectors
     assert plan(fwd_params(L=4)) == "generic"
-    assert plan(fwd_params(L=64, round_mode=1)) == "generic"
+    assert plan(fwd_params(L=64, round_mode=1)) == "bcl_vec_short"
     # strided but aligned rows (a channel slice of a bigger tensor) stay vectorised
     assert plan(fwd_params(C=128, x_stride_b=4096 * 1024, x_stride_c=1024)) == "bcl_vec"
 
@@ -187,7 +189,7 @@ def test_update_plan_and_validation():
     assert uplan(update_params(state_stride_b=3456 * 3 + 1)) == "update_generic"   # rows of a state pool off the grid
     assert uplan(update_params(state_stride_b=3456 * 3 + 2)) == "update_vec"
     assert uplan(update_params(state_stride_s=2, state_stride_c=6, state_stride_b=3456 * 6)) == "update_generic"
-    assert uplan(update_params(round_mode=1)) == "update_generic"
+    assert uplan(update_params(round_mode=1)) == "update_vec"        # eager rounding: the same kernel
     assert uplan(update_params(conv_state_indices=FAKE_STATE + 64)) == "update_vec"       # state pool: row indirection
     assert uplan(update_params(cache_seqlens=FAKE_STATE + 64)) == "update_generic"        # circular buffer
     for over, needle in [(dict(S=2), "state_len"), (dict(width=7), "width"),

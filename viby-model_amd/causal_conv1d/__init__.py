@@ -485,7 +485,9 @@ def causal_conv1d_update(
                 shifted; the token is written to slot ``cache_seqlens % state_len`` and the W-1
                 slots before it (cyclically) are the history.
     conv_state_indices  (batch,) int32: batch entry b uses row ``conv_state_indices[b]`` of
-                ``conv_state`` (a pool of any number of rows).
+                ``conv_state`` (a pool of any number of rows).  An entry whose index is negative
+                or not below the pool's size is skipped (upstream's padding slots): no state row
+                is touched and its output row is zero.
     token_mask  (batch,) multiplies the token before everything else
                 (``model/model.py:277-282``).
     residual    False | True ('masked': adds the masked token,
@@ -552,13 +554,16 @@ def causal_conv1d_update(
 
 
 def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
-    out = torch.empty(tuple(x2.shape), dtype=x2.dtype, device=x2.device)
+    # entries of a state pool whose index lies outside the pool are skipped by the kernel: their output rows are zeros
+    alloc = torch.empty if conv_state_indices is None else torch.zeros
+    out = alloc(tuple(x2.shape), dtype=x2.dtype, device=x2.device)
     if out.numel():
         p = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
         if cache_seqlens is not None:
             p.cache_seqlens = cache_seqlens.data_ptr()
         if conv_state_indices is not None:
             p.conv_state_indices = conv_state_indices.data_ptr()
+            p.state_rows = conv_state.shape[0]
         rc = _call(_lib.lib().canon_conv1d_update, x2.device, ctypes.byref(p))
         _lib.check(rc, "causal_conv1d_update")
     return out

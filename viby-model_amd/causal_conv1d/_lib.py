@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -50,7 +50,7 @@ class UpdateParams(ctypes.Structure):
         ("struct_size", _u32),
         ("x_dtype", _i32), ("w_dtype", _i32), ("mask_dtype", _i32),
         ("width", _i32), ("activation", _i32), ("residual_mode", _i32), ("round_mode", _i32),
-        ("state_len", _i32), ("reserved0", _i32),
+        ("state_len", _i32), ("state_rows", _i32),
         ("batch", _i64), ("channels", _i64),
         ("x", _vp), ("x_stride_b", _i64), ("x_stride_c", _i64),
         ("out", _vp), ("out_stride_b", _i64), ("out_stride_c", _i64),

@@ -135,13 +135,12 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const int E = 16 / elem_bytes(p->x_dtype);
     const uint64_t rows = (uint64_t)a.B * a.C;
     a.nt = 2 * rows * a.L * elem_bytes(p->x_dtype) >= kStreamBytes;
-    const bool fused = p->round_mode == CANON_ROUND_FUSED;
     const bool ptr_ok = aligned16(p->x) && aligned16(p->out);
     // packed sequences: the channel-contiguous kernel has a variant (the index is uniform per time row);
     // time-contiguous rows take the strided kernel
     // shorter rows leave most of a wave idle: measured slower than the strided kernel below 16 vectors
     const uint32_t kBclMinVectors = 16;
-    const bool bcl_rows = !p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L / E >= kBclMinVectors;
+    const bool bcl_rows = !p->seq_idx && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && a.L / E >= kBclMinVectors;
     // every row starts on a 16-byte boundary and is a whole number of vectors ...
     const bool bcl_aligned = a.L % E == 0 && a.x_sb % E == 0 && a.x_sc % E == 0 && a.o_sb % E == 0 && a.o_sc % E == 0;
     // ... or x and out share one geometry, so that a row is misaligned by the same amount in both
@@ -149,16 +148,20 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const bool bcl_ok = bcl_rows && (bcl_aligned || bcl_edge);
     const uint32_t EB = kBlcVecBytes / elem_bytes(p->x_dtype);   // channels per lane of the channel-contiguous kernel
     const bool ptr8_ok = (((uintptr_t)p->x | (uintptr_t)p->out) & (kBlcVecBytes - 1)) == 0;
-    const bool blc_ok = fused && ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
+    const bool blc_ok = ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
                         a.x_sb % EB == 0 && a.x_sl % EB == 0 && a.o_sb % EB == 0 && a.o_sl % EB == 0 &&
-                        a.x_sl != 1;
+                        a.x_sl != 1 &&
+                        // rows are addressed by 32-bit scalar offsets inside a wave's buffer resource
+                        a.x_sl > 0 && a.o_sl > 0 &&
+                        (uint64_t)(kBlcRows + 3) * (uint64_t)a.x_sl * elem_bytes(p->x_dtype) + 64 * kBlcVecBytes < (1ull << 31) &&
+                        (uint64_t)(kBlcRows + 3) * (uint64_t)a.o_sl * elem_bytes(p->x_dtype) + 64 * kBlcVecBytes < (1ull << 31);
 
     // Time-contiguous rows of at most 32 whole, aligned vectors share waves (canon_fwd_bcl_short_kernel):
     // measured against one row per wave, the kernel below, 2.3x faster at 16 vectors per row, 1.3x at 32.
     // (Longer rows packed back to back the same way lose to the kernel below even where it leaves half of its
     // lanes idle: 4.4-4.6 against 5.1-5.7 TB/s.)
     const uint32_t kBclShortMaxVectors = 32;
-    if (!p->seq_idx && fused && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && bcl_aligned && a.L / E >= 1 &&
+    if (!p->seq_idx && ptr_ok && a.x_sl == 1 && a.o_sl == 1 && bcl_aligned && a.L / E >= 1 &&
         a.L / E <= kBclShortMaxVectors && rows < (1ull << 31)) {
         const uint32_t nvec = a.L / E;
         uint32_t shift = 0;
@@ -203,13 +206,19 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     }
     if (blc_ok) {
         const uint32_t nvec = a.C / EB;
-        const uint32_t nct = (nvec + 63) / 64;                                   // channel tiles per row
+        const uint32_t nct = (nvec + 64 * kBlcWC - 1) / (64 * kBlcWC);          // channel tiles per row
         const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
-        const uint64_t nblocks = (uint64_t)a.B * ntt * nct;
+        // `group` consecutive time tiles of a channel tile run back to back on one XCD (see blc_block_body): the
+        // fewest equal groups of at most kBlcGroup tiles
+        const uint32_t ngroups = (ntt + kBlcGroup - 1) / kBlcGroup;
+        const uint32_t group = (ntt + ngroups - 1) / ngroups;
+        const uint64_t ncols = (uint64_t)a.B * ngroups * nct;
+        const uint64_t nblocks = (ncols + 7) / 8 * 8 * group;
         if (nblocks < (1ull << 31) - 8) {
             plan->kind = FWD_BLC;
-            a.nvec = nvec; a.nct = nct; a.ntt = ntt; a.ntasks = (uint32_t)nblocks;
-            a.div_nct = make_fastdiv(nct); a.div_ntt = make_fastdiv(ntt);
+            a.nvec = nvec; a.nct = nct; a.ntt = ntt; a.ntasks = (uint32_t)ncols;
+            a.nseg = ngroups; a.chunk = group;
+            a.div_nct = make_fastdiv(nct); a.div_ntt = make_fastdiv(ngroups); a.div_nseg = make_fastdiv(group);
             a.nblocks = (uint32_t)nblocks;
             plan->grid = a.nblocks;
             return CANON_OK;
@@ -247,6 +256,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown round_mode %d", p->round_mode);
     if (((uintptr_t)p->cache_seqlens | (uintptr_t)p->conv_state_indices) & 3u)
         return fail(CANON_ERR_INVALID_ARGUMENT, "cache_seqlens and conv_state_indices must be 4-byte aligned");
+    if (p->state_rows < 0) return fail(CANON_ERR_INVALID_ARGUMENT, "state_rows %d is negative", p->state_rows);
     if (p->cache_seqlens && p->width - 1 > p->state_len)
         return fail(CANON_ERR_INVALID_ARGUMENT, "state_len %d is shorter than width-1 = %d", p->state_len, p->width - 1);
     if (p->batch < 0 || p->channels < 0)
@@ -265,7 +275,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     memset(&a, 0, sizeof(a));
     a.x = (const char *)p->x; a.out = (char *)p->out; a.state = (char *)p->conv_state;
     a.weight = p->weight; a.bias = p->bias; a.tmask = p->token_mask;
-    a.seqlens = p->cache_seqlens; a.indices = p->conv_state_indices;
+    a.seqlens = p->cache_seqlens; a.indices = p->conv_state_indices; a.state_rows = (uint32_t)p->state_rows;
     a.x_sb = p->x_stride_b; a.x_sc = p->x_stride_c; a.o_sb = p->out_stride_b; a.o_sc = p->out_stride_c;
     a.s_sb = p->state_stride_b; a.s_sc = p->state_stride_c; a.s_ss = p->state_stride_s;
     a.w_sc = p->w_stride_c; a.w_sk = p->w_stride_k; a.m_sb = p->mask_stride_b;
@@ -282,7 +292,7 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
     const int BY = elem_bytes(p->x_dtype);
     const int E = upd_lane_channels(BY, S);           // channels per lane
     const int XB = E * BY;                            // bytes of x / out per lane (2 or 4)
-    const bool vec_ok = !p->cache_seqlens && p->round_mode == CANON_ROUND_FUSED && (S == 3 || S == 4 || S == 8) &&
+    const bool vec_ok = !p->cache_seqlens && (S == 3 || S == 4 || S == 8) &&
                         ((uintptr_t)p->x | (uintptr_t)p->out) % XB == 0 && (uintptr_t)p->conv_state % 4 == 0 &&
                         a.x_sc == 1 && a.o_sc == 1 && a.C % E == 0 && a.x_sb * BY % XB == 0 && a.o_sb * BY % XB == 0 &&
                         a.s_ss == 1 && a.s_sc == S && a.s_sb * BY % 4 == 0;

@@ -62,6 +62,16 @@ template <int DT> __device__ __forceinline__ float round_through(float v)
     }
 }
 
+// value -> storage type -> value where the value was just computed: for fp16 it is hidden from the
+// instruction selector first, which would otherwise merge the operation that produced it and the conversion
+// into one mixed-precision instruction (v_fma_mixlo_f16) whose result is not that of the two separate steps
+// in every case (see mul_round below).
+template <int DT> __device__ __forceinline__ float round_result(float v)
+{
+    if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(v));
+    return round_through<DT>(v);
+}
+
 // x * m rounded to the storage type.  For fp16 the product is hidden from the
 // instruction selector: it would otherwise fuse multiply and conversion into
 // v_fma_mixlo_f16 with a +0 addend, which turns a -0 product into +0, and the
@@ -275,6 +285,22 @@ __device__ __forceinline__ void load_mask_rows_wave(const void *p, int64_t row_b
     for (int j = 0; j < N; ++j) m[j] = bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
 }
 
+// The same in two steps, so that the load can be in flight while other work is done: lane j requests entry j ...
+template <int N>
+__device__ __forceinline__ float mask_rows_issue(const void *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
+                                                 int dt, int lane)
+{
+    int64_t t = t_first + (lane < N ? lane : N - 1);
+    t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
+    return load_mask(p, row_base + t * stride, dt);
+}
+
+// ... and entry j is read from lane j when it is needed
+__device__ __forceinline__ float mask_rows_get(float v, int j)
+{
+    return bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
+}
+
 // The same for N sequence indices.
 template <int N>
 __device__ __forceinline__ void load_seq_rows_wave(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L,
@@ -333,6 +359,53 @@ template <> struct VecIO<8> {
         else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
     }
 };
+
+// Buffer accesses: address = resource base + vector offset (checked against the resource's size: a lane
+// beyond it loads zeros and stores nothing) + scalar offset (not checked).
+constexpr int kBufFlags = 0x00020000;   // raw buffer, 32-bit data format
+template <int VB> struct BufIO;
+template <> struct BufIO<8> {
+    template <bool NT> static __device__ __forceinline__ uint2 load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+    {
+        const u32x2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, NT ? 2 : 0);
+        return make_uint2(v.x, v.y);
+    }
+    template <bool NT> static __device__ __forceinline__ void store(const uint2 &v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+    {
+        const u32x2_t q = {v.x, v.y};
+        __builtin_amdgcn_raw_buffer_store_b64(q, r, (int)voff, (int)soff, NT ? 2 : 0);
+    }
+};
+template <> struct BufIO<16> {
+    template <bool NT> static __device__ __forceinline__ uint4 load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+    {
+        const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, NT ? 2 : 0);
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+    template <bool NT> static __device__ __forceinline__ void store(const uint4 &v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff)
+    {
+        const u32x4_t q = {v.x, v.y, v.z, v.w};
+        __builtin_amdgcn_raw_buffer_store_b128(q, r, (int)voff, (int)soff, NT ? 2 : 0);
+    }
+};
+
+// N consecutive 32-bit words through a buffer resource (zeros where out of its range)
+template <int N> __device__ __forceinline__ void buf_load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t *d)
+{
+    if constexpr (N == 1) {
+        d[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, 0, 0);
+    } else if constexpr (N == 2) {
+        const u32x2_t q = __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, 0, 0);
+        d[0] = q.x; d[1] = q.y;
+    } else if constexpr (N == 4) {
+        const u32x4_t q = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, 0, 0);
+        d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+    } else {
+        static_assert(N % 4 == 0 && N > 4, "1, 2 or a multiple of 4 words");
+        buf_load_words<4>(r, voff, d);
+        buf_load_words<N - 4>(r, voff + 16u, d + 4);
+    }
+}
 
 // N sequence indices of consecutive time steps t_first .. t_first+N-1 (clamped to [0, L-1]) of one batch row
 template <int N>
@@ -516,10 +589,28 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f)
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
 
-// The activated, residual-added output of one element (fused rounding mode).
-__device__ __forceinline__ float finish(float acc, int act, int res_mode, float xm, float xr)
+// Activation of N accumulators.  Fused rounding: fp32 throughout (the only rounding is the one at the
+// store).  Eager rounding: the eager module's rounding points, i.e. the convolution result is rounded to the
+// storage type, and so is the activation (the residual sum is rounded by the store).
+template <int DT, int N> __device__ __forceinline__ void activate(float *o, bool act, bool eager)
 {
-    if (act) acc = silu_fast(acc);
+    if (eager) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) o[j] = round_result<DT>(o[j]);
+        if (act) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) o[j] = round_result<DT>(silu_precise(o[j]));
+        }
+    } else if (act) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) o[j] = silu_fast(o[j]);
+    }
+}
+
+// The activated, residual-added output of one element.
+template <int DT> __device__ __forceinline__ float finish(float acc, int act, int res_mode, int eager, float xm, float xr)
+{
+    activate<DT, 1>(&acc, act != 0, eager != 0);
     if (res_mode == CANON_RESIDUAL_MASKED) acc += xm;
     else if (res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
     return acc;
@@ -772,8 +863,13 @@ __device__ __forceinline__ void decode_taps_contiguous(const TapWords<WDT, E> &r
 #pragma unroll
     for (int e = 0; e < E; ++e) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) w[e][k] = round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(r.w, e * 4 + k)));
-        bv[e] = has_bias ? round_through<DT>(Packed<WDT>::as_float(Packed<WDT>::get(r.b, e))) : 0.0f;
+        // weights that already have the storage type of x need no rounding
+        for (int k = 0; k < 4; ++k) {
+            const float t = Packed<WDT>::as_float(Packed<WDT>::get(r.w, e * 4 + k));
+            w[e][k] = WDT == DT ? t : round_through<DT>(t);
+        }
+        const float tb = Packed<WDT>::as_float(Packed<WDT>::get(r.b, e));
+        bv[e] = has_bias ? (WDT == DT ? tb : round_through<DT>(tb)) : 0.0f;
     }
 }
 

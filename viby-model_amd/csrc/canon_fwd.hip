@@ -85,7 +85,7 @@ __device__ __forceinline__ void bcl_edge_finish(const FwdArgs &a, const float (*
     float acc = bv;
 #pragma unroll
     for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], win[(4 - W) + k], acc);
-    store1<DT>(orow, t, finish(acc, a.act, a.res_mode, win[3], e.x[3]));
+    store1<DT>(orow, t, finish<DT>(acc, a.act, a.res_mode, a.eager, win[3], e.x[3]));
 }
 
 // EDGE: the rows are contiguous in time but do not start on 16-byte boundaries (a length or a
@@ -229,10 +229,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
             for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
             o[j] = acc;
         }
-        if (a.act) {
-#pragma unroll
-            for (int j = 0; j < E; ++j) o[j] = silu_fast(o[j]);
-        }
+        activate<DT, E>(o, a.act, a.eager);
         if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
 #pragma unroll
             for (int j = 0; j < E; ++j) o[j] += xr[j];
@@ -323,10 +320,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
         for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
         o[j] = acc;
     }
-    if (a.act) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) o[j] = silu_fast(o[j]);
-    }
+    activate<DT, E>(o, a.act, a.eager);
     if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
 #pragma unroll
         for (int j = 0; j < E; ++j) o[j] += xr[j];
@@ -346,22 +340,33 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
 //
 // One lane owns E adjacent channels (VB = 8 bytes of every row: 4 x 16-bit or
 // 2 x fp32; 16-byte lanes need 142 registers and measured 4-9 % slower) and R
-// consecutive time steps; the four waves of a block own four consecutive
-// R-row slabs of the same 64-lane channel tile, so a block streams a
-// [4R rows] x [512 B] tile and consecutive blocks sweep memory in address
-// order (short-lived waves over a compact window: measured to be what HBM
-// wants; long per-lane time runs lose 10-20 %).  The three rows a wave needs from before its slab are the
-// last three rows of the previous wave: each wave publishes the raw tail of
-// its slab in LDS, one barrier, the next wave picks it up -- only the first
-// wave of a block reads its halo from memory.  All loads (slab, halo, taps)
-// are issued before the first wait.
+// consecutive time steps; the WT waves of a block own WT consecutive R-row
+// slabs of the same 64-lane channel tile, so a block streams a
+// [WT * R rows] x [512 B] tile (short-lived waves over a compact window:
+// measured to be what HBM wants; long per-lane time runs lose 10-20 %).
+// Memory is reached through buffer resources, one per tensor and wave: the
+// row is a scalar offset and the lane a 32-bit vector offset, so an access
+// costs no 64-bit address arithmetic, and lanes past the last channel are
+// dropped by the range check of the resource.
+// The three rows a wave needs from before its slab are the last three rows of
+// the previous wave: each wave publishes the raw tail of its slab in LDS, one
+// barrier, the next wave picks it up -- only the first wave of a block reads
+// its history from memory, and the block order makes that a hit in the L2 of
+// its XCD (see blc_block_body).  The same barrier passes on the taps: the
+// waves of a tile fetch a WT-th of its taps and bias each (every wave fetching
+// all of them cost 3 % at B = 32: 2.5 KB of L2 traffic per 8 KB of x).
+// All loads (slab, history, taps) are issued before the first wait.
 // ---------------------------------------------------------------------------
+// One row of a slab: out = act(bias + taps . (history, x)) (+ residual), written through the wave's buffer
+// resource.  ACT / RES / EAGER: the activation flag, the residual mode and the rounding mode when they are
+// known at compile time (-1: read from the arguments; a select per element and a branch per row then).
 // keep0..2 (wave uniform): whether the rows t-3, t-2, t-1 belong to the packed sequence of row t
 // (always true without seq_idx); a row of another sequence enters as zeros.
-template <int DT, int W, bool MASK, bool NT, int VB>
-__device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], const float *bias,
-                                        float (*hist)[VB / Elem<DT>::bytes], const typename VecIO<VB>::type &X, float m,
-                                        char *optr, bool active, bool keep0 = true, bool keep1 = true, bool keep2 = true)
+template <int DT, int W, bool MASK, bool NT, int VB, int ACT = -1, int RES = -1, int EAGER = -1>
+__device__ __forceinline__ void blc_row_buf(const FwdArgs &a, const float (*w)[W], const float *bias,
+                                            float (*hist)[VB / Elem<DT>::bytes], const typename VecIO<VB>::type &X, float m,
+                                            __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t soff,
+                                            bool keep0 = true, bool keep1 = true, bool keep2 = true)
 {
     constexpr int E = VB / Elem<DT>::bytes;
     float xr[E], xm_store[MASK ? E : 1], o[E];
@@ -383,62 +388,139 @@ __device__ __forceinline__ void blc_row(const FwdArgs &a, const float (*w)[W], c
         hist[1][e] = hist[2][e];
         hist[2][e] = xm[e];
     }
-    if (a.act) {
-#pragma unroll
-        for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
-    }
-    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+    const bool act = ACT < 0 ? a.act != 0 : ACT != 0;
+    const int res = RES < 0 ? a.res_mode : RES;
+    const bool eager = EAGER < 0 ? a.eager != 0 : EAGER != 0;
+    activate<DT, E>(o, act, eager);
+    if (res == CANON_RESIDUAL_UNMASKED || (!MASK && res)) {
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] += xr[e];
-    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+    } else if (res == CANON_RESIDUAL_MASKED) {
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] += xm[e];
     }
-    if (active) VecIO<VB>::template store<NT>(optr, VecIO<VB>::template pack<DT>(o));
+    BufIO<VB>::template store<NT>(VecIO<VB>::template pack<DT>(o), ro, voff, soff);
+}
+
+// All rows first .. rows-1 of a slab.
+template <int DT, int W, int R, bool MASK, bool NT, int VB, int ACT, int RES, int EAGER>
+__device__ __forceinline__ void blc_rows_buf(const FwdArgs &a, const float (&w)[VB / Elem<DT>::bytes][W], const float (&bias)[VB / Elem<DT>::bytes],
+                                             float (&hist)[3][VB / Elem<DT>::bytes], const typename VecIO<VB>::type (&X)[R], const float (&m)[R],
+                                             __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t os, int rows)
+{
+    if (rows == R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) blc_row_buf<DT, W, MASK, NT, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (r < rows) blc_row_buf<DT, W, MASK, NT, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+    }
+}
+
+// ... with activation, residual and rounding mode as compile-time constants for the settings CanonLayer uses
+// (no activation; residual added or not; either rounding mode), read from the arguments otherwise.
+template <int DT, int W, int R, bool MASK, bool NT, int VB>
+__device__ __forceinline__ void blc_rows_dispatch(const FwdArgs &a, const float (&w)[VB / Elem<DT>::bytes][W], const float (&bias)[VB / Elem<DT>::bytes],
+                                                  float (&hist)[3][VB / Elem<DT>::bytes], const typename VecIO<VB>::type (&X)[R], const float (&m)[R],
+                                                  __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t os, int rows)
+{
+    // without a mask both residual modes add the raw input
+    const int res = (!MASK && a.res_mode) ? CANON_RESIDUAL_UNMASKED : a.res_mode;
+    constexpr int XR = CANON_RESIDUAL_UNMASKED, XM = CANON_RESIDUAL_MASKED, NONE = CANON_RESIDUAL_NONE;
+    if (a.act) blc_rows_buf<DT, W, R, MASK, NT, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == XR) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XR, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == XM) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XM, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == NONE) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, NONE, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (res == XR) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XR, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (res == XM) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XM, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else blc_rows_buf<DT, W, R, MASK, NT, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
 }
 
 template <int DT, int W, int R, bool MASK, bool NT, bool SEQ, int VB, int MODE>
 __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t blk,
-                                               typename VecIO<VB>::type (*tail)[3][64])   // LDS: raw last three rows of each wave's slab
+                                               typename VecIO<VB>::type (*tail)[3][64],   // LDS: raw last three rows of each wave's slab
+                                               uint32_t (*taps_lds)[64 * (VB / 2) * 5])   // LDS: taps and bias of each channel tile
 {
     constexpr int E = VB / Elem<DT>::bytes;
+    constexpr int BY = Elem<DT>::bytes;
     constexpr int WDT = MODE == TAPS_WIDE ? CANON_DTYPE_F32 : DT;   // weight type of the straight-line tap modes
+    constexpr int WT = kBlcWaves, WC = kBlcWC;
     using V = VecIO<VB>;
     using vec_t = typename V::type;
     static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
 
-    // blocks in plain memory order (an XCD-contiguous remap measured 3 % slower here)
-    // blk = (b * ntt + tt) * nct + ct : channel tile fastest, i.e. memory order
-    const uint32_t bt = fdiv(blk, a.div_nct);
-    const uint32_t ct = blk - bt * a.nct;
-    const uint32_t b = fdiv(bt, a.div_ntt);
-    const uint32_t tt = bt - b * a.ntt;
-    const int lane = threadIdx.x & 63;
+    // Block -> tile.  Workgroups are dealt to the eight XCDs (each with its own L2) in turn, block i to XCD
+    // i % 8.  The tiles are numbered so that `chunk` consecutive time tiles of one channel tile follow each
+    // other on ONE XCD: the three rows of history that the first wave of a tile re-reads were requested by
+    // the tile before it a moment earlier and come out of that L2 instead of memory.  The columns
+    // q = (b * ngroups + tg) * nct + ct (tg: a group of `chunk` time tiles) are dealt to the XCDs in turn,
+    // so the launch still sweeps memory in address order.
+    const uint32_t jq = blk >> 3;
+    const uint32_t jg = fdiv(jq, a.div_nseg);
+    const uint32_t q = jg * 8u + (blk & 7u);
+    if (q >= a.ntasks) return;   // whole block, before the barrier
+    const uint32_t qr = fdiv(q, a.div_nct);
+    const uint32_t ct = q - qr * a.nct;
+    const uint32_t b = fdiv(qr, a.div_ntt);
+    const uint32_t tt = (qr - b * a.nseg) * a.chunk + (jq - jg * a.chunk);
+    if (tt >= a.ntt) return;
+    const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t cv = ct * 64u + lane;
-    const bool active = cv < a.nvec;
-    const uint32_t c0 = (active ? cv : a.nvec - 1u) * E;   // idle lanes shadow the last vector, loads need no predicate
-
-    const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * Elem<DT>::bytes;
-    char *ob = a.out + ((int64_t)b * a.o_sb + c0) * Elem<DT>::bytes;
-    const int64_t xs = a.x_sl * Elem<DT>::bytes, os = a.o_sl * Elem<DT>::bytes;
-    const int64_t t0 = ((int64_t)tt * kBlcWaves + wv) * R;
+    const uint32_t wt = wv / WC, wc = wv - wt * WC;
+    const uint32_t cv0 = (ct * WC + wc) * 64u;                 // the wave's first channel vector
+    const int64_t t0 = ((int64_t)tt * WT + wt) * R;
     const int64_t left = (int64_t)a.L - t0;
-    const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
-    const int64_t t_last = (int64_t)a.L - 1;
+    const bool idle = cv0 >= a.nvec || left <= 0;              // wave uniform: nothing to do but the barrier
+    const int rows = idle ? 0 : (left >= R ? R : (int)left);
+    const uint32_t nl = idle ? 0u : (a.nvec - cv0 < 64u ? a.nvec - cv0 : 64u);   // lanes that hold channels
+    const bool active = lane < nl;
+    const uint32_t cvl = cv0 + lane < a.nvec ? cv0 + lane : a.nvec - 1u;   // idle lanes shadow the last vector (taps, state)
+    const uint32_t c0 = cvl * E;
 
-    // taps (contiguous layouts: first, they come from the cache and nothing waits for them before the rows
-    // are requested), slab rows, then (first wave only) the three rows before the block.
-    // Rows past the end of the sequence are clamped to the last row (loaded, never used).
+    // One buffer resource per tensor and wave: lanes by vector offset, rows by scalar offset.  The x resource
+    // starts three rows early.
+    const uint32_t xs = (uint32_t)(a.x_sl * BY), os = (uint32_t)(a.o_sl * BY);
+    const char *xw = a.x + ((int64_t)b * a.x_sb + (int64_t)cv0 * E) * BY + (t0 - 3) * (int64_t)xs;
+    char *ow = a.out + ((int64_t)b * a.o_sb + (int64_t)cv0 * E) * BY + t0 * (int64_t)os;
+    // Every access the wave issues lies inside the resources (rows past the end of the sequence are neither
+    // loaded nor stored); only lanes without channels are sent out of range, by their vector offset.
+    const uint32_t xrec = idle ? 0u : (uint32_t)(R + 2) * xs + nl * VB, orec = idle ? 0u : (uint32_t)(R - 1) * os + nl * VB;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)xw, 0, (int)xrec, kBufFlags);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)ow, 0, (int)orec, kBufFlags);
+    const uint32_t voff = active ? lane * VB : 0x80000000u;
+
     vec_t X[R], H[3];
     float m[R], mh[3];
     int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
     TapWords<WDT, E> tw;
-    if constexpr (MODE != TAPS_ANY) fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
+    // The waves that share a channel tile fetch its taps and bias together, each a contiguous WT-th of them, and
+    // pass them on through LDS with the hand-over of the slab tails (one barrier for both).
+    constexpr bool kShare = MODE != TAPS_ANY && WT > 1;
+    constexpr int NW = TapWords<WDT, E>::NW, NB = TapWords<WDT, E>::NB;   // words per lane
+    constexpr int PW = NW / WT > 0 ? NW / WT : 1, PB = (NB + WT - 1) / WT;   // words per thread
+    static_assert(!kShare || NW % WT == 0, "taps of a lane split evenly over the waves of a tile");
+    uint32_t tpw[PW], tpb[PB];
+    const uint32_t g = wt * 64u + lane;                         // thread within the tile's group of waves
+    if constexpr (kShare) {
+        constexpr int WBY = Elem<WDT>::bytes;
+        const uint32_t ctile = cv0 < a.nvec ? cv0 * E : 0u;     // first channel of the tile
+        const uint32_t cleft = cv0 < a.nvec ? a.C - ctile : 0u;
+        const uint32_t wbytes = (cleft < 64u * E ? cleft : 64u * E) * 4u * WBY;
+        const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.weight + (int64_t)ctile * 4 * WBY), 0, (int)wbytes, kBufFlags);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)(a.bias ? a.bias : a.weight) + (int64_t)ctile * WBY), 0, (int)(wbytes / 4u), kBufFlags);
+        buf_load_words<PW>(rw, g * (PW * 4u), tpw);
+        // (words past the tile's bias are out of range of the resource and read zero)
+        buf_load_words<PB>(rb, g * (PB * 4u) < 64u * NB * 4u ? g * (PB * 4u) : 0x80000000u, tpb);
+    } else if constexpr (MODE != TAPS_ANY) {
+        fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        X[r] = V::zero();
+        // rows past the end of the sequence: the slab's last row again (loaded, never used)
+        const uint32_t rr = r < rows ? (uint32_t)r : (rows > 0 ? (uint32_t)(rows - 1) : 0u);
+        X[r] = BufIO<VB>::template load<NT>(rx, voff, (rr + 3u) * xs);
         m[r] = 0.0f;
     }
 #pragma unroll
@@ -448,20 +530,12 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
         H[j] = V::zero();
         mh[j] = 0.0f;
     }
+    if (wt == 0 && t0 > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<false>(rx, voff, (uint32_t)j * xs);
+    }
     if (rows > 0) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t t = t0 + r < t_last ? t0 + r : t_last;
-            X[r] = V::template load<NT>(xb + t * xs);
-        }
-        if (wv == 0) {
-#pragma unroll
-            for (int j = 0; j < 3; ++j) {
-                const int64_t t = t0 - 3 + j;
-                if (j >= 3 - (W - 1) && t >= 0) H[j] = V::template load<false>(xb + t * xs);
-            }
-        }
-        // every wave fetches the taps itself (cache hits); sharing them through LDS was measured slower
         if constexpr (MODE == TAPS_ANY)
             fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
         if constexpr (SEQ) load_seq_rows_wave<R + 3>(a.seq, (int64_t)b * a.q_sb, t0 - 3, a.L, a.q_sl, lane, sq);
@@ -476,14 +550,32 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
         }
     }
 
-    // hand the raw tail of this slab to the next wave
+    // hand the raw tail of this slab to the wave that owns the next slab of the same channel tile
+    if constexpr (WT > 1) {
+        if constexpr (kShare) {
+            uint32_t *tl = taps_lds[wc];
 #pragma unroll
-    for (int j = 0; j < 3; ++j) tail[wv][j][lane] = X[R - 3 + j];
-    __syncthreads();
-    if (wv > 0) {
+            for (int i = 0; i < PW; ++i) tl[g * PW + i] = tpw[i];
+            if (g * PB < 64u * NB) {
 #pragma unroll
-        for (int j = 0; j < 3; ++j)
-            if (j >= 3 - (W - 1)) H[j] = tail[wv - 1][j][lane];
+                for (int i = 0; i < PB; ++i) tl[64 * NW + g * PB + i] = tpb[i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 3; ++j) tail[wv][j][lane] = X[R - 3 + j];
+        __syncthreads();
+        if (wt > 0) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+                if (j >= 3 - (W - 1)) H[j] = tail[wv - WC][j][lane];
+        }
+        if constexpr (kShare) {
+            const uint32_t *tl = taps_lds[wc];
+#pragma unroll
+            for (int i = 0; i < NW; ++i) tw.w[i] = tl[lane * NW + i];
+#pragma unroll
+            for (int i = 0; i < NB; ++i) tw.b[i] = tl[64 * NW + lane * NB + i];
+        }
     }
     if (rows == 0) return;   // after the barrier
 
@@ -509,7 +601,6 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
     float w[E][W], bias[E];
     if constexpr (MODE == TAPS_ANY) decode_taps<DT, W, E>(raw, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
     else decode_taps_contiguous<DT, WDT, E>(tw, a.bias != nullptr, w, bias);
-
     if constexpr (SEQ) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -518,26 +609,22 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
             // so the all-kept case takes the plain code
             const int32_t cur = sq[3 + r];
             const bool k0 = sq[r] == cur, k1 = sq[r + 1] == cur, k2 = sq[r + 2] == cur;
-            if (k0 && k1 && k2) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
-            else blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active, k0, k1, k2);
+            if (k0 && k1 && k2) blc_row_buf<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+            else blc_row_buf<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os, k0, k1, k2);
         }
-    } else if (rows == R) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
     } else {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-            if (r < rows) blc_row<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ob + (t0 + r) * os, active);
+        blc_rows_dispatch<DT, W, R, MASK, NT, VB>(a, w, bias, hist, X, m, ro, voff, os, rows);
     }
 
     if (a.fin && active && t0 + rows == (int64_t)a.L) {
+        const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * BY;
         for (int slot = 0; slot < a.S_out; ++slot) {
             const int64_t t = (int64_t)a.L - a.S_out + slot;
             float v[E];
 #pragma unroll
             for (int e = 0; e < E; ++e) v[e] = 0.0f;
             if (t >= 0) {
-                V::template unpack<DT>(V::template load<false>(xb + t * xs), v);
+                V::template unpack<DT>(V::template load<false>(xb + t * (int64_t)xs), v);
                 if constexpr (MASK) {
                     const float mm = load_mask(a.mask, b * a.m_sb + t * a.m_sl, a.mask_dtype);
 #pragma unroll
@@ -560,37 +647,41 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
 template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
 __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 {
-    __shared__ typename VecIO<VB>::type tail[kBlcWaves][3][64];
+    __shared__ typename VecIO<VB>::type tail[kBlcWaves * kBlcWC][3][64];
+    // taps and bias of the block's channel tiles as fetched by its waves together: fp32 weights of 16-bit x are the
+    // largest case, 64 lanes x 4 channels x (4 taps + bias) x 4 bytes
+    constexpr int kTapWordsLds = 64 * (VB / 2) * 5;
+    __shared__ uint32_t taps_lds[kBlcWC][kTapWordsLds];
     if constexpr (W == 4) {
         if (a.tap_mode == TAPS_SAME) {
-            blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_SAME>(a, blk, tail);
+            blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_SAME>(a, blk, tail, taps_lds);
             return;
         }
         if constexpr (DT != CANON_DTYPE_F32) {
             if (a.tap_mode == TAPS_WIDE) {
-                blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_WIDE>(a, blk, tail);
+                blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_WIDE>(a, blk, tail, taps_lds);
                 return;
             }
         }
     }
-    blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_ANY>(a, blk, tail);
+    blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_ANY>(a, blk, tail, taps_lds);
 }
 
 template <int DT, int W, int R, bool MASK, bool NT>
-__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_kernel(const FwdArgs a)
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const FwdArgs a)
 {
     blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
 }
 
 // the same over packed variable-length sequences (seq_idx)
 template <int DT, int W, int R, bool MASK>
-__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_seq_kernel(const FwdArgs a)
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_seq_kernel(const FwdArgs a)
 {
     blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
 template <int DT, int W, int R, bool MASK, bool NT>
-__global__ __launch_bounds__(64 * kBlcWaves) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
 {
     const uint32_t p = part_of_block(m, blockIdx.x);
     blc_block<DT, W, R, MASK, NT>(m.part[p], blockIdx.x - m.first_block[p]);
@@ -671,15 +762,7 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
                 acc = fmaf(w[2], h[2], acc);
                 acc = fmaf(w[3], xm, acc);
             }
-            if (a.eager) {
-                acc = round_through<DT>(acc);
-                if (a.act) acc = round_through<DT>(silu_precise(acc));
-                if (a.res_mode == CANON_RESIDUAL_MASKED) acc += xm;
-                else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr;
-            } else {
-                acc = finish(acc, a.act, a.res_mode, xm, xr);
-            }
-            store1<DT>(a.out, oo + t * a.o_sl, acc);
+            store1<DT>(a.out, oo + t * a.o_sl, finish<DT>(acc, a.act, a.res_mode, a.eager, xm, xr));
             h[0] = h[1];
             h[1] = h[2];
             h[2] = xm;
@@ -743,15 +826,7 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
                 acc = fmaf(w[2], x2, acc);
                 acc = fmaf(w[3], x3, acc);
             }
-            if (a.eager) {
-                acc = round_through<DT>(acc);
-                if (a.act) acc = round_through<DT>(silu_precise(acc));
-                if (a.res_mode == CANON_RESIDUAL_MASKED) acc += x3;
-                else if (a.res_mode == CANON_RESIDUAL_UNMASKED) acc += xr[j + 3];
-            } else {
-                acc = finish(acc, a.act, a.res_mode, x3, xr[j + 3]);
-            }
-            store1<DT>(a.out, oo + t * a.o_sl, acc);
+            store1<DT>(a.out, oo + t * a.o_sl, finish<DT>(acc, a.act, a.res_mode, a.eager, x3, xr[j + 3]));
         }
     }
     if (a.fin && ch == a.nseg - 1)
@@ -783,15 +858,15 @@ template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &
 {
     if (pl.kind == FWD_BCL_SHORT) hipLaunchKernelGGL((canon_fwd_bcl_short_kernel<DT, W, MASK>), dim3(pl.grid), dim3(256), 0, s, pl.args);
     else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
-    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
 }
 
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 {
     const bool mask = pl.args.mask != nullptr;
     if (pl.args.seq) {   // only the channel-contiguous kernel is planned with seq_idx
-        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
-        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(64 * kBlcWaves), 0, s, pl.args);
+        if (mask) hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, true>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
+        else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
         return;
     }
     // the streaming (non-temporal) variants exist for width 4 only
@@ -821,7 +896,7 @@ template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
 template <int DT, bool MASK, bool NT>
 void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(64 * kBlcWaves), 0, s, m);
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(kBlcThreads), 0, s, m);
 }
 
 template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)

@@ -56,14 +56,14 @@ struct FwdArgs {
     int32_t W, w_dtype, mask_dtype, act, res_mode, eager, S_in, S_out, w_vec, b_pair, m_vec, nt, tap_mode;
     // launch geometry
     uint32_t nvec;      // bcl: vectors per row        blc: channel vectors per time row
-    uint32_t nseg;      // bcl: segments per row       generic: time chunks per row
-    uint32_t chunk;     // generic: time steps per chunk
-    uint32_t ntasks;    // bcl: wave tasks   blc: blocks   generic: threads
+    uint32_t nseg;      // bcl: segments per row       generic: time chunks per row     blc: groups of time tiles per sequence
+    uint32_t chunk;     // generic: time steps per chunk                                 blc: time tiles per group
+    uint32_t ntasks;    // bcl: wave tasks   blc: columns (batch x group x channel tile)   generic: threads
     uint32_t nblocks;   // blocks to launch
-    FastDiv div_nseg, div_C;
+    FastDiv div_nseg, div_C;   // blc: div_nseg divides by `chunk`
     // blc: tiles
     uint32_t nct, ntt;  // channel tiles per row, time tiles per sequence
-    FastDiv div_nct, div_ntt;
+    FastDiv div_nct, div_ntt;   // div_ntt divides by the groups per sequence
 };
 
 struct UpdArgs {
@@ -88,6 +88,7 @@ struct UpdArgs {
     const int32_t *indices;   // conv_state row of batch entry b (state pool shared by many sequences)
     int64_t w_sc, w_sk;
     int32_t w_vec;
+    uint32_t state_rows;      // rows of the state pool (0: not stated, indices are only checked for a negative value)
     // the rest: strided kernel, ring buffer, launch geometry
     const int32_t *seqlens;   // circular-buffer mode: conv_state is written at seqlens[b] % S, not shifted
     int64_t x_sc, o_sc;
@@ -172,7 +173,13 @@ template <typename Args> struct PartTable {
 #ifndef CANON_BLC_WAVES
 #define CANON_BLC_WAVES 4
 #endif
-constexpr int kBlcWaves = CANON_BLC_WAVES;   // waves (time slabs) per block
+constexpr int kBlcWaves = CANON_BLC_WAVES;   // time slabs per block
+#ifndef CANON_BLC_WC
+#define CANON_BLC_WC 1
+#endif
+constexpr int kBlcWC = CANON_BLC_WC;         // 64-lane channel tiles per block
+constexpr int kBlcThreads = 64 * kBlcWaves * kBlcWC;
+constexpr int kBlcGroup = 8;                 // most consecutive time tiles of a channel tile that follow each other on one XCD
 constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 % faster than 16 (half the registers, twice the waves)
 #ifndef CANON_BWD_SLAB
 #define CANON_BWD_SLAB 8

@@ -4,6 +4,17 @@
 
 namespace canon {
 
+// Row of the state pool that batch entry b uses (conv_state_indices), or kSkipRow when the index lies outside
+// the pool (negative, or not below state_rows when the caller stated the pool's size): such an entry is
+// left alone -- no state row and no output is touched.
+constexpr uint32_t kSkipRow = 0xFFFFFFFFu;
+__device__ __forceinline__ uint32_t pool_row(const UpdArgs &a, uint32_t b)
+{
+    const int32_t i = a.indices[b];
+    if (i < 0 || (a.state_rows > 0 && (uint32_t)i >= a.state_rows)) return kSkipRow;
+    return (uint32_t)i;
+}
+
 // ---------------------------------------------------------------------------
 // decode update, vectorised: contiguous [B, C, S] state, channel-contiguous
 // x / out.  One lane owns the state rows of E adjacent channels, E chosen so
@@ -17,7 +28,23 @@ namespace canon {
 // pass.  Each lane walks NB batch rows so the taps are fetched once per NB
 // tokens.
 // ---------------------------------------------------------------------------
-template <int DT, int W, int S, int NB, int MODE>
+// One output of the eager module's step (rounding mode "eager"): history taken from packed state words
+// starting at element `first`, the token last.
+template <int DT, int W>
+__device__ __forceinline__ float eager_step(const float *w, float bias, const uint32_t *state_words, int first, float xt, bool act)
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < W - 1; ++k)
+        s = __fadd_rn(s, mul_round<DT>(Packed<DT>::as_float(Packed<DT>::get(state_words, first + k)), w[k]));
+    s = __fadd_rn(s, mul_round<DT>(xt, w[W - 1]));
+    s = round_result<DT>(s);
+    float acc = round_result<DT>(__fadd_rn(bias, s));
+    if (act) acc = round_result<DT>(silu_precise(acc));
+    return acc;
+}
+
+template <int DT, int W, int S, int NB, int MODE, bool POOL>
 __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t bg, const uint32_t c0,
                                                 const uint32_t (*X)[(upd_lane_channels(Elem<DT>::bytes, S) * Elem<DT>::bytes + 3) / 4],
                                                 const uint32_t (*ST)[upd_lane_channels(Elem<DT>::bytes, S) * S * Elem<DT>::bytes / 4],
@@ -60,7 +87,7 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
         const uint32_t b = bg * NB + n;
-        if (b >= a.B) continue;
+        if (b >= a.B || (POOL && srow[n] == kSkipRow)) continue;
         float xr[E], xt[E], o[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) xr[e] = Packed<DT>::as_float(Packed<DT>::get(X[n], e));
@@ -71,24 +98,31 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
 #pragma unroll
             for (int e = 0; e < E; ++e) xt[e] = xr[e];
         }
+        if (!a.eager) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-            float acc = bias[e];
+            for (int e = 0; e < E; ++e) {
+                float acc = bias[e];
 #pragma unroll
-            for (int k = 0; k < W - 1; ++k)
-                acc = fmaf(w[e][k], Packed<DT>::as_float(Packed<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
-            o[e] = fmaf(w[e][W - 1], xt[e], acc);
-        }
-        if (a.act) {
+                for (int k = 0; k < W - 1; ++k)
+                    acc = fmaf(w[e][k], Packed<DT>::as_float(Packed<DT>::get(ST[n], e * S + (S - (W - 1) + k))), acc);
+                o[e] = fmaf(w[e][W - 1], xt[e], acc);
+            }
+            if (a.act) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
+                for (int e = 0; e < E; ++e) o[e] = silu_fast(o[e]);
+            }
+        } else {
+            // the eager module's step: every product rounded to the storage type, their fp32 sum rounded, then
+            // the bias added and rounded, then the activation rounded
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] = eager_step<DT, W>(w[e], bias[e], &ST[n][0], e * S + (S - (W - 1)), xt[e], a.act != 0);
         }
         if (a.res_mode == CANON_RESIDUAL_MASKED) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) o[e] += xt[e];
+            for (int e = 0; e < E; ++e) o[e] = __fadd_rn(o[e], xt[e]);
         } else if (a.res_mode == CANON_RESIDUAL_UNMASKED) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) o[e] += xr[e];
+            for (int e = 0; e < E; ++e) o[e] = __fadd_rn(o[e], xr[e]);
         }
         uint32_t ow[NX] = {};
 #pragma unroll
@@ -132,27 +166,33 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
 #pragma unroll
     for (int n = 0; n < NB; ++n) {
         const uint32_t b = bg * NB + n;
+        srow[n] = b;
         if (b < a.B) {
+            // POOL: rows of a state pool (conv_state_indices); an entry whose index is outside the pool is skipped
+            // (nothing of it is read or written)
+            if constexpr (POOL) {
+                srow[n] = pool_row(a, b);
+                if (srow[n] == kSkipRow) continue;
+            }
             const char *xp = a.x + ((int64_t)b * a.x_sb + c0) * BY;
             if constexpr (E * BY == 2) X[n][0] = *(const uint16_t *)xp;
             else load_words<NX>(xp, X[n]);
-            srow[n] = POOL ? (uint32_t)a.indices[b] : b;   // POOL: rows of a state pool (conv_state_indices)
             load_words<ND>(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
         }
     }
     if constexpr (W == 4) {
         if (a.tap_mode == TAPS_SAME) {
-            update_vec_body<DT, W, S, NB, TAPS_SAME>(a, bg, c0, X, ST, srow);
+            update_vec_body<DT, W, S, NB, TAPS_SAME, POOL>(a, bg, c0, X, ST, srow);
             return;
         }
         if constexpr (DT != CANON_DTYPE_F32) {
             if (a.tap_mode == TAPS_WIDE) {
-                update_vec_body<DT, W, S, NB, TAPS_WIDE>(a, bg, c0, X, ST, srow);
+                update_vec_body<DT, W, S, NB, TAPS_WIDE, POOL>(a, bg, c0, X, ST, srow);
                 return;
             }
         }
     }
-    update_vec_body<DT, W, S, NB, TAPS_ANY>(a, bg, c0, X, ST, srow);
+    update_vec_body<DT, W, S, NB, TAPS_ANY, POOL>(a, bg, c0, X, ST, srow);
 }
 
 template <int DT, int W, int S, int NB>
@@ -189,7 +229,8 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
     for (int k = 0; k < W; ++k)
         w[4 - W + k] = round_through<DT>(load_w(a.weight, (int64_t)c * a.w_sc + k * a.w_sk, a.w_dtype));
     const float bv = a.bias ? round_through<DT>(load_w(a.bias, c, a.w_dtype)) : 0.0f;
-    const uint32_t srow = a.indices ? (uint32_t)a.indices[b] : b;
+    const uint32_t srow = a.indices ? pool_row(a, b) : b;
+    if (srow == kSkipRow) return;
     const int64_t so = (int64_t)srow * a.s_sb + (int64_t)c * a.s_sc;
     // circular-buffer mode: the token goes to slot pos, the W-1 slots before it (cyclically) are the history
     int pos = -1;
@@ -216,7 +257,7 @@ __global__ __launch_bounds__(256) void canon_update_generic_kernel(const UpdArgs
         if (W >= 3) acc = fmaf(w[1], win[1], acc);
         acc = fmaf(w[2], win[2], acc);
         acc = fmaf(w[3], win[3], acc);
-        acc = finish(acc, a.act, a.res_mode, xt, xr);
+        acc = finish<DT>(acc, a.act, a.res_mode, 0, xt, xr);
     } else {
         float s = 0.0f;
         for (int k = 4 - W; k < 4; ++k) s = __fadd_rn(s, mul_round<DT>(win[k], w[k]));

@@ -336,8 +336,10 @@ int canon_conv1d_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_
 int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts,
                               void *stream);
 
-/* Scratch bytes canon_conv1d_bwd needs for these sizes and strides (the
- * pointers in *p are not read); negative if the arguments are rejected. */
+/* Scratch bytes canon_conv1d_bwd needs for these sizes, strides and pointer
+ * alignments; with x, dout or dx missing (NULL) the figure also covers the
+ * kernel a misaligned pointer would select.  Negative if the arguments are
+ * rejected. */
 int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params *p);
 int64_t canon_conv1d_update_bwd_workspace_bytes(const canon_conv1d_update_bwd_params *p);
 

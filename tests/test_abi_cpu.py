@@ -338,6 +338,36 @@ def test_bwd_plan_and_workspace():
     assert "alias" in last_error()
 
 
+def _demanded_workspace(p):
+    """What canon_conv1d_bwd itself asks for: its complaint about a one-byte workspace names the size."""
+    import re
+    p.workspace, p.workspace_bytes = FAKE_W + 0x200000, 1
+    assert _lib.lib().canon_conv1d_bwd(ctypes.byref(p), None) == _lib.ERR_INVALID_ARGUMENT
+    m = re.search(r"at least (\d+) bytes", last_error())
+    assert m, last_error()
+    return int(m.group(1))
+
+
+def test_bwd_workspace_query_covers_misaligned_pointers():
+    L = _lib.lib()
+    # time-contiguous rows with a padded row stride, x off by one element: the call takes the strided kernel,
+    # which needs more scratch than the vector kernel an aligned x would get
+    for over in (dict(x=FAKE_X + 2), dict(dout=FAKE_OUT + 2), dict(dx=FAKE_STATE + 2), dict()):
+        q = bwd_params(layout="bcl", x_stride_c=1032, x_stride_b=3456 * 1032, **over)
+        want_kernel = b"bwd_generic" if over else b"bwd_bcl_vec"
+        assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == want_kernel, over
+        assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(q)) == _demanded_workspace(q), over
+    for over in (dict(x=FAKE_X + 4), dict(dx=FAKE_STATE + 2)):          # channel-contiguous: 8-byte lanes
+        q = bwd_params(**over)
+        assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == b"bwd_generic"
+        assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(q)) == _demanded_workspace(q), over
+    # sizes asked for before the tensors exist (NULL pointers): enough for whichever kernel the call will take
+    for layout in ("bcl", "blc"):
+        unknown = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(layout=layout, x=0, dout=0, dx=0)))
+        for over in (dict(), dict(x=FAKE_X + 2)):
+            assert unknown >= _demanded_workspace(bwd_params(layout=layout, **over)), (layout, over)
+
+
 def update_bwd_params(B=256, C=3456, S=3, dtype=1, **over):
     p = UpdateBwdParams()
     p.struct_size = ctypes.sizeof(UpdateBwdParams)

@@ -436,7 +436,9 @@ int plan_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_pa
 // ---------------------------------------------------------------------------
 // backward: planning and launch
 // ---------------------------------------------------------------------------
-int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointers)
+// check_pointers: the call itself (x, dout, dx, weight, dweight and the workspace must be there).  Without it
+// (queries) NULL pointers pass and count as aligned.  force_generic: plan the strided kernel whatever the layout.
+int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointers, bool force_generic = false)
 {
     if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(canon_conv1d_bwd_params))
@@ -512,9 +514,9 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     const int E = 16 / elem_bytes(p->x_dtype);
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
-    const bool ptrs16 = !check_pointers || (aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx));
+    const bool ptrs16 = aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx);
     // packed sequences and an initial state: only the walk kernel gates taps by sequence index / reads the history
-    const bool packed = p->seq_idx != nullptr || p->initial_state != nullptr || p->dfinal_state != nullptr;
+    const bool packed = force_generic || p->seq_idx != nullptr || p->initial_state != nullptr || p->dfinal_state != nullptr;
     const bool rows = !packed && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
                       a.d_sb % E == 0 && a.d_sc % E == 0;
@@ -550,7 +552,7 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     }
     // channel-contiguous tensors: 8-byte groups of channels per lane
     const int E8 = 8 / elem_bytes(p->x_dtype);
-    const bool ptrs8 = !check_pointers || ((((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0);
+    const bool ptrs8 = (((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0;
     const bool vec = !packed && a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
                      a.x_sb % E8 == 0 && a.x_sl % E8 == 0 && a.g_sb % E8 == 0 && a.g_sl % E8 == 0 &&
                      a.d_sb % E8 == 0 && a.d_sl % E8 == 0 && ptrs8;
@@ -792,7 +794,14 @@ CANON_API int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params
 {
     BwdPlan pl;
     if (plan_bwd(p, &pl, false) != CANON_OK) return -1;
-    return pl.workspace_bytes;
+    int64_t need = pl.workspace_bytes;
+    // Which kernel runs depends on the alignment of x, dout and dx as well.  With all three given the answer is that
+    // of the call; with one missing it covers the strided kernel too, which a misaligned pointer would select.
+    if (!p->x || !p->dout || !p->dx) {
+        if (plan_bwd(p, &pl, false, true) != CANON_OK) return -1;
+        if (pl.workspace_bytes > need) need = pl.workspace_bytes;
+    }
+    return need;
 }
 
 CANON_API int canon_conv1d_update_bwd(const canon_conv1d_update_bwd_params *p, void *stream)

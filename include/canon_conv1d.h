@@ -336,6 +336,24 @@ int canon_conv1d_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_
 int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_conv1d_part *parts, int32_t nparts,
                               void *stream);
 
+/*
+ * canon_conv1d_bwd for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same arguments and results as
+ * canon_conv1d_bwd, except that p->workspace / p->workspace_bytes are ignored:
+ * the partial sums of dweight / dbias go to a buffer of
+ * CANON_CONV1D_STATIC_SCRATCH_BYTES that is part of the library's device image
+ * (every GPU the library runs on holds its own copy until the process ends).
+ * Nothing is allocated or freed, by the library or by the runtime on its
+ * behalf.  A problem whose scratch exceeds the buffer is rejected with
+ * CANON_ERR_UNSUPPORTED (the metric shape, bf16 [8, 3456, 1024], needs 2.2 MB).
+ * All calls on one GPU share that GPU's buffer: calls that overlap in time on
+ * one GPU (different streams, different threads) race and must be serialised
+ * by the caller; calls that follow each other on one stream are safe.
+ */
+#define CANON_CONV1D_STATIC_SCRATCH_BYTES (8 << 20)
+int canon_conv1d_bwd_static(const canon_conv1d_bwd_params *p, void *stream);
+
 /* Scratch bytes canon_conv1d_bwd needs for these sizes, strides and pointer
  * alignments; with x, dout or dx missing (NULL) the figure also covers the
  * kernel a misaligned pointer would select.  Negative if the arguments are

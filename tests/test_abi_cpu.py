@@ -368,6 +368,13 @@ def test_bwd_workspace_query_covers_misaligned_pointers():
             assert unknown >= _demanded_workspace(bwd_params(layout=layout, **over)), (layout, over)
 
 
+def test_static_scratch_backward_checks_on_the_host():
+    L = _lib.lib()
+    assert L.canon_conv1d_bwd_static(None, None) == _lib.ERR_INVALID_ARGUMENT
+    assert L.canon_conv1d_bwd_static(ctypes.byref(bwd_params(struct_size=4)), None) == _lib.ERR_INVALID_ARGUMENT
+    assert "struct_size" in last_error()
+
+
 def update_bwd_params(B=256, C=3456, S=3, dtype=1, **over):
     p = UpdateBwdParams()
     p.struct_size = ctypes.sizeof(UpdateBwdParams)

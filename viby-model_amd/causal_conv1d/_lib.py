@@ -123,6 +123,7 @@ EXPORTS = (
     "canon_conv1d_fwd_plan",
     "canon_conv1d_update_plan",
     "canon_conv1d_bwd",
+    "canon_conv1d_bwd_static",
     "canon_conv1d_bwd_workspace_bytes",
     "canon_conv1d_bwd_plan",
     "canon_conv1d_update_bwd",
@@ -159,6 +160,8 @@ def lib() -> ctypes.CDLL:
         L.canon_conv1d_update_plan.argtypes = [ctypes.POINTER(UpdateParams)]
         L.canon_conv1d_bwd.restype = ctypes.c_int
         L.canon_conv1d_bwd.argtypes = [ctypes.POINTER(BwdParams), _vp]
+        L.canon_conv1d_bwd_static.restype = ctypes.c_int
+        L.canon_conv1d_bwd_static.argtypes = [ctypes.POINTER(BwdParams), _vp]
         L.canon_conv1d_bwd_workspace_bytes.restype = ctypes.c_int64
         L.canon_conv1d_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdParams)]
         L.canon_conv1d_bwd_plan.restype = ctypes.c_char_p

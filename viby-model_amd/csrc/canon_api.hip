@@ -1,7 +1,9 @@
 // libcanon_conv1d.so, host side: argument validation, choice of kernel family
 // and launch geometry (the plan), and the extern "C" entry points declared in
-// include/canon_conv1d.h.  No device code in this file.
+// include/canon_conv1d.h.  No kernels in this file; the only device object is
+// the static scratch array of canon_conv1d_bwd_static.
 #include <stdarg.h>
+#include <mutex>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -802,6 +804,52 @@ CANON_API int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params
         if (pl.workspace_bytes > need) need = pl.workspace_bytes;
     }
     return need;
+}
+
+// The scratch of canon_conv1d_bwd_static: one copy per GPU, at its own address on each.  On the host the
+// array's name is only a handle for hipGetSymbolAddress; kernels and fills take the device address it returns.
+constexpr int64_t kStaticScratchBytes = CANON_CONV1D_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+CANON_API int canon_conv1d_bwd_static(const canon_conv1d_bwd_params *p, void *stream)
+{
+    if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
+    if (p->struct_size != sizeof(canon_conv1d_bwd_params))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_bwd_params (%zu)",
+                    p->struct_size, sizeof(canon_conv1d_bwd_params));
+    // device address of this GPU's copy, looked up once per device
+    constexpr int kMaxDevices = 64;
+    static void *ptr_of_device[kMaxDevices];
+    static std::mutex lookup;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "canon_conv1d_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(CANON_ERR_UNSUPPORTED, "canon_conv1d_bwd_static: device %d", dev);
+    void *ptr;
+    {
+        std::lock_guard<std::mutex> hold(lookup);
+        if (!ptr_of_device[dev]) {
+            void *q = nullptr;
+            e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !q)
+                return fail(CANON_ERR_LAUNCH, "canon_conv1d_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            ptr_of_device[dev] = q;
+        }
+        ptr = ptr_of_device[dev];
+    }
+    canon_conv1d_bwd_params q = *p;
+    q.workspace = ptr;
+    q.workspace_bytes = kStaticScratchBytes;
+    BwdPlan pl;
+    int rc = plan_bwd(&q, &pl, false);
+    if (rc != CANON_OK) return rc;
+    if (pl.workspace_bytes > kStaticScratchBytes)
+        return fail(CANON_ERR_UNSUPPORTED,
+                    "canon_conv1d_bwd_static: this problem needs %lld bytes of scratch, the library's static buffer holds %lld; "
+                    "use canon_conv1d_bwd with a workspace of the caller's",
+                    (long long)pl.workspace_bytes, (long long)kStaticScratchBytes);
+    // every partial set the reduction reads is written by this launch first: nothing of an earlier call is read
+    return canon_conv1d_bwd(&q, stream);
 }
 
 CANON_API int canon_conv1d_update_bwd(const canon_conv1d_update_bwd_params *p, void *stream)

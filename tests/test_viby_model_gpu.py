@@ -1,63 +1,17 @@
 """Benchmark configuration 5: a Viby-shaped model (tests/viby_harness.py) run with the HIP Canon layers
 and with reference Canon back ends inside an otherwise identical network."""
 import time
-import types
 
 import pytest
 import torch
 from torch import nn
 
+from canon_backends import NoCanon, OracleCanon, TorchEagerCanon, hip_factory
 from helpers import bits
-from oracle import canon_oracle as co
-from oracle.canon_eager import EagerCanon
 from viby_harness import generate_graphed, VibyShaped, init_weights, viby_config
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-
-
-class TorchEagerCanon(nn.Module):
-    """The eager restatement (plain torch ops) on whatever device the input lives on."""
-
-    def __init__(self, C, cfg, name):
-        super().__init__()
-        self.name = name
-        self.weight = nn.Parameter(torch.randn(C, 1, cfg.canon_kernel))
-        self.act = cfg.canon_activation
-
-    def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
-        store = cache.__dict__.setdefault("eager_states", {})
-        return EagerCanon(self.weight, None, self.act).forward(x, attention_mask, store, (self.name, layer_idx))
-
-
-class OracleCanon(nn.Module):
-    """The C oracle on the host (eager rounding points), called with the semantics of the eager CanonLayer."""
-
-    def __init__(self, C, cfg, name, round_mode):
-        super().__init__()
-        self.name, self.K, self.round_mode = name, cfg.canon_kernel, round_mode
-        self.weight = nn.Parameter(torch.randn(C, 1, cfg.canon_kernel))
-
-    def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
-        store = cache.__dict__.setdefault("oracle_states", {})
-        key = (self.name, layer_idx)
-        xc, w = x.detach().cpu(), self.weight.detach().cpu().squeeze(1)
-        B, T, D = xc.shape
-        if T == 1 and key in store:
-            tok = xc[:, 0]
-            xt = (tok * attention_mask[:, -1].cpu().unsqueeze(-1).to(tok.dtype)) if attention_mask is not None else tok
-            y = co.conv1d_update(xt.contiguous(), store[key], w, None, round_mode=1)
-            return (tok + y).unsqueeze(1).to(x.device)     # residual on the unmasked token, rounded
-        mask = attention_mask.cpu() if attention_mask is not None else None
-        out, fs = co.conv1d_fwd(xc.transpose(1, 2), w, None, mask=mask, final_state_len=max(8, self.K),
-                                residual=1, round_mode=1)
-        store[key] = fs
-        return out.transpose(1, 2).contiguous().to(x.device)
-
-
-def hip_factory(cfg, rounding):
-    from causal_conv1d.canon import CanonLayer
-    return lambda C, name: CanonLayer(C, cfg, name, rounding=rounding)
 
 
 def test_small_model_hip_equals_oracle_bit_for_bit():
@@ -114,7 +68,7 @@ def test_model_with_concat_free_canon_b_d_is_bit_identical(capsys):
               f"parts {times['parts']:.3f} s")
 
 
-def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
+def test_config5_full_model_fused_rounding_timing_and_noise_bound(capsys):
     cfg = viby_config()
     B, T, steps = 16, 1024, 128
     ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(5)).to(DEV)
@@ -143,9 +97,6 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
 
     # the same network with the Canon layers switched off: what is left is everything else (projections,
     # attention, norms, python), so the difference is the share of the 72 Canon calls per forward
-    class NoCanon(torch.nn.Module):
-        def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
-            return x
     bare = init_weights(VibyShaped(cfg, lambda C, n: NoCanon()), 11, torch.bfloat16, DEV)
     bare.generate(ids[:2, :64], 2)
     torch.cuda.synchronize()
@@ -156,8 +107,9 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
     del bare
     torch.cuda.empty_cache()
 
-    # the HIP layers round once where the eager module rounds three times: logits agree to bf16
-    # noise accumulated over 18 layers, and the greedy choice agrees wherever it is not a near tie
+    # A second, weaker check beside the bit-exact one above: in the default rounding mode the HIP layers round once
+    # where the eager module rounds three times, so logits agree to bf16 noise accumulated over 18 layers and the
+    # greedy choice agrees wherever it is not a near tie
     diff = (logits - logits_r).abs()
     scale = logits_r.abs().max().item()
     assert diff.max().item() <= 0.05 * scale, (diff.max().item(), scale)
@@ -173,6 +125,36 @@ def test_config5_full_model_prefill_and_128_greedy_steps(capsys):
               f"greedy tokens equal at {agree.float().mean().item() * 100:.1f} % of steps "
               f"({decided.float().mean().item() * 100:.1f} % decided beyond rounding noise), "
               f"max |dlogit| {diff.max().item():.4f} of scale {scale:.2f}")
+
+
+def test_config5_full_size_eager_rounding_equals_the_cpu_eager_module_bit_for_bit(capsys):
+    """Configuration 5 by its own criterion: 18 layers, B16 x L1024 prefill, 128 greedy steps through the conv
+    caches, bf16.  The HIP Canon layers with the eager module's rounding points against the eager module itself
+    (torch operations on the host, the reference's CPU path) inside the same network: identical greedy tokens,
+    identical logits at every step and all 72 conv states equal bit for bit.  Both runs decode freely (no
+    teacher forcing): one differing bit anywhere would show."""
+    cfg = viby_config()
+    B, T, steps = 16, 1024, 128
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(5)).to(DEV)
+    hip = init_weights(VibyShaped(cfg, hip_factory(cfg, "eager")), 11, torch.bfloat16, DEV)
+    toks, logits, cache = hip.generate(ids, steps)
+    states = {(site, layer): getattr(cache, f"canon_cache_{site}")[layer].cpu()
+              for site in "abcd" for layer in range(cfg.num_hidden_layers)}
+    del hip, cache
+    torch.cuda.empty_cache()
+    ref = init_weights(VibyShaped(cfg, lambda C, n: TorchEagerCanon(C, cfg, n, host=True)), 11, torch.bfloat16, DEV)
+    t0 = time.perf_counter()
+    toks_r, logits_r, cache_r = ref.generate(ids, steps)
+    torch.cuda.synchronize()
+    t_ref = time.perf_counter() - t0
+    assert len(states) == 72
+    assert torch.equal(toks, toks_r), f"greedy tokens differ first at step {(toks != toks_r).any(0).nonzero()[0].item()}"
+    assert torch.equal(bits(logits.bfloat16()), bits(logits_r.bfloat16())) and torch.equal(logits, logits_r)
+    for key, got in states.items():
+        assert torch.equal(bits(got), bits(cache_r.eager_states[key])), key
+    with capsys.disabled():
+        print(f"\n[config 5, eager rounding] B{B} x L{T} prefill + {steps} greedy steps: tokens, logits and all 72 conv "
+              f"states identical to the host eager module (which took {t_ref:.1f} s)")
 
 
 def test_config5_decode_as_one_hip_graph_per_token(capsys):

@@ -29,9 +29,21 @@ for p in (ROOT, os.path.join(ROOT, "viby-model_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, vendor figure
-# HBM bytes per launch of the headline kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
-# plain copy of known size (profiles/prefill_time_contiguous_bf16_B8_C3456_L1024.txt)
-MEASURED_TRAFFIC_BYTES = 113.54e6
+# HBM bytes per launch of the headline kernel as rocprofv3 counted them (FETCH_SIZE / WRITE_SIZE scaled by a plain
+# copy of known size): read from the committed summary of that profile, not measured by this run
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "prefill_time_contiguous_bf16_B8_C3456_L1024.txt")
+
+
+def profiled_traffic_bytes():
+    """'traffic per launch N MB' of the committed profile of the headline kernel, in bytes (None if absent)."""
+    import re
+    try:
+        m = re.search(r"traffic per launch ([0-9.]+) MB", open(TRAFFIC_PROFILE).read())
+    except OSError:
+        return None
+    return float(m.group(1)) * 1e6 if m else None
+
+
 B, C, L, W = 8, 3456, 1024, 4   # the configuration the metric is quoted on
 DEC_B, DEC_S, DEC_STEPS = 256, 3, 64
 
@@ -69,29 +81,38 @@ def time_region(fn, steps, warmup, ramp=True):
     return e0.elapsed_time(e1) / steps  # ms per step
 
 
-def bench_prefill(layout, steps, warmup, nbuf, ramp=True):
+def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None, rounding=0, with_mask=False):
+    """One prefill launch per step over `nbuf` rotating buffer pairs.  shape: (B, C, L), the metric's by default;
+    dtype: torch.bfloat16 by default; rounding: 0 fused, 1 the eager module's rounding points; with_mask: a
+    right-padded padding mask of x's type and the masked residual (what CanonLayer passes)."""
     import torch
     import causal_conv1d as cc
     from causal_conv1d import _lib
     dev = "cuda:0"
+    Bx, Cx, Lx = shape or (B, C, L)
+    dtype = dtype or torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(0)
-    w = (torch.randn(C, W, generator=g, device=dev) * 0.02).bfloat16()
-    bias = (torch.randn(C, generator=g, device=dev) * 0.01).bfloat16()
+    w = (torch.randn(Cx, W, generator=g, device=dev) * 0.02).to(dtype)
+    bias = (torch.randn(Cx, generator=g, device=dev) * 0.01).to(dtype)
+    mask = None
+    if with_mask:
+        lens = torch.randint(Lx // 8, Lx + 1, (Bx,), generator=g, device=dev)
+        mask = (torch.arange(Lx, device=dev)[None, :] < lens[:, None]).to(dtype)
     # all buffer pairs are carved out of ONE allocation, as an arena-allocating runtime would hold them:
     # measured 1 % faster than separately allocated tensors (fewer, larger address-translation fragments)
-    n = B * C * L
-    pool = torch.empty(2 * nbuf * n, dtype=torch.bfloat16, device=dev)
+    n = Bx * Cx * Lx
+    pool = torch.empty(2 * nbuf * n, dtype=dtype, device=dev)
     xs, outs, params = [], [], []
     for i in range(nbuf):
         x, o = pool[2 * i * n:(2 * i + 1) * n], pool[(2 * i + 1) * n:(2 * i + 2) * n]
         if layout == "bcl":
-            x, o = x.view(B, C, L), o.view(B, C, L)
+            x, o = x.view(Bx, Cx, Lx), o.view(Bx, Cx, Lx)
         else:
-            x, o = x.view(B, L, C).transpose(1, 2), o.view(B, L, C).transpose(1, 2)
+            x, o = x.view(Bx, Lx, Cx).transpose(1, 2), o.view(Bx, Lx, Cx).transpose(1, 2)
         x.copy_(torch.randn(x.shape, generator=g, device=dev))
         xs.append(x)
         outs.append(o)
-        params.append(cc._fill_fwd(x, o, w, bias, None, None, None, 0, 1, 0))
+        params.append(cc._fill_fwd(x, o, w, bias, mask, None, None, 0, 1, rounding))
     plan = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(params[0])).decode()
     fwd = _lib.lib().canon_conv1d_fwd
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -330,6 +351,102 @@ def bench_backward(steps, warmup, nbuf):
     return ms, plan, ws.numel()
 
 
+def bench_canon_shapes(steps, warmup):
+    """The other shapes the Canon layers are called with (reference: causal-conv1d-mps/bench.py:89-164 benches
+    Canon A/C, B and D): C = 640 (A, C), 960 (B), 3456 (D) at B8 L1024 bf16 in both layouts, the fp32 B1 C640
+    case of configuration 1, and the masked B16 calls of configuration 5's prefill.  These are small: a launch
+    moves 5-60 MB, so part of each figure is the cost of a launch itself (see launch_floor)."""
+    import torch
+    rows = []
+    cases = [("configs[1] Canon-A/C", (8, 640, 1024), torch.bfloat16, False),
+             ("configs[1] Canon-B", (8, 960, 1024), torch.bfloat16, False),
+             ("configs[0] Canon-A fp32", (1, 640, 1024), torch.float32, False),
+             ("configs[4] prefill Canon-A/C, padding mask", (16, 640, 1024), torch.bfloat16, True),
+             ("configs[4] prefill Canon-B, padding mask", (16, 960, 1024), torch.bfloat16, True),
+             ("configs[4] prefill Canon-D, padding mask", (16, 3456, 1024), torch.bfloat16, True)]
+    for what, shape, dtype, masked in cases:
+        esize = 4 if dtype == torch.float32 else 2
+        nbytes = prefill_bytes(*shape, esize, esize) + (shape[0] * shape[2] * esize if masked else 0)
+        nbuf = max(3, min(48, int(700e6 / nbytes) + 1))
+        row = {"workload": f"{what}: {'fp32' if esize == 4 else 'bf16'} x[{shape[0]},{shape[1]},{shape[2]}]", "bytes": nbytes}
+        for layout, key in (("bcl", "time_contiguous"), ("blc", "channel_last")):
+            ms, plan = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked)
+            row[key] = {"kernel": plan, "us_per_step": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        rows.append(row)
+    return rows
+
+
+def bench_launch_floor(steps, warmup):
+    """What one launch through this entry point costs when it moves next to nothing: canon_conv1d_update on a
+    [1, 8] token (one wave), back to back on the stream every other leg uses."""
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d import _lib
+    dev = "cuda:0"
+    x = torch.zeros(1, 8, dtype=torch.bfloat16, device=dev)
+    out, state = torch.empty_like(x), torch.zeros(1, 8, 3, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(8, W, dtype=torch.bfloat16, device=dev)
+    p = cc._fill_update(x, out, state, w, None, None, 0, 0, 0)
+    ref, upd = ctypes.byref(p), _lib.lib().canon_conv1d_update
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step(i):
+        rc = upd(ref, stream)
+        if rc:
+            _lib.check(rc, "canon_conv1d_update")
+
+    return time_region(step, steps, warmup) * 1e3
+
+
+def bench_decode_host_cost(calls=5000):
+    """Host time of one decode call through the Python API, no synchronisation inside the loop (the GPU side of
+    these calls is ~3 us, so the queue never fills): causal_conv1d_update and one CanonLayer.forward step at the
+    shapes of configuration 5 (B16, Canon-D, the eager module's 8-slot state)."""
+    import types
+    import torch
+    import causal_conv1d as cc
+    from causal_conv1d.canon import CanonLayer
+    dev = "cuda:0"
+    Bd, Cd = 16, C
+    x = torch.randn(Bd, Cd, device=dev).bfloat16()
+    state = torch.zeros(Bd, Cd, 8, dtype=torch.bfloat16, device=dev)
+    w = torch.randn(Cd, W, device=dev).bfloat16()
+    layer = CanonLayer(Cd, types.SimpleNamespace(canon_kernel=W, canon_bias=False, canon_activation=False), "d")
+    layer = layer.to(dev).to(torch.bfloat16)
+    cache = types.SimpleNamespace(_max_layers=1)
+    xt = torch.randn(Bd, 1, Cd, device=dev).bfloat16()
+    mask = torch.ones(Bd, 1100, dtype=torch.int64, device=dev)
+
+    def per_call(fn):
+        for _ in range(200):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        dt = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return dt / calls * 1e6
+
+    with torch.no_grad():
+        layer(xt.expand(Bd, 16, Cd).contiguous(), attention_mask=mask[:, :16], cache=cache, layer_idx=0)
+        return {"causal_conv1d_update": round(per_call(lambda: cc.causal_conv1d_update(x, state, w)), 2),
+                "canon_layer_step": round(per_call(lambda: layer(xt, attention_mask=mask, cache=cache, layer_idx=0)), 2),
+                "what": "host microseconds per call (time.perf_counter over %d calls, no sync), bf16 B16 C3456, "
+                        "8-slot state; the layer step includes the token mask and nn.Module.__call__" % calls}
+
+
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def _median_time(fn, budget_s, max_runs):
     fn()
     times = []
@@ -371,7 +488,7 @@ def cpu_baseline(budget_s=10.0):
     nbytes = prefill_bytes(B, C, L)
     return {
         "value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": cores,
-        "kind": "port",
+        "kind": "port", "cpu": _cpu_model(), "torch": torch.__version__,
         "sample": f"{n} passes of the full bf16 [8,3456,1024] step, eager torch restatement "
                   f"(oracle/canon_eager.py), median {med * 1e3:.1f} ms",
         "ms": round(med * 1e3, 2), "tokens_per_s": round(B * L / med),
@@ -416,6 +533,7 @@ def main():
     ms_warm, _ = bench_prefill("bcl", max(20, args.steps // 10), 5, 1, ramp=False)
     ms_copy = bench_copy(args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
+    ms_blc_eager, plan_blc_eager = bench_prefill("blc", args.steps, args.warmup, nbuf, rounding=1)
     ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
     rag_steps, rag_warm = max(20, args.steps // 4), max(4, args.warmup // 4)
     ms_rag, plan_rag, rag_bytes = bench_ragged("blc", rag_steps, rag_warm, 3)     # 3 x 453 MB between reuses
@@ -424,6 +542,9 @@ def main():
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
     us_dbwd, dbwd_bytes, ws_dbwd = bench_decode_backward(max(50, args.steps), max(5, args.warmup))
+    shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
+    floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
+    host_cost = bench_decode_host_cost()
 
     nbytes = prefill_bytes(B, C, L)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -443,7 +564,12 @@ def main():
                                  "what": "the headline launch repeated on ONE buffer pair (113 MB, inside the 256 MB "
                                          "Infinity Cache): a cache rate, reported beside the HBM rate, never as it"},
         "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
-                                 "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1)},
+                                 "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1),
+                                 "frac_of_hbm_peak": round(nbytes / (ms_blc * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+        "prefill_channel_last_eager_rounding": {"kernel": plan_blc_eager, "ms_per_step": round(ms_blc_eager, 6),
+                                                "GB/s": round(nbytes / (ms_blc_eager * 1e-3) / 1e9, 1),
+                                                "what": "the same launch with round_mode = eager (the eager module's "
+                                                        "rounding points: bit-identical to the reference's CPU path)"},
         "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",
                                        "kernel": plan_parts, "ms_per_step": round(ms_parts, 6),
                                        "GB/s": round(nbytes / (ms_parts * 1e-3) / 1e9, 1)},
@@ -457,7 +583,12 @@ def main():
         "decode": {"workload": f"configs[3]: bf16 state[{DEC_B},{C},{DEC_S}], {DEC_STEPS} carried steps",
                    "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
                    "us_per_step_hipgraph": round(dec_graph_us, 3),
-                   "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1)},
+                   "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1),
+                   "host_us_per_call": host_cost},
+        "canon_shapes": shapes,
+        "launch_floor": {"us_per_launch": round(floor_us, 3),
+                         "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what "
+                                 "a launch costs before it moves any data; every us_per_step above includes it"},
         "backward_channel_last": {"kernel": plan_bwd, "ms_per_step": round(ms_bwd, 6),
                                   "GB/s": round(1.5 * nbytes / (ms_bwd * 1e-3) / 1e9, 1),
                                   "bytes": "x and dout read, dx written (3 tensor passes)",
@@ -467,7 +598,8 @@ def main():
                             "us_per_step": round(us_dbwd, 3),
                             "GB/s": round(dbwd_bytes / (us_dbwd * 1e-6) / 1e9, 1), "scratch_bytes": ws_dbwd},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": profiled_traffic_bytes(),
+                     "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE)},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

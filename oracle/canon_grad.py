@@ -8,8 +8,9 @@ gradients are what ``loss.backward()`` of the reference computes
 (trainer/base_trainer.py:274).  Everything is evaluated in float64 from the
 quantised inputs, so the result is the exact-arithmetic gradient up to 1e-15.
 
-With ``seq_idx`` (packed sequences, the varlen contract of
-causal_conv1d_mps/causal_conv1d_interface.py:253-261) a tap contributes only
+With ``seq_idx`` (packed sequences: the slot of the call signature that the
+reference passes as None, model/model.py:465, and that its MPS back end rejects,
+causal_conv1d_mps/autograd.py:64-65) a tap contributes only
 when its time step carries the same sequence index as the output step, so the
 convolution is written as a sum of shifted, gated copies of ``xm``.  That
 form is pinned by the tests in two ways: its output against the C oracle of

@@ -291,7 +291,9 @@ int canon_oracle_update(const void *x, void *conv_state, const void *weight, con
  * Decode update with the two state-addressing modes of the upstream call
  * signature that the reference never uses (model/model.py:305-311 passes
  * neither; the signature slots are listed at causal_conv1d_mps/__init__.py:304-312):
- *   conv_state_indices[b]  row of conv_state (a pool of `rows` rows) used by batch entry b
+ *   conv_state_indices[b]  row of conv_state (a pool of `rows` rows) used by batch entry b; an entry whose
+ *                          index is negative or not below `rows` is skipped (upstream's padding slots):
+ *                          no state row is touched and its row of out is left as it was
  *   cache_seqlens[b]       circular-buffer mode: the token is written to slot
  *                          cache_seqlens[b] % S, the W-1 slots before it
  *                          (cyclically) are the history, nothing is shifted
@@ -302,12 +304,13 @@ int canon_oracle_update(const void *x, void *conv_state, const void *weight, con
  */
 int canon_oracle_update_ext(const void *x, void *conv_state, const void *weight, const void *bias, void *out,
                             int64_t B, int64_t C, int W, int S, int dtype, int w_dtype, int use_silu,
-                            int residual, const int32_t *cache_seqlens, const int32_t *conv_state_indices)
+                            int residual, const int32_t *cache_seqlens, const int32_t *conv_state_indices, int64_t rows)
 {
     if (W < 1 || W > 8 || S < 1 || S < W - 1 || B < 0 || C < 0) return -1;
     const size_t es = (dtype == CANON_F32) ? 4 : 2;
     for (int64_t b = 0; b < B; ++b) {
         const int64_t srow = conv_state_indices ? conv_state_indices[b] : b;
+        if (conv_state_indices && (srow < 0 || srow >= rows)) continue;
         for (int64_t c = 0; c < C; ++c) {
             const int64_t r = b * C + c, sr = srow * C + c;
             float w[8], window[8];

@@ -43,7 +43,7 @@ def lib() -> ctypes.CDLL:
         L.canon_oracle_fwd_seq.restype = i32
         L.canon_oracle_fwd_seq.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, i32, i32, i32, i32]
         L.canon_oracle_update_ext.restype = i32
-        L.canon_oracle_update_ext.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i32, i32, vp, vp]
+        L.canon_oracle_update_ext.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i32, i32, vp, vp, i64]
         L.canon_oracle_update.restype = i32
         L.canon_oracle_update.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32,
                                           i32, i32, i32, i32, i32]
@@ -193,7 +193,8 @@ def conv1d_update_ext(
     conv_state_indices: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Decode-step oracle with circular-buffer (``cache_seqlens``) and state-pool (``conv_state_indices``)
-    addressing; ``conv_state`` (rows, C, S), contiguous, is updated in place.  See ``canon_oracle_update_ext``."""
+    addressing; ``conv_state`` (rows, C, S), contiguous, is updated in place.  Entries whose index lies outside
+    the pool are skipped: their output rows are zero.  See ``canon_oracle_update_ext``."""
     assert x.dim() == 2 and conv_state.dim() == 3 and conv_state.is_contiguous() and x.device.type == "cpu"
     B, C = x.shape
     assert conv_state.shape[1] == C and conv_state.dtype == x.dtype
@@ -204,10 +205,11 @@ def conv1d_update_ext(
     ix = conv_state_indices.to(torch.int32).contiguous() if conv_state_indices is not None else None
     if ix is None:
         assert conv_state.shape[0] == B
-    out = torch.empty_like(xc)
+    out = torch.zeros_like(xc)
     rc = lib().canon_oracle_update_ext(
         _ptr(xc), _ptr(conv_state), _ptr(wc), _ptr(bc), _ptr(out), B, C, weight.shape[1], S,
-        _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype], _act(activation), int(bool(residual)), _ptr(sl), _ptr(ix))
+        _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype], _act(activation), int(bool(residual)), _ptr(sl), _ptr(ix),
+        conv_state.shape[0])
     if rc != 0:
         raise ValueError("canon_oracle_update_ext rejected its arguments")
     return out

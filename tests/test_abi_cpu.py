@@ -133,6 +133,7 @@ def test_fwd_validation_messages():
         (dict(round_mode=2), "round_mode"),
         (dict(batch=-1), "negative"),
         (dict(out=FAKE_X), "alias"),
+        (dict(out=FAKE_X + 4096), "ranges overlap"),                      # a shifted view of the same buffer
         (dict(x=0), "NULL"),
         (dict(mask=FAKE_STATE, mask_dtype=17), "mask_dtype"),
         (dict(initial_state=FAKE_STATE, initial_len=2), "initial_len"),
@@ -373,6 +374,24 @@ def test_static_scratch_backward_checks_on_the_host():
     assert L.canon_conv1d_bwd_static(None, None) == _lib.ERR_INVALID_ARGUMENT
     assert L.canon_conv1d_bwd_static(ctypes.byref(bwd_params(struct_size=4)), None) == _lib.ERR_INVALID_ARGUMENT
     assert "struct_size" in last_error()
+
+
+def test_mask_narrowing_works_on_inference_tensors():
+    """An int64 padding mask is converted to x's type once and cached on its identity and version; tensors made
+    under torch.inference_mode() have no version counter, so they are converted without the cache."""
+    import causal_conv1d as cc
+    x = torch.zeros(2, 4, 8, dtype=torch.bfloat16)
+    big = cc._NARROW_MIN_ELEMENTS
+    mask = torch.ones(2, 8, dtype=torch.int64)
+    first = cc._narrow_mask(mask, x, big)
+    assert first.dtype == torch.bfloat16 and cc._narrow_mask(mask, x, big) is first          # cached
+    assert cc._narrow_mask(mask, x, big - 1) is mask                                         # small problems: as given
+    with torch.inference_mode():
+        imask = torch.ones(2, 8, dtype=torch.int64)
+        got = cc._narrow_mask(imask, x, big)
+        assert got.dtype == torch.bfloat16 and torch.equal(got.float(), imask.float())
+    mask[0, 3] = 0                                                                           # a new version: converted again
+    assert cc._narrow_mask(mask, x, big)[0, 3].item() == 0
 
 
 def update_bwd_params(B=256, C=3456, S=3, dtype=1, **over):

@@ -479,6 +479,16 @@ def test_ring_buffer_and_state_pool_update_equal_the_shift_register():
             assert torch.equal(pool[rows_of.long()], shift)
         others = [r for r in range(rows) if r not in rows_of.tolist()]
         assert torch.equal(pool[others], untouched[others])
+        # entries whose index lies outside the pool are skipped: the rest is the call without them
+        before = pool.clone()
+        x = torch.randn(B, C, generator=g).to(dtype)
+        want = co.conv1d_update_ext(x[1:2], pool, w, b, activation="silu", residual=True, conv_state_indices=rows_of[1:2])
+        after = pool.clone()
+        pool.copy_(before)
+        got = co.conv1d_update_ext(x, pool, w, b, activation="silu", residual=True,
+                                   conv_state_indices=torch.tensor([-1, int(rows_of[1]), rows], dtype=torch.int32))
+        assert torch.equal(got[1:2], want) and torch.equal(pool, after)
+        assert not got[0].any() and not got[2].any()
 
 
 def test_update_gradient_oracle_chained_equals_the_prefill_gradient_oracle():

@@ -22,6 +22,7 @@ or a rejected call raises.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import List, Optional, Tuple, Union
 
 import torch
@@ -137,6 +138,8 @@ def _narrow_mask(mask: torch.Tensor, x: torch.Tensor, numel: int) -> torch.Tenso
         return mask
     if torch.compiler.is_compiling():
         return mask.to(x.dtype)      # one node of the traced graph; identical conversions are merged there
+    if mask.is_inference():
+        return mask.to(x.dtype)      # tensors made under torch.inference_mode() carry no version counter to key on
     global _narrow_cache
     key = (mask.data_ptr(), mask._version, tuple(mask.shape), mask.stride(), mask.dtype, x.dtype, mask.device)
     entry = _narrow_cache
@@ -257,7 +260,11 @@ def causal_conv1d_fn(
     ``out[b,c,t] = act(bias[c] + sum_k weight[c,k] * x[b,c,t-(W-1)+k])`` with
     fp32 accumulation and one rounding to ``x.dtype``.  ``x`` may be time
     contiguous or channel contiguous (a transposed (batch, seqlen, dim) tensor,
-    which is what ``model/model.py:459`` passes); the output has x's strides.
+    which is what ``model/model.py:459`` passes): both run vectorised kernels.
+    Any other strides are read as they are by a strided kernel (several times
+    slower; nothing is copied).  The output is ``torch.empty_like(x)``: x's
+    strides when x is dense in some order of its dimensions, contiguous
+    (batch, dim, seqlen) otherwise.
 
     seq_idx          (batch, seqlen) int32: packed variable-length sequences; positions
                      with different values do not see each other (the slot the
@@ -295,8 +302,6 @@ def causal_conv1d_fn(
     bias, attention_mask, final_states = _check_fwd_args(
         x, tuple(x.shape), weight, bias, attention_mask, initial_states, return_final_states, final_states_out)
 
-    if x.stride(2) != 1 and x.stride(1) != 1:
-        x = x.contiguous()
     if x.numel() == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
@@ -495,6 +500,32 @@ def causal_conv1d_update(
     rounding    'fused' | 'eager' (the rounding points of
                 ``model/model.py:385-396``).
     """
+    # A serving loop makes this call 72 times per generated token with the same shapes, strides, types and flags:
+    # such a call, once it has passed every check below, is recognised by that signature and launched from a
+    # prepared argument block with only the five addresses filled in.
+    if cache_seqlens is None and conv_state_indices is None and not (
+            torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad or conv_state.requires_grad
+                                         or (bias is not None and bias.requires_grad))):
+        key = (x.shape, x.stride(), x.dtype, x.device, conv_state.shape, conv_state.stride(), conv_state.dtype,
+               conv_state.device, weight.shape, weight.stride(), weight.dtype, weight.device,
+               None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device),
+               None if token_mask is None else (token_mask.shape, token_mask.stride(), token_mask.dtype, token_mask.device),
+               activation, residual, rounding)
+        known = _known_updates()
+        p = known.get(key)
+        if p is not None and not torch.compiler.is_compiling():
+            out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+            p.x, p.out, p.conv_state, p.weight = x.data_ptr(), out.data_ptr(), conv_state.data_ptr(), weight.data_ptr()
+            if bias is not None:
+                p.bias = bias.data_ptr()
+            if token_mask is not None:
+                p.token_mask = token_mask.data_ptr()
+            rc = _call(_lib.lib().canon_conv1d_update, x.device, ctypes.byref(p))
+            if rc:
+                _lib.check(rc, "causal_conv1d_update")
+            return out
+    else:
+        key = None
     act = _activation_flag(activation)
     res = _residual_mode(residual)
     rnd = _round_mode(rounding)
@@ -550,7 +581,66 @@ def causal_conv1d_update(
                                             act, res, rnd)
     else:
         out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
+        if (key is not None and not squeeze_back and out.numel() and len(_known_updates()) < _KNOWN_UPDATES_MAX
+                and (bias is None or (bias.dtype == weight.dtype and bias.is_contiguous()))):
+            # the call went through: remember its signature with an argument block whose sizes, strides and flags are set
+            _known_updates()[key] = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
     return out.unsqueeze(-1) if squeeze_back else out
+
+
+def _canon_decode_step(x: torch.Tensor, conv_state: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
+                       attention_mask: Optional[torch.Tensor], activation: Optional[str], rounding: str) -> torch.Tensor:
+    """The single-token call of ``canon.CanonLayer`` (inference): ``x`` is the layer's (batch, 1, dim) input as it
+    is, ``attention_mask`` the whole-history (batch, >= 1) mask whose LAST column scales the token, the residual
+    is the unmasked token; returns (batch, 1, dim).  Same kernel and same checks as ``causal_conv1d_update`` on
+    ``x[:, 0]`` / ``attention_mask[:, -1]``, without building those views and the output's: a signature that
+    has been through ``causal_conv1d_update`` once is launched from its prepared argument block."""
+    if torch.compiler.is_compiling():
+        token_mask = attention_mask[:, -1] if attention_mask is not None else None
+        return causal_conv1d_update(x[:, 0], conv_state, taps, bias, activation=activation, token_mask=token_mask,
+                                    residual="unmasked", rounding=rounding).unsqueeze(1)
+    key = (x.shape, x.stride(), x.dtype, x.device, conv_state.shape, conv_state.stride(), conv_state.dtype,
+           conv_state.device, taps.shape, taps.stride(), taps.dtype, taps.device,
+           None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device),
+           None if attention_mask is None else (attention_mask.shape[0], attention_mask.stride(1), attention_mask.dtype,
+                                                attention_mask.device),
+           activation, rounding)
+    known = _known_updates()
+    p = known.get(key)
+    if p is None:
+        token_mask = attention_mask[:, -1] if attention_mask is not None else None
+        y = causal_conv1d_update(x[:, 0], conv_state, taps, bias, activation=activation, token_mask=token_mask,
+                                 residual="unmasked", rounding=rounding)
+        if y.numel() and len(known) < _KNOWN_UPDATES_MAX and (
+                bias is None or (bias.dtype == taps.dtype and bias.is_contiguous())):
+            # x[:, 0] and a contiguous (batch, dim) output: the strides of every later call with this signature
+            known[key] = _fill_update(x[:, 0], y, conv_state, taps, bias, token_mask, _activation_flag(activation),
+                                      _residual_mode("unmasked"), _round_mode(rounding))
+        return y.unsqueeze(1)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    p.x, p.out, p.conv_state, p.weight = x.data_ptr(), out.data_ptr(), conv_state.data_ptr(), taps.data_ptr()
+    if bias is not None:
+        p.bias = bias.data_ptr()
+    if attention_mask is not None:
+        p.token_mask = attention_mask.data_ptr() + (attention_mask.shape[1] - 1) * attention_mask.stride(1) * attention_mask.element_size()
+        p.mask_stride_b = attention_mask.stride(0)
+    rc = _call(_lib.lib().canon_conv1d_update, x.device, ctypes.byref(p))
+    if rc:
+        _lib.check(rc, "causal_conv1d_update")
+    return out
+
+
+# signature of a checked decode call -> its prepared argument block; per thread, because the block is written to
+_KNOWN_UPDATES_MAX = 256
+_update_tls = threading.local()
+
+
+def _known_updates() -> dict:
+    try:
+        return _update_tls.known
+    except AttributeError:
+        _update_tls.known = {}
+        return _update_tls.known
 
 
 def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
@@ -727,7 +817,6 @@ def causal_conv1d_fn_parts(
     if batch * dim * seqlen == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
-    xs = [x if (x.stride(2) == 1 or x.stride(1) == 1) else x.contiguous() for x in xs]
     if _wants_grad(*xs, weight, bias) and initial_states is not None:
         raise NotImplementedError("gradients through a call with initial_states are not implemented")
     if torch.compiler.is_compiling():

@@ -48,7 +48,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from . import causal_conv1d_fn, causal_conv1d_fn_parts, causal_conv1d_update, causal_conv1d_update_parts
+from . import (_canon_decode_step, causal_conv1d_fn, causal_conv1d_fn_parts, causal_conv1d_update,
+               causal_conv1d_update_parts)
 
 STATE_LEN_MIN = 8  # model/model.py:286, :626
 
@@ -67,6 +68,7 @@ class CanonLayer(nn.Module):
             self.bias_param = nn.Parameter(torch.zeros(hidden_size))
         else:
             self.register_parameter("bias_param", None)
+        self._taps_view = None   # (address of the weight, its (C, K) view): see _taps
 
     def reset_parameters(self) -> None:
         nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
@@ -95,24 +97,42 @@ class CanonLayer(nn.Module):
                 return attention_mask[:, -T:]
         return None
 
+    def _taps(self) -> torch.Tensor:
+        """``weight`` as (C, K).  Outside autograd the view is kept (it stays valid while the parameter keeps its
+        storage; in-place updates show through it), which saves the decode step a tensor operation."""
+        w = self.weight
+        if torch.is_grad_enabled() and w.requires_grad:
+            return w.squeeze(1)
+        kept = self._taps_view
+        if kept is None or kept[0] != w.data_ptr() or kept[1].device != w.device or kept[1].dtype != w.dtype:
+            kept = (w.data_ptr(), w.detach().squeeze(1))
+            self._taps_view = kept
+        return kept[1]
+
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 cache=None, layer_idx: Optional[int] = None) -> torch.Tensor:
         B, T, D = x.shape
         use_cache = cache is not None and layer_idx is not None
-        state = self._slot(cache)[layer_idx] if use_cache else None
-        taps = self.weight.squeeze(1)
         act = "silu" if self.activation else None
 
         if use_cache and T == 1:
-            token_mask = None
+            slot = self._slot(cache)
+            state = slot[layer_idx]
+            token_mask = None          # the whole mask here: its last column scales the token (model/model.py:277-282)
             if attention_mask is not None and attention_mask.dim() == 2 and attention_mask.shape[0] == B:
-                token_mask = attention_mask[:, -1]
+                token_mask = attention_mask
             if state is None:
                 state = torch.zeros(B, D, self._state_len(), dtype=x.dtype, device=x.device)
-            y = causal_conv1d_update(x[:, 0], state, taps, self.bias_param, activation=act,
-                                     token_mask=token_mask, residual="unmasked", rounding=self.rounding)
-            self._slot(cache)[layer_idx] = state
-            return y.unsqueeze(1)
+                slot[layer_idx] = state
+            if torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad or state.requires_grad):
+                y = causal_conv1d_update(x[:, 0], state, self._taps(), self.bias_param, activation=act,
+                                         token_mask=token_mask[:, -1] if token_mask is not None else None,
+                                         residual="unmasked", rounding=self.rounding)
+                return y.unsqueeze(1)
+            return _canon_decode_step(x, state, self._taps(), self.bias_param, token_mask, act, self.rounding)
+
+        state = self._slot(cache)[layer_idx] if use_cache else None
+        taps = self._taps()
 
         mask = self._block_mask(attention_mask, B, T)
 
@@ -144,7 +164,7 @@ class CanonLayer(nn.Module):
             raise ValueError(f"the parts hold {D} channels, the layer has {self.hidden_size}")
         use_cache = cache is not None and layer_idx is not None
         state = self._slot(cache)[layer_idx] if use_cache else None
-        taps = self.weight.squeeze(1)
+        taps = self._taps()
         act = "silu" if self.activation else None
 
         if use_cache and T == 1:

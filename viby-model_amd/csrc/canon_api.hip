@@ -67,6 +67,27 @@ bool mask_run_aligned(const void *mask, int mask_dtype, int64_t stride_b, int64_
     return ((uintptr_t)mask % align) == 0 && (stride_b * msize[mask_dtype]) % align == 0;
 }
 
+// Byte range [lo, hi) that a [B, C, L] tensor with these element strides touches, and whether it fills it.
+struct Extent {
+    uintptr_t lo, hi;
+    bool dense;
+};
+
+Extent extent_of(const void *base, int64_t B, int64_t C, int64_t L, int64_t sb, int64_t sc, int64_t sl, int bytes)
+{
+    int64_t lo = 0, hi = 0;   // smallest / largest element offset
+    const int64_t n[3] = {B - 1, C - 1, L - 1}, s[3] = {sb, sc, sl};
+    for (int i = 0; i < 3; ++i) {
+        if (s[i] < 0) lo += n[i] * s[i];
+        else hi += n[i] * s[i];
+    }
+    Extent e;
+    e.lo = (uintptr_t)base + (uintptr_t)(lo * bytes);
+    e.hi = (uintptr_t)base + (uintptr_t)((hi + 1) * bytes);
+    e.dense = hi - lo + 1 == B * C * L;
+    return e;
+}
+
 int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
 {
     if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
@@ -93,6 +114,14 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     if (!empty) {
         if (!p->x || !p->out || !p->weight) return fail(CANON_ERR_INVALID_ARGUMENT, "x, out and weight must not be NULL");
         if (p->x == p->out) return fail(CANON_ERR_INVALID_ARGUMENT, "out must not alias x");
+        // Overlapping byte ranges: an output element would overwrite an input another thread still has to read.
+        // (Two views that both leave holes may interleave in one buffer without sharing an element; that case is
+        // left to the caller.)
+        const int xb = elem_bytes(p->x_dtype);
+        const Extent ex = extent_of(p->x, p->batch, p->channels, p->seqlen, p->x_stride_b, p->x_stride_c, p->x_stride_l, xb);
+        const Extent eo = extent_of(p->out, p->batch, p->channels, p->seqlen, p->out_stride_b, p->out_stride_c, p->out_stride_l, xb);
+        if (ex.lo < eo.hi && eo.lo < ex.hi && (ex.dense || eo.dense))
+            return fail(CANON_ERR_INVALID_ARGUMENT, "out must not alias x: their memory ranges overlap");
     }
     if (p->mask && !valid_mask_dtype(p->mask_dtype))
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);

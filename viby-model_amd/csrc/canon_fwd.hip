@@ -92,7 +92,7 @@ __device__ __forceinline__ void bcl_edge_finish(const FwdArgs &a, const float (*
 // row stride that is not a multiple of E).  The aligned middle of every row runs through the
 // same vector code, shifted by `head` elements; the up to E-1 elements before it and after it
 // are computed one per lane by the waves that own the first and the last segment.
-template <int DT, int W, int U, bool MASK, bool NT, bool EDGE = false>
+template <int DT, int W, int U, bool MASK, bool BIG, bool EDGE = false>
 __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
     for (int u = 0; u < U; ++u) {
         const uint32_t v = v0 + u * 64u;
         X[u] = make_uint4(0, 0, 0, 0);
-        if (v < nvec) X[u] = load_vec<NT>(xvec + (int64_t)v * 16);
+        if (v < nvec) X[u] = load_vec<true>(xvec + (int64_t)v * 16);
     }
 
     // EDGE: lanes 0 .. head-1 of the first segment take the elements before the first vector,
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
 #pragma unroll
             for (int j = 0; j < E; ++j) o[j] += xm[j];
         }
-        if (v < nvec) store_vec<NT>(ovec + (int64_t)v * 16, pack_vec<DT>(o));
+        if (v < nvec) store_vec<true>(ovec + (int64_t)v * 16, pack_vec<DT>(o));
     }
 
     if constexpr (EDGE) {
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
     const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * Elem<DT>::bytes;
     char *orow = a.out + ((int64_t)b * a.o_sb + (int64_t)c * a.o_sc) * Elem<DT>::bytes;
 
-    const uint4 X = load_vec<false>(xrow + (int64_t)v * 16);
+    const uint4 X = load_vec<true>(xrow + (int64_t)v * 16);
     RawTaps<1> raw;
     fetch_taps<W, 1>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c, raw);
     float M[1][E];
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
 #pragma unroll
         for (int j = 0; j < E; ++j) o[j] += xm[j];
     }
-    if (active) store_vec<false>(orow + (int64_t)v * 16, pack_vec<DT>(o));
+    if (active) store_vec<true>(orow + (int64_t)v * 16, pack_vec<DT>(o));
 
     if (a.fin && row_ok)
         for (uint32_t slot = sub; slot < (uint32_t)a.S_out; slot += P) capture_row_state<DT>(a, b, c, (int)slot);
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
 // known at compile time (-1: read from the arguments; a select per element and a branch per row then).
 // keep0..2 (wave uniform): whether the rows t-3, t-2, t-1 belong to the packed sequence of row t
 // (always true without seq_idx); a row of another sequence enters as zeros.
-template <int DT, int W, bool MASK, bool NT, int VB, int ACT = -1, int RES = -1, int EAGER = -1>
+template <int DT, int W, bool MASK, bool BIG, int VB, int ACT = -1, int RES = -1, int EAGER = -1>
 __device__ __forceinline__ void blc_row_buf(const FwdArgs &a, const float (*w)[W], const float *bias,
                                             float (*hist)[VB / Elem<DT>::bytes], const typename VecIO<VB>::type &X, float m,
                                             __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t soff,
@@ -399,28 +399,28 @@ __device__ __forceinline__ void blc_row_buf(const FwdArgs &a, const float (*w)[W
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] += xm[e];
     }
-    BufIO<VB>::template store<NT>(VecIO<VB>::template pack<DT>(o), ro, voff, soff);
+    BufIO<VB>::template store<store_policy<BIG>()>(VecIO<VB>::template pack<DT>(o), ro, voff, soff);
 }
 
 // All rows first .. rows-1 of a slab.
-template <int DT, int W, int R, bool MASK, bool NT, int VB, int ACT, int RES, int EAGER>
+template <int DT, int W, int R, bool MASK, bool BIG, int VB, int ACT, int RES, int EAGER>
 __device__ __forceinline__ void blc_rows_buf(const FwdArgs &a, const float (&w)[VB / Elem<DT>::bytes][W], const float (&bias)[VB / Elem<DT>::bytes],
                                              float (&hist)[3][VB / Elem<DT>::bytes], const typename VecIO<VB>::type (&X)[R], const float (&m)[R],
                                              __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t os, int rows)
 {
     if (rows == R) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) blc_row_buf<DT, W, MASK, NT, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+        for (int r = 0; r < R; ++r) blc_row_buf<DT, W, MASK, BIG, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
     } else {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (r < rows) blc_row_buf<DT, W, MASK, NT, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+            if (r < rows) blc_row_buf<DT, W, MASK, BIG, VB, ACT, RES, EAGER>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
     }
 }
 
 // ... with activation, residual and rounding mode as compile-time constants for the settings CanonLayer uses
 // (no activation; residual added or not; either rounding mode), read from the arguments otherwise.
-template <int DT, int W, int R, bool MASK, bool NT, int VB>
+template <int DT, int W, int R, bool MASK, bool BIG, int VB>
 __device__ __forceinline__ void blc_rows_dispatch(const FwdArgs &a, const float (&w)[VB / Elem<DT>::bytes][W], const float (&bias)[VB / Elem<DT>::bytes],
                                                   float (&hist)[3][VB / Elem<DT>::bytes], const typename VecIO<VB>::type (&X)[R], const float (&m)[R],
                                                   __amdgpu_buffer_rsrc_t ro, uint32_t voff, uint32_t os, int rows)
@@ -428,16 +428,16 @@ __device__ __forceinline__ void blc_rows_dispatch(const FwdArgs &a, const float 
     // without a mask both residual modes add the raw input
     const int res = (!MASK && a.res_mode) ? CANON_RESIDUAL_UNMASKED : a.res_mode;
     constexpr int XR = CANON_RESIDUAL_UNMASKED, XM = CANON_RESIDUAL_MASKED, NONE = CANON_RESIDUAL_NONE;
-    if (a.act) blc_rows_buf<DT, W, R, MASK, NT, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else if (!a.eager && res == XR) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XR, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else if (!a.eager && res == XM) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XM, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else if (!a.eager && res == NONE) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, NONE, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else if (res == XR) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XR, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else if (res == XM) blc_rows_buf<DT, W, R, MASK, NT, VB, 0, XM, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
-    else blc_rows_buf<DT, W, R, MASK, NT, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    if (a.act) blc_rows_buf<DT, W, R, MASK, BIG, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == XR) blc_rows_buf<DT, W, R, MASK, BIG, VB, 0, XR, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == XM) blc_rows_buf<DT, W, R, MASK, BIG, VB, 0, XM, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (!a.eager && res == NONE) blc_rows_buf<DT, W, R, MASK, BIG, VB, 0, NONE, 0>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (res == XR) blc_rows_buf<DT, W, R, MASK, BIG, VB, 0, XR, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else if (res == XM) blc_rows_buf<DT, W, R, MASK, BIG, VB, 0, XM, 1>(a, w, bias, hist, X, m, ro, voff, os, rows);
+    else blc_rows_buf<DT, W, R, MASK, BIG, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
 }
 
-template <int DT, int W, int R, bool MASK, bool NT, bool SEQ, int VB, int MODE>
+template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE>
 __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t blk,
                                                typename VecIO<VB>::type (*tail)[3][64],   // LDS: raw last three rows of each wave's slab
                                                uint32_t (*taps_lds)[64 * (VB / 2) * 5])   // LDS: taps and bias of each channel tile
@@ -520,7 +520,7 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
     for (int r = 0; r < R; ++r) {
         // rows past the end of the sequence: the slab's last row again (loaded, never used)
         const uint32_t rr = r < rows ? (uint32_t)r : (rows > 0 ? (uint32_t)(rows - 1) : 0u);
-        X[r] = BufIO<VB>::template load<NT>(rx, voff, (rr + 3u) * xs);
+        X[r] = BufIO<VB>::template load<kAuxStream>(rx, voff, (rr + 3u) * xs);
         m[r] = 0.0f;
     }
 #pragma unroll
@@ -533,7 +533,7 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
     if (wt == 0 && t0 > 0) {
 #pragma unroll
         for (int j = 0; j < 3; ++j)
-            if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<false>(rx, voff, (uint32_t)j * xs);
+            if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<kAuxPlain>(rx, voff, (uint32_t)j * xs);
     }
     if (rows > 0) {
         if constexpr (MODE == TAPS_ANY)
@@ -609,11 +609,11 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
             // so the all-kept case takes the plain code
             const int32_t cur = sq[3 + r];
             const bool k0 = sq[r] == cur, k1 = sq[r + 1] == cur, k2 = sq[r + 2] == cur;
-            if (k0 && k1 && k2) blc_row_buf<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
-            else blc_row_buf<DT, W, MASK, NT, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os, k0, k1, k2);
+            if (k0 && k1 && k2) blc_row_buf<DT, W, MASK, BIG, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os);
+            else blc_row_buf<DT, W, MASK, BIG, VB>(a, w, bias, hist, X[r], m[r], ro, voff, (uint32_t)r * os, k0, k1, k2);
         }
     } else {
-        blc_rows_dispatch<DT, W, R, MASK, NT, VB>(a, w, bias, hist, X, m, ro, voff, os, rows);
+        blc_rows_dispatch<DT, W, R, MASK, BIG, VB>(a, w, bias, hist, X, m, ro, voff, os, rows);
     }
 
     if (a.fin && active && t0 + rows == (int64_t)a.L) {
@@ -644,7 +644,7 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
 
 // The block's code once per tap layout (wave-uniform choice): the contiguous layouts are straight-line
 // loads, the general one branches on the run-time weight type between its loads and waits there.
-template <int DT, int W, int R, bool MASK, bool NT, bool SEQ = false, int VB = kBlcVecBytes>
+template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ = false, int VB = kBlcVecBytes>
 __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
 {
     __shared__ typename VecIO<VB>::type tail[kBlcWaves * kBlcWC][3][64];
@@ -654,23 +654,23 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     __shared__ uint32_t taps_lds[kBlcWC][kTapWordsLds];
     if constexpr (W == 4) {
         if (a.tap_mode == TAPS_SAME) {
-            blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_SAME>(a, blk, tail, taps_lds);
+            blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_SAME>(a, blk, tail, taps_lds);
             return;
         }
         if constexpr (DT != CANON_DTYPE_F32) {
             if (a.tap_mode == TAPS_WIDE) {
-                blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_WIDE>(a, blk, tail, taps_lds);
+                blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_WIDE>(a, blk, tail, taps_lds);
                 return;
             }
         }
     }
-    blc_block_body<DT, W, R, MASK, NT, SEQ, VB, TAPS_ANY>(a, blk, tail, taps_lds);
+    blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_ANY>(a, blk, tail, taps_lds);
 }
 
-template <int DT, int W, int R, bool MASK, bool NT>
+template <int DT, int W, int R, bool MASK, bool BIG>
 __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const FwdArgs a)
 {
-    blc_block<DT, W, R, MASK, NT>(a, blockIdx.x);
+    blc_block<DT, W, R, MASK, BIG>(a, blockIdx.x);
 }
 
 // the same over packed variable-length sequences (seq_idx)
@@ -680,11 +680,11 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_seq_kernel(const Fw
     blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
-template <int DT, int W, int R, bool MASK, bool NT>
+template <int DT, int W, int R, bool MASK, bool BIG>
 __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
 {
     const uint32_t p = part_of_block(m, blockIdx.x);
-    blc_block<DT, W, R, MASK, NT>(m.part[p], blockIdx.x - m.first_block[p]);
+    blc_block<DT, W, R, MASK, BIG>(m.part[p], blockIdx.x - m.first_block[p]);
 }
 
 // ---------------------------------------------------------------------------
@@ -838,27 +838,27 @@ __global__ __launch_bounds__(256) void canon_fwd_generic_kernel(const FwdArgs a)
 // ---------------------------------------------------------------------------
 namespace {
 
-template <int DT, int W, bool MASK, bool NT, bool EDGE> void launch_bcl_e(const FwdPlan &pl, hipStream_t s)
+template <int DT, int W, bool MASK, bool BIG, bool EDGE> void launch_bcl_e(const FwdPlan &pl, hipStream_t s)
 {
     const dim3 g(pl.grid), b(256);
     switch (pl.U) {
-    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
-    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, NT, EDGE>), g, b, 0, s, pl.args); break;
+    case 4: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 4, MASK, BIG, EDGE>), g, b, 0, s, pl.args); break;
+    case 2: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 2, MASK, BIG, EDGE>), g, b, 0, s, pl.args); break;
+    default: hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, 1, MASK, BIG, EDGE>), g, b, 0, s, pl.args); break;
     }
 }
 
-template <int DT, int W, bool MASK, bool NT> void launch_bcl(const FwdPlan &pl, hipStream_t s)
+template <int DT, int W, bool MASK, bool BIG> void launch_bcl(const FwdPlan &pl, hipStream_t s)
 {
-    if (pl.edge) launch_bcl_e<DT, W, MASK, NT, true>(pl, s);
-    else launch_bcl_e<DT, W, MASK, NT, false>(pl, s);
+    if (pl.edge) launch_bcl_e<DT, W, MASK, BIG, true>(pl, s);
+    else launch_bcl_e<DT, W, MASK, BIG, false>(pl, s);
 }
 
-template <int DT, int W, bool MASK, bool NT> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
+template <int DT, int W, bool MASK, bool BIG> void launch_fwd_vec(const FwdPlan &pl, hipStream_t s)
 {
     if (pl.kind == FWD_BCL_SHORT) hipLaunchKernelGGL((canon_fwd_bcl_short_kernel<DT, W, MASK>), dim3(pl.grid), dim3(256), 0, s, pl.args);
-    else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, NT>(pl, s);
-    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, NT>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
+    else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, BIG>(pl, s);
+    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
 }
 
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
@@ -869,7 +869,7 @@ template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
         else hipLaunchKernelGGL((canon_fwd_blc_seq_kernel<DT, W, kBlcRows, false>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
         return;
     }
-    // the streaming (non-temporal) variants exist for width 4 only
+    // the variants for large launches (stores written through, see store_policy) exist for width 4 only
     if (W == 4 && pl.args.nt) {
         if (mask) launch_fwd_vec<DT, W, true, W == 4>(pl, s);
         else launch_fwd_vec<DT, W, false, W == 4>(pl, s);
@@ -893,10 +893,10 @@ template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
     }
 }
 
-template <int DT, bool MASK, bool NT>
+template <int DT, bool MASK, bool BIG>
 void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, NT>), dim3(grid), dim3(kBlcThreads), 0, s, m);
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, BIG>), dim3(grid), dim3(kBlcThreads), 0, s, m);
 }
 
 template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)

@@ -507,6 +507,9 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the legs that run the headline kernels on other shapes (canon_shapes, launch_floor, "
+                         "host cost, eager rounding): a profile of the command then has one workload per kernel name")
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="also run this many plain device-to-device copies of one x-sized buffer "
                          "(a kernel of known traffic to scale profiler byte counters by)")
@@ -533,7 +536,8 @@ def main():
     ms_warm, _ = bench_prefill("bcl", max(20, args.steps // 10), 5, 1, ramp=False)
     ms_copy = bench_copy(args.steps, args.warmup, nbuf)
     ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
-    ms_blc_eager, plan_blc_eager = bench_prefill("blc", args.steps, args.warmup, nbuf, rounding=1)
+    if not args.no_extra:
+        ms_blc_eager, plan_blc_eager = bench_prefill("blc", args.steps, args.warmup, nbuf, rounding=1)
     ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
     rag_steps, rag_warm = max(20, args.steps // 4), max(4, args.warmup // 4)
     ms_rag, plan_rag, rag_bytes = bench_ragged("blc", rag_steps, rag_warm, 3)     # 3 x 453 MB between reuses
@@ -542,9 +546,10 @@ def main():
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
     us_dbwd, dbwd_bytes, ws_dbwd = bench_decode_backward(max(50, args.steps), max(5, args.warmup))
-    shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
-    floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
-    host_cost = bench_decode_host_cost()
+    if not args.no_extra:
+        shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
+        floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
+        host_cost = bench_decode_host_cost()
 
     nbytes = prefill_bytes(B, C, L)
     gbps = nbytes / (ms * 1e-3) / 1e9
@@ -566,10 +571,6 @@ def main():
         "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
                                  "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1),
                                  "frac_of_hbm_peak": round(nbytes / (ms_blc * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
-        "prefill_channel_last_eager_rounding": {"kernel": plan_blc_eager, "ms_per_step": round(ms_blc_eager, 6),
-                                                "GB/s": round(nbytes / (ms_blc_eager * 1e-3) / 1e9, 1),
-                                                "what": "the same launch with round_mode = eager (the eager module's "
-                                                        "rounding points: bit-identical to the reference's CPU path)"},
         "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",
                                        "kernel": plan_parts, "ms_per_step": round(ms_parts, 6),
                                        "GB/s": round(nbytes / (ms_parts * 1e-3) / 1e9, 1)},
@@ -583,12 +584,7 @@ def main():
         "decode": {"workload": f"configs[3]: bf16 state[{DEC_B},{C},{DEC_S}], {DEC_STEPS} carried steps",
                    "kernel": dec_plan, "us_per_step_stream": round(dec_us, 3),
                    "us_per_step_hipgraph": round(dec_graph_us, 3),
-                   "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1),
-                   "host_us_per_call": host_cost},
-        "canon_shapes": shapes,
-        "launch_floor": {"us_per_launch": round(floor_us, 3),
-                         "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what "
-                                 "a launch costs before it moves any data; every us_per_step above includes it"},
+                   "GB/s_hipgraph": round(decode_bytes(DEC_B, C, DEC_S) / (dec_graph_us * 1e-6) / 1e9, 1)},
         "backward_channel_last": {"kernel": plan_bwd, "ms_per_step": round(ms_bwd, 6),
                                   "GB/s": round(1.5 * nbytes / (ms_bwd * 1e-3) / 1e9, 1),
                                   "bytes": "x and dout read, dx written (3 tensor passes)",
@@ -601,6 +597,18 @@ def main():
                      "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": profiled_traffic_bytes(),
                      "traffic_source": "profiles/" + os.path.basename(TRAFFIC_PROFILE)},
     }
+    if not args.no_extra:
+        out["prefill_channel_last_eager_rounding"] = {
+            "kernel": plan_blc_eager, "ms_per_step": round(ms_blc_eager, 6),
+            "GB/s": round(nbytes / (ms_blc_eager * 1e-3) / 1e9, 1),
+            "what": "prefill_channel_last with round_mode = eager (the eager module's rounding points: bit-identical "
+                    "to the reference's CPU path)"}
+        out["decode"]["host_us_per_call"] = host_cost
+        out["canon_shapes"] = shapes
+        out["launch_floor"] = {
+            "us_per_launch": round(floor_us, 3),
+            "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what a launch "
+                    "costs before it moves any data (host and device side together); every us_per_step includes it"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -88,6 +88,22 @@ __device__ __forceinline__ void bcl_edge_finish(const FwdArgs &a, const float (*
     store1<DT>(orow, t, finish<DT>(acc, a.act, a.res_mode, a.eager, win[3], e.x[3]));
 }
 
+// Activation, residual and store of one 16-byte vector of accumulators.
+template <int DT, bool MASK, bool EAGER>
+__device__ __forceinline__ void bcl_finish_vec(const FwdArgs &a, float *o, const float *xr, const float *xm, char *dst, bool write)
+{
+    constexpr int E = Elem<DT>::per_vec;
+    activate<DT, E>(o, a.act != 0, EAGER);
+    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) o[j] += xr[j];
+    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) o[j] += xm[j];
+    }
+    if (write) store_vec<true>(dst, pack_vec<DT>(o));
+}
+
 // EDGE: the rows are contiguous in time but do not start on 16-byte boundaries (a length or a
 // row stride that is not a multiple of E).  The aligned middle of every row runs through the
 // same vector code, shifted by `head` elements; the up to E-1 elements before it and after it
@@ -229,15 +245,10 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const FwdArgs a)
             for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
             o[j] = acc;
         }
-        activate<DT, E>(o, a.act, a.eager);
-        if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
-#pragma unroll
-            for (int j = 0; j < E; ++j) o[j] += xr[j];
-        } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
-#pragma unroll
-            for (int j = 0; j < E; ++j) o[j] += xm[j];
-        }
-        if (v < nvec) store_vec<true>(ovec + (int64_t)v * 16, pack_vec<DT>(o));
+        // the rounding mode is branched on around the whole epilogue, store included, so that the eager module's
+        // extra roundings are not evaluated and then discarded (selects) on the usual path
+        if (a.eager) bcl_finish_vec<DT, MASK, true>(a, o, xr, xm, ovec + (int64_t)v * 16, v < nvec);
+        else bcl_finish_vec<DT, MASK, false>(a, o, xr, xm, ovec + (int64_t)v * 16, v < nvec);
     }
 
     if constexpr (EDGE) {
@@ -320,15 +331,8 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
         for (int k = 0; k < W; ++k) acc = fmaf(w[0][k], seq[j + (4 - W) + k], acc);
         o[j] = acc;
     }
-    activate<DT, E>(o, a.act, a.eager);
-    if (a.res_mode == CANON_RESIDUAL_UNMASKED || (!MASK && a.res_mode)) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) o[j] += xr[j];
-    } else if (a.res_mode == CANON_RESIDUAL_MASKED) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) o[j] += xm[j];
-    }
-    if (active) store_vec<true>(orow + (int64_t)v * 16, pack_vec<DT>(o));
+    if (a.eager) bcl_finish_vec<DT, MASK, true>(a, o, xr, xm, orow + (int64_t)v * 16, active);
+    else bcl_finish_vec<DT, MASK, false>(a, o, xr, xm, orow + (int64_t)v * 16, active);
 
     if (a.fin && row_ok)
         for (uint32_t slot = sub; slot < (uint32_t)a.S_out; slot += P) capture_row_state<DT>(a, b, c, (int)slot);

@@ -304,9 +304,9 @@ def bench_decode_backward(steps, warmup, nbuf=8):
     return ms * 1e3, (3 * DEC_S + 3) * elems * 2, ws.numel()
 
 
-def bench_backward(steps, warmup, nbuf):
+def bench_backward(steps, warmup, nbuf, layout="channel_last"):
     """Backward of the same prefill step (channel-contiguous, as a training step through the model
-    produces it): reads x and dout, writes dx, reduces dweight / dbias."""
+    produces it, or time-contiguous): reads x and dout, writes dx, reduces dweight / dbias."""
     import torch
     import causal_conv1d as cc
     from causal_conv1d import _lib
@@ -318,8 +318,12 @@ def bench_backward(steps, warmup, nbuf):
     db = torch.empty(C, dtype=torch.float32, device=dev)
     keep, params = [], []
     for _ in range(nbuf):
-        x = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
-        dy = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        if layout == "channel_last":
+            x = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+            dy = torch.randn(B, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
+        else:
+            x = torch.randn(B, C, L, generator=g, device=dev).bfloat16()
+            dy = torch.randn(B, C, L, generator=g, device=dev).bfloat16()
         dx = torch.empty_like(x)
         p = _lib.BwdParams()
         p.struct_size = ctypes.sizeof(_lib.BwdParams)

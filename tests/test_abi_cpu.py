@@ -318,10 +318,14 @@ def test_bwd_plan_and_workspace():
         assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == b"bwd_generic"
     assert L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(bwd_params(seq_idx=FAKE_X + 2))) == -1
     assert "seq_idx must be 4-byte aligned" in last_error()
-    # an initial state: the walk kernel reads the history; its checks
-    q = bwd_params(initial_state=FAKE_X + 0x800000, initial_len=3, init_stride_b=3456 * 3, init_stride_c=3, init_stride_s=1)
-    assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == b"bwd_generic"
-    assert L.canon_conv1d_bwd_plan(ctypes.byref(bwd_params(dfinal_state=FAKE_X + 0x900000, final_len=4))) == b"bwd_generic"
+    # an initial state / the gradient of the captured final state: the channel-contiguous kernel handles both,
+    # time-contiguous rows go to the walk kernel; its checks
+    for layout, want in (("blc", b"bwd_blc_vec"), ("bcl", b"bwd_generic")):
+        q = bwd_params(layout=layout, initial_state=FAKE_X + 0x800000, initial_len=3, init_stride_b=3456 * 3, init_stride_c=3,
+                       init_stride_s=1)
+        assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == want
+        q = bwd_params(layout=layout, dfinal_state=FAKE_X + 0x900000, final_len=4)
+        assert L.canon_conv1d_bwd_plan(ctypes.byref(q)) == want
     for over, msg in [(dict(initial_state=FAKE_X, initial_len=2), "shorter than width-1"),
                       (dict(dinitial_state=FAKE_X), "needs initial_state"),
                       (dict(dfinal_state=FAKE_X, final_len=0), "final_len 0"),

@@ -401,7 +401,8 @@ def test_backward_through_initial_states(cc, dtype, layout):
     history, several time chunks per row, all widths."""
     torch.manual_seed(17)
     for (B, C, L, S, W), act, residual, masked in itertools.product(
-            [(2, 24, 1, 3, 4), (2, 24, 2, 4, 4), (3, 40, 5, 8, 4), (2, 16, 700, 3, 4), (2, 24, 37, 2, 3), (2, 24, 9, 4, 2)],
+            [(2, 24, 1, 3, 4), (2, 24, 2, 4, 4), (3, 40, 5, 8, 4), (2, 16, 700, 3, 4), (2, 24, 37, 2, 3), (2, 24, 9, 4, 2),
+             (2, 520, 70, 4, 4)],
             [None, "silu"], [False, True, "unmasked"], [False, True]):
         x = torch.randn(B, C, L).to(dtype)
         w, b = (torch.randn(C, W) * 0.5).to(dtype), (torch.randn(C) * 0.1).to(dtype)
@@ -440,7 +441,7 @@ def test_backward_through_final_states(cc, dtype, layout):
     inputs for the next call) reaches x, and initial_states where the state is longer than the row."""
     torch.manual_seed(23)
     for (B, C, L, S_in, S_out), act, residual, masked in itertools.product(
-            [(2, 24, 40, 0, 4), (2, 24, 2, 3, 8), (3, 16, 5, 4, 3), (2, 16, 300, 0, 8), (2, 24, 1, 8, 4)],
+            [(2, 24, 40, 0, 4), (2, 24, 2, 3, 8), (3, 16, 5, 4, 3), (2, 16, 300, 0, 8), (2, 24, 1, 8, 4), (2, 520, 70, 3, 8)],
             [None, "silu"], [False, True], [False, True]):
         W = 4
         x = torch.randn(B, C, L).to(dtype)

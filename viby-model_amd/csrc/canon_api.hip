@@ -546,9 +546,11 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     a.m_vec = mask_run_aligned(p->mask, p->mask_dtype, p->mask_stride_b, p->mask_stride_l, p->x_dtype);
     const bool ptrs16 = aligned16(p->x) && aligned16(p->dout) && aligned16(p->dx);
-    // packed sequences and an initial state: only the walk kernel gates taps by sequence index / reads the history
-    const bool packed = force_generic || p->seq_idx != nullptr || p->initial_state != nullptr || p->dfinal_state != nullptr;
-    const bool rows = !packed && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
+    // packed sequences: only the walk kernel gates taps by sequence index.  States (the history before t = 0, the
+    // gradient of the captured final state): the walk kernel and the channel-contiguous one.
+    const bool packed = force_generic || p->seq_idx != nullptr;
+    const bool states = p->initial_state != nullptr || p->dfinal_state != nullptr;
+    const bool rows = !packed && !states && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
                       a.d_sb % E == 0 && a.d_sc % E == 0;
     if (rows) {

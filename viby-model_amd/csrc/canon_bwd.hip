@@ -292,6 +292,9 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 // At the end the four waves' sums are added in a fixed order through LDS and
 // written as one partial set entry per channel.
 // ---------------------------------------------------------------------------
+// x and dout are read once and dx is written once: streamed (non-temporal) accesses, as in the forward kernels
+// (measured at B 8, C 3456, L 1024, bf16: 40.7 -> 37.8 us channel-contiguous, 33.6 -> 30.9 us time-contiguous).
+constexpr bool kBwdStream = true;
 template <int DT> __device__ __forceinline__ void unpack_half(const uint2 &v, float *f)
 {
     if constexpr (DT == CANON_DTYPE_F32) {
@@ -359,12 +362,14 @@ __device__ __forceinline__ void bwd_dz(const float (*w)[W], const float *bias, c
 
 // The sweep over one slab, last step first.  X / H hold xm in storage bits, dzh the dz of the
 // first three steps (already zero past the end of the sequence), dzf the dz of the three steps
-// after the slab.  FULL: all R steps exist.
-template <int DT, int W, bool MASK, bool ACT, bool FULL, int R, int E>
+// after the slab.  FULL: all R steps exist.  FIN: some steps of the slab were captured into the final state
+// (slot t - fin_first for t >= fin_first = L - S_out) and get that slot's gradient, read at `fin` (the lane's
+// first channel of slot 0) where it is needed: at most S_out steps per sequence.
+template <int DT, int W, bool MASK, bool ACT, bool FULL, bool FIN, int R, int E>
 __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W], const float *bias, const uint2 *X,
                                           const uint2 *H, const uint2 *G, const float *mm, const float (*dzh)[E],
                                           float (*dzf)[E], float (*dw)[W], float *dbs, char *dxp, int64_t ds, int rows,
-                                          bool active)
+                                          bool active, const char *fin = nullptr, int64_t fin_first_row = 0)
 {
     float xw[4][E];   // xm of rows r-3 .. r
 #pragma unroll
@@ -401,6 +406,14 @@ __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W],
 #pragma unroll
             for (int e = 0; e < E; ++e) o[e] += g[e];
         }
+        if constexpr (FIN) {
+            // fin_first_row: the slab row of the first captured step (may be negative)
+            if (r >= fin_first_row && r < rows) {
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    o[e] += load1<DT>(fin, (int64_t)e * a.k_sc + ((int64_t)r - fin_first_row) * a.k_ss);
+            }
+        }
         if constexpr (MASK) {
             if (mm[3 + r] != 1.0f) {
 #pragma unroll
@@ -411,7 +424,7 @@ __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W],
 #pragma unroll
             for (int e = 0; e < E; ++e) o[e] += g[e];
         }
-        if ((FULL || r < rows) && active) *(uint2 *)(dxp + r * ds) = pack_half<DT>(o);
+        if ((FULL || r < rows) && active) VecIO<8>::store<kBwdStream>(dxp + r * ds, pack_half<DT>(o));
         if (r > 0) {
             // slide the window one step back: the new oldest row is r - 4
 #pragma unroll
@@ -561,8 +574,8 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
-            X[r] = *(const uint2 *)(xb + t * xs);
-            G[r] = *(const uint2 *)(gb + t * gs);
+            X[r] = VecIO<8>::load<kBwdStream>(xb + t * xs);
+            G[r] = VecIO<8>::load<kBwdStream>(gb + t * gs);
         }
 #pragma unroll
         for (int j = 0; j < 3; ++j) H[j] = make_uint2(0, 0);
@@ -607,6 +620,19 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
             if (wv == 0) {
 #pragma unroll
                 for (int j = 0; j < 3; ++j) H[j] = bwd_mask_row<DT, MASK>(H[j], mm[j], true);   // zero already when t < 0
+            }
+        }
+        if (a.init && t0 == 0 && wv == 0) {
+            // rows before t = 0: entries of the initial state, not masked
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int s_ = a.S_in - 3 + j;
+                if (s_ < 0) continue;
+                float f[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    f[e] = load1<DT>(a.init, (int64_t)b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (int64_t)s_ * a.i_ss);
+                H[j] = pack_half<DT>(f);
             }
         }
         if constexpr (!ACT) {
@@ -669,10 +695,38 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         }
 
         // ---- sweep the slab from its last step to its first --------------------------
-        if (rows == R)
-            bwd_sweep<DT, W, MASK, ACT, true, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+        const int64_t fin_first = (int64_t)a.L - a.S_out;   // first captured step (S_out is 0 without dfinal_state)
+        if (a.dfin && t0 + rows > fin_first) {
+            // slot 0 of the final state's gradient holds step fin_first
+            const char *fin = a.dfin + ((int64_t)b * a.k_sb + (int64_t)c0 * a.k_sc) * BY;
+            bwd_sweep<DT, W, MASK, ACT, false, true, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows,
+                                                           active, fin, fin_first - t0);
+        } else if (rows == R)
+            bwd_sweep<DT, W, MASK, ACT, true, false, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
         else
-            bwd_sweep<DT, W, MASK, ACT, false, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+            bwd_sweep<DT, W, MASK, ACT, false, false, R, E>(a, w, bias, X, H, G, mm, dzh, dzf, dw, dbs, db_ + t0 * ds, ds, rows, active);
+    }
+
+    if (a.dinit && ch == 0 && wv == 0 && active) {
+        // here dzf[i] = dz[i] (zero past the end of the row).  Entry s is the input at t = s - S_in = -d:
+        // its gradient is sum_i w[W-1-d-i] * dz[i] over the taps that exist
+        for (int s_ = 0; s_ < a.S_in; ++s_) {
+            const int d = a.S_in - s_;
+            // a final state longer than the row also captured this entry (input at t = -d) in slot S_out - L - d
+            const int64_t slot = (int64_t)a.S_out - (int64_t)a.L - d;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    const int k = W - 1 - d - i;
+                    if (k >= 0) acc = fmaf(w[e][k < 0 ? 0 : k], dzf[i][e], acc);
+                }
+                if (a.dfin && slot >= 0)
+                    acc += load1<DT>(a.dfin, (int64_t)b * a.k_sb + (int64_t)(c0 + e) * a.k_sc + slot * a.k_ss);
+                store1<DT>(a.dinit, (int64_t)b * a.j_sb + (int64_t)(c0 + e) * a.j_sc + (int64_t)s_ * a.j_ss, acc);
+            }
+        }
     }
 
     // ---- the four waves' sums, added in the order 0, 1, 2, 3 -----------------------------
@@ -766,8 +820,8 @@ __global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
     for (int u = 0; u < U; ++u) {
         const uint32_t v = v0 + u * 64u;
         const uint32_t vc = v < nvec ? v : nvec - 1u;
-        X[u] = load_vec<false>(xrow + (int64_t)vc * 16);
-        G[u] = load_vec<false>(grow + (int64_t)vc * 16);
+        X[u] = load_vec<kBwdStream>(xrow + (int64_t)vc * 16);
+        G[u] = load_vec<kBwdStream>(grow + (int64_t)vc * 16);
     }
     RawTaps<1> raw;
     fetch_taps_uniform<W>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, a.b_pair != 0, c, raw);
@@ -912,7 +966,7 @@ __global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
 #pragma unroll
             for (int j = 0; j < E; ++j) o[j] += gg[u][j];
         }
-        if (v < nvec) store_vec<false>(drow + (int64_t)v * 16, pack_vec<DT>(o));
+        if (v < nvec) store_vec<kBwdStream>(drow + (int64_t)v * 16, pack_vec<DT>(o));
     }
 
     // the wave's dweight / dbias -> partial[(b * nseg + seg) * C + c][5]

@@ -113,9 +113,9 @@ struct BwdArgs {
     float *dbias;
     const int32_t *seq;   // packed-sequence indices [B, L] or nullptr (walk kernel only)
     int64_t q_sb, q_sl;
-    const char *init;     // inputs before t = 0, [B, C, S_in], or nullptr (walk kernel only)
+    const char *init;     // inputs before t = 0, [B, C, S_in], or nullptr (walk and channel-contiguous kernels)
     char *dinit;          // their gradient, or nullptr
-    const char *dfin;     // gradient of the captured final state [B, C, S_out], or nullptr (walk kernel only)
+    const char *dfin;     // gradient of the captured final state [B, C, S_out], or nullptr (same kernels)
     int64_t i_sb, i_sc, i_ss, j_sb, j_sc, j_ss, k_sb, k_sc, k_ss;
     int32_t S_in, S_out;
     int64_t x_sb, x_sc, x_sl;
@@ -199,7 +199,10 @@ constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised
 constexpr int upd_lane_channels(int elem_bytes, int S) { return (elem_bytes == 2 && S != 8) ? 2 : 1; }
 enum BwdKind { BWD_BLC_VEC, BWD_BCL_VEC, BWD_GENERIC };
 constexpr int kBwdRows = 4;   // rows fetched ahead per lane in the backward walk
-constexpr int kBwdHalfBlocksPerCU = 3;   // grid target of the channel-contiguous backward, in half blocks per CU
+#ifndef CANON_BWD_HALF_BLOCKS
+#define CANON_BWD_HALF_BLOCKS 3
+#endif
+constexpr int kBwdHalfBlocksPerCU = CANON_BWD_HALF_BLOCKS;   // grid target of the channel-contiguous backward, in half blocks per CU
 
 // ---------------------------------------------------------------------------
 // launch plans: what the validated arguments of one call turn into

@@ -550,6 +550,7 @@ def main():
     ms_bwd, plan_bwd, ws_bwd = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4)
 
     us_dbwd, dbwd_bytes, ws_dbwd = bench_decode_backward(max(50, args.steps), max(5, args.warmup))
+    ms_bwd_t, plan_bwd_t, ws_bwd_t = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4, "time_contiguous")
     if not args.no_extra:
         shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
         floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
@@ -593,6 +594,10 @@ def main():
                                   "GB/s": round(1.5 * nbytes / (ms_bwd * 1e-3) / 1e9, 1),
                                   "bytes": "x and dout read, dx written (3 tensor passes)",
                                   "scratch_bytes": ws_bwd},
+        "backward_time_contiguous": {"kernel": plan_bwd_t, "ms_per_step": round(ms_bwd_t, 6),
+                                     "GB/s": round(1.5 * nbytes / (ms_bwd_t * 1e-3) / 1e9, 1),
+                                     "bytes": "x and dout read, dx written (3 tensor passes)",
+                                     "scratch_bytes": ws_bwd_t},
         "decode_backward": {"workload": f"backward of one decode step, bf16 state[{DEC_B},{C},{DEC_S}], SiLU, state "
                                         "gradients in and out; two launches (step kernel + fixed-order reduction)",
                             "us_per_step": round(us_dbwd, 3),

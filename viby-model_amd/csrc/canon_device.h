@@ -285,22 +285,6 @@ __device__ __forceinline__ void load_mask_rows_wave(const void *p, int64_t row_b
     for (int j = 0; j < N; ++j) m[j] = bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
 }
 
-// The same in two steps, so that the load can be in flight while other work is done: lane j requests entry j ...
-template <int N>
-__device__ __forceinline__ float mask_rows_issue(const void *p, int64_t row_base, int64_t t_first, int64_t L, int64_t stride,
-                                                 int dt, int lane)
-{
-    int64_t t = t_first + (lane < N ? lane : N - 1);
-    t = t < 0 ? 0 : (t > L - 1 ? L - 1 : t);
-    return load_mask(p, row_base + t * stride, dt);
-}
-
-// ... and entry j is read from lane j when it is needed
-__device__ __forceinline__ float mask_rows_get(float v, int j)
-{
-    return bits_f((uint32_t)__builtin_amdgcn_readlane((int)f_bits(v), j));
-}
-
 // The same for N sequence indices.
 template <int N>
 __device__ __forceinline__ void load_seq_rows_wave(const int32_t *p, int64_t row_base, int64_t t_first, int64_t L,
@@ -360,8 +344,10 @@ template <> struct VecIO<8> {
     }
 };
 
-// Buffer accesses: address = resource base + vector offset (checked against the resource's size: a lane
-// beyond it loads zeros and stores nothing) + scalar offset (not checked).
+// Buffer accesses: address = resource base + vector offset + scalar offset, the sum checked against the
+// resource's size (measured on this hardware: the scalar offset counts; an access beyond the size loads zeros
+// and stores nothing).  A resource therefore spans every row its wave touches, and lanes that must not access
+// memory get a vector offset beyond any size.
 constexpr int kBufFlags = 0x00020000;   // raw buffer, 32-bit data format
 // Cache policy of a buffer access (its auxiliary bits).  Streamed data (x is read once, out written once) is
 // marked non-temporal whatever its size: measured on plain copies of 10 .. 450 MB each way, 9-17 % faster than

@@ -159,6 +159,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     a.b_pair = p->bias && ((uintptr_t)p->bias & 3u) == 0 && (p->w_dtype == CANON_DTYPE_F32 || p->channels % 2 == 0);
     plan->U = 1;
     plan->edge = false;
+    plan->wpb = 4;
     plan->grid = 0;
     plan->kind = FWD_GENERIC;
     if (empty) return CANON_OK;
@@ -230,7 +231,9 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
             plan->edge = !bcl_aligned;
             a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
             a.div_nseg = make_fastdiv(a.nseg); a.div_C = make_fastdiv(a.C);
-            a.nblocks = (uint32_t)((ntasks + 3) / 4);
+            const uint32_t wpb = ntasks >= kBclBigLaunch ? (uint32_t)kBclMaxWaves : 4u;
+            plan->wpb = wpb;
+            a.nblocks = (uint32_t)((ntasks + wpb - 1) / wpb);
             plan->grid = a.nblocks;
             return CANON_OK;
         }

@@ -116,14 +116,17 @@ __device__ __forceinline__ void bcl_finish_vec(const FwdArgs &a, float *o, const
 // Measured at B 8, C 3456, L 1024, bf16: 20.3 -> 19.6 us, half of it from the preload and half from the
 // scalars sharing one line of the argument segment.  (The channel-contiguous prefill and the decode update
 // gained nothing from the same change, or lost: they take their arguments as one block.)
+// `wpb`: waves per block, 4 or 8 (the waves are independent; large launches run 0.5-1 % faster in blocks of 8:
+// 19.6 -> 19.5 us at B 8, 70.0 -> 69.1 us at B 32; 16 are 7 % slower).
 template <int DT, int W, int U, bool MASK, bool BIG, bool EDGE = false>
-__global__ __launch_bounds__(256) void canon_fwd_bcl_kernel(const char *x_base, int64_t x_sb, int64_t x_sc, uint32_t ntasks,
-                                                            uint32_t nseg, uint32_t C, uint32_t divC_m, uint32_t divC_s1,
-                                                            uint32_t divC_s2, uint32_t nvec_row, const FwdArgs a)
+__global__ __launch_bounds__(64 * kBclMaxWaves) void canon_fwd_bcl_kernel(const char *x_base, int64_t x_sb, int64_t x_sc,
+                                                                          uint32_t ntasks, uint32_t nseg, uint32_t C,
+                                                                          uint32_t divC_m, uint32_t divC_s1, uint32_t divC_s2,
+                                                                          uint32_t nvec_row, uint32_t wpb, const FwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
     const int lane = threadIdx.x & 63;
-    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
+    const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * wpb + (threadIdx.x >> 6));
     if (task >= ntasks) return;
     uint32_t row = task, seg = 0;
     if (nseg > 1) {
@@ -855,12 +858,13 @@ namespace {
 
 template <int DT, int W, bool MASK, bool BIG, bool EDGE> void launch_bcl_e(const FwdPlan &pl, hipStream_t s)
 {
-    const dim3 g(pl.grid), b(256);
     const FwdArgs &a = pl.args;
+    const uint32_t wpb = pl.wpb;
+    const dim3 g(pl.grid), b(64 * wpb);
     switch (pl.U) {
 #define CANON_BCL_LAUNCH(UU)                                                                                             \
     hipLaunchKernelGGL((canon_fwd_bcl_kernel<DT, W, UU, MASK, BIG, EDGE>), g, b, 0, s, a.x, a.x_sb, a.x_sc, a.ntasks, a.nseg, \
-                       a.C, a.div_C.m, a.div_C.s1, a.div_C.s2, a.nvec, a)
+                       a.C, a.div_C.m, a.div_C.s1, a.div_C.s2, a.nvec, wpb, a)
     case 4: CANON_BCL_LAUNCH(4); break;
     case 2: CANON_BCL_LAUNCH(2); break;
     default: CANON_BCL_LAUNCH(1); break;

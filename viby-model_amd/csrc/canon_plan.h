@@ -207,10 +207,15 @@ constexpr int kBwdHalfBlocksPerCU = CANON_BWD_HALF_BLOCKS;   // grid target of t
 // ---------------------------------------------------------------------------
 // launch plans: what the validated arguments of one call turn into
 // ---------------------------------------------------------------------------
+// waves per block of the time-contiguous prefill: 4, or 8 in launches of at least kBclBigLaunch waves (64 per CU)
+constexpr int kBclMaxWaves = 8;
+constexpr uint32_t kBclBigLaunch = 16384;
+
 struct FwdPlan {
     FwdKind kind;
     int U;
     bool edge;   // bcl: rows do not start on 16-byte boundaries
+    uint32_t wpb; // bcl: waves per block
     FwdArgs args;
     uint32_t grid;
 };

@@ -698,11 +698,16 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_seq_kernel(const Fw
     blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
+// fb1..fb3: the first blocks of parts 1..3 once more as leading scalars, which arrive in registers with the wave:
+// the block knows its part at once and reads that part's arguments in one round instead of two.
 template <int DT, int W, int R, bool MASK, bool BIG>
-__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(const PartTable<FwdArgs> m)
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(uint32_t fb1, uint32_t fb2, uint32_t fb3,
+                                                                          const PartTable<FwdArgs> m)
 {
-    const uint32_t p = part_of_block(m, blockIdx.x);
-    blc_block<DT, W, R, MASK, BIG>(m.part[p], blockIdx.x - m.first_block[p]);
+    const uint32_t blk = blockIdx.x;
+    const uint32_t p = (blk >= fb1 ? 1u : 0u) + (blk >= fb2 ? 1u : 0u) + (blk >= fb3 ? 1u : 0u);
+    const uint32_t first = p == 0 ? 0u : (p == 1 ? fb1 : (p == 2 ? fb2 : fb3));
+    blc_block<DT, W, R, MASK, BIG>(m.part[p], blk - first);
 }
 
 // ---------------------------------------------------------------------------
@@ -920,7 +925,9 @@ template <int DT> void launch_fwd(const FwdPlan &pl, hipStream_t s)
 template <int DT, bool MASK, bool BIG>
 void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, BIG>), dim3(grid), dim3(kBlcThreads), 0, s, m);
+    static_assert(kMaxParts == 4, "the parts kernel takes three first-block scalars");
+    hipLaunchKernelGGL((canon_fwd_blc_parts_kernel<DT, 4, kBlcRows, MASK, BIG>), dim3(grid), dim3(kBlcThreads), 0, s,
+                       m.first_block[1], m.first_block[2], m.first_block[3], m);
 }
 
 template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)

@@ -707,7 +707,9 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(uint32
     const uint32_t blk = blockIdx.x;
     const uint32_t p = (blk >= fb1 ? 1u : 0u) + (blk >= fb2 ? 1u : 0u) + (blk >= fb3 ? 1u : 0u);
     const uint32_t first = p == 0 ? 0u : (p == 1 ? fb1 : (p == 2 ? fb2 : fb3));
-    blc_block<DT, W, R, MASK, BIG>(m.part[p], blk - first);
+    // a copy: its loads are issued together here, not one round after the other where the fields are used
+    const FwdArgs a = m.part[p];
+    blc_block<DT, W, R, MASK, BIG>(a, blk - first);
 }
 
 // ---------------------------------------------------------------------------

@@ -210,10 +210,17 @@ __global__ __launch_bounds__(256) void canon_update_vec_pool_kernel(const UpdArg
 
 // the token of one step given as several channel ranges (separate projections), one launch
 template <int DT, int W, int S, int NB>
-__global__ __launch_bounds__(256) void canon_update_vec_parts_kernel(const PartTable<UpdArgs> m)
+__global__ __launch_bounds__(256) void canon_update_vec_parts_kernel(uint32_t fb1, uint32_t fb2, uint32_t fb3,
+                                                                     const PartTable<UpdArgs> m)
 {
-    const uint32_t p = part_of_block(m, blockIdx.x);
-    update_vec_block<DT, W, S, NB>(m.part[p], blockIdx.x - m.first_block[p]);
+    // fb1..fb3: the first blocks of parts 1..3 once more as leading scalars, which arrive in registers with the
+    // wave (the block knows its part without a first read of the table); the part's arguments are copied, so
+    // that their loads are issued together.
+    const uint32_t blk = blockIdx.x;
+    const uint32_t p = (blk >= fb1 ? 1u : 0u) + (blk >= fb2 ? 1u : 0u) + (blk >= fb3 ? 1u : 0u);
+    const uint32_t first = p == 0 ? 0u : (p == 1 ? fb1 : (p == 2 ? fb2 : fb3));
+    const UpdArgs a = m.part[p];
+    update_vec_block<DT, W, S, NB>(a, blk - first);
 }
 
 // decode update, any strides / state length / rounding mode: one thread per (b, c)
@@ -328,9 +335,9 @@ template <int DT, int NB> void launch_update_parts_nb(const PartTable<UpdArgs> &
 {
     const dim3 g(grid), b(256);
     switch (S) {
-    case 3: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 3, NB>), g, b, 0, s, m); break;
-    case 4: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 4, NB>), g, b, 0, s, m); break;
-    default: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 8, NB>), g, b, 0, s, m); break;
+    case 3: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 3, NB>), g, b, 0, s, m.first_block[1], m.first_block[2], m.first_block[3], m); break;
+    case 4: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 4, NB>), g, b, 0, s, m.first_block[1], m.first_block[2], m.first_block[3], m); break;
+    default: hipLaunchKernelGGL((canon_update_vec_parts_kernel<DT, 4, 8, NB>), g, b, 0, s, m.first_block[1], m.first_block[2], m.first_block[3], m); break;
     }
 }
 

@@ -81,10 +81,29 @@ def time_region(fn, steps, warmup, ramp=True):
     return e0.elapsed_time(e1) / steps  # ms per step
 
 
-def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None, rounding=0, with_mask=False):
+def graph_of(run):
+    """`run(stream)` captured as one HIP graph on torch's current stream (after one uncaptured pass on a side
+    stream, which loads what the launches need)."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(ctypes.c_void_p(side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    return graph
+
+
+def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None, rounding=0, with_mask=False,
+                  as_graph=False):
     """One prefill launch per step over `nbuf` rotating buffer pairs.  shape: (B, C, L), the metric's by default;
     dtype: torch.bfloat16 by default; rounding: 0 fused, 1 the eager module's rounding points; with_mask: a
-    right-padded padding mask of x's type and the masked residual (what CanonLayer passes)."""
+    right-padded padding mask of x's type and the masked residual (what CanonLayer passes); as_graph: the launches
+    of one pass over the buffer pairs replayed as a HIP graph (for kernels shorter than the few microseconds this
+    host needs to issue a launch from Python: back-to-back launches would measure the host)."""
     import torch
     import causal_conv1d as cc
     from causal_conv1d import _lib
@@ -123,6 +142,15 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None
         if rc:
             _lib.check(rc, "canon_conv1d_fwd")
 
+    if as_graph:
+        def one_pass(stream_):
+            for r in refs:
+                rc = fwd(r, stream_)
+                if rc:
+                    _lib.check(rc, "canon_conv1d_fwd")
+        graph = graph_of(one_pass)
+        ms = time_region(lambda i: graph.replay(), max(20, 4 * steps // nbuf), 3, ramp) / nbuf
+        return ms, plan
     ms = time_region(step, steps, warmup, ramp)
     return ms, plan
 
@@ -238,15 +266,7 @@ def bench_decode(reps, warmup):
     ms_eager = time_region(lambda i: run64(cur), reps, warmup) / DEC_STEPS
 
     # the same 64 carried steps as one HIP graph (what a decode loop would replay)
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        run64(ctypes.c_void_p(side.cuda_stream))
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    with torch.cuda.graph(graph):
-        run64(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    graph = graph_of(run64)
     ms_graph = time_region(lambda i: graph.replay(), reps, warmup) / DEC_STEPS
     return ms_eager * 1e3, ms_graph * 1e3, plan
 
@@ -359,7 +379,10 @@ def bench_canon_shapes(steps, warmup):
     """The other shapes the Canon layers are called with (reference: causal-conv1d-mps/bench.py:89-164 benches
     Canon A/C, B and D): C = 640 (A, C), 960 (B), 3456 (D) at B8 L1024 bf16 in both layouts, the fp32 B1 C640
     case of configuration 1, and the masked B16 calls of configuration 5's prefill.  These are small: a launch
-    moves 5-60 MB, so part of each figure is the cost of a launch itself (see launch_floor)."""
+    moves 5-60 MB, so part of each figure is the cost of a launch itself (see launch_floor), and the shortest
+    finish faster than Python can issue the next one: each is timed as a HIP graph of one pass over its buffer
+    pairs (us_per_step_hipgraph) and as launches issued one by one from Python (us_per_step_host_issued); us_per_step
+    is the smaller of the two (a slow host inflates the second, few replays of a short graph the first)."""
     import torch
     rows = []
     cases = [("configs[1] Canon-A/C", (8, 640, 1024), torch.bfloat16, False),
@@ -374,9 +397,12 @@ def bench_canon_shapes(steps, warmup):
         nbuf = max(3, min(48, int(700e6 / nbytes) + 1))
         row = {"workload": f"{what}: {'fp32' if esize == 4 else 'bf16'} x[{shape[0]},{shape[1]},{shape[2]}]", "bytes": nbytes}
         for layout, key in (("bcl", "time_contiguous"), ("blc", "channel_last")):
-            ms, plan = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked)
+            ms_host, plan = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked)
+            ms, _ = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked, as_graph=True)
+            ms_graph, ms = ms, min(ms, ms_host)
             row[key] = {"kernel": plan, "us_per_step": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                        "us_per_step_hipgraph": round(ms_graph * 1e3, 3), "us_per_step_host_issued": round(ms_host * 1e3, 3)}
         rows.append(row)
     return rows
 
@@ -400,7 +426,15 @@ def bench_launch_floor(steps, warmup):
         if rc:
             _lib.check(rc, "canon_conv1d_update")
 
-    return time_region(step, steps, warmup) * 1e3
+    def run64(stream_):
+        for _ in range(64):
+            rc = upd(ref, stream_)
+            if rc:
+                _lib.check(rc, "canon_conv1d_update")
+
+    graph = graph_of(run64)
+    us_graph = time_region(lambda i: graph.replay(), max(4, steps // 64), 2) * 1e3 / 64
+    return time_region(step, steps, warmup) * 1e3, us_graph
 
 
 def bench_decode_host_cost(calls=5000):
@@ -615,9 +649,10 @@ def main():
         out["decode"]["host_us_per_call"] = host_cost
         out["canon_shapes"] = shapes
         out["launch_floor"] = {
-            "us_per_launch": round(floor_us, 3),
+            "us_per_launch": round(floor_us[0], 3), "us_per_launch_hipgraph": round(floor_us[1], 3),
             "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what a launch "
-                    "costs before it moves any data (host and device side together); every us_per_step includes it"}
+                    "costs before it moves any data, issued one by one from Python (host and device side together) "
+                    "and as 64 nodes of a HIP graph (the device side alone)"}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -231,7 +231,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
             plan->edge = !bcl_aligned;
             a.nvec = nvec; a.nseg = (uint32_t)nseg; a.ntasks = (uint32_t)ntasks;
             a.div_nseg = make_fastdiv(a.nseg); a.div_C = make_fastdiv(a.C);
-            const uint32_t wpb = ntasks >= kBclBigLaunch ? (uint32_t)kBclMaxWaves : 4u;
+            const uint32_t wpb = ntasks >= kBclBigLaunch && !a.mask ? (uint32_t)kBclMaxWaves : 4u;
             plan->wpb = wpb;
             a.nblocks = (uint32_t)((ntasks + wpb - 1) / wpb);
             plan->grid = a.nblocks;

@@ -407,6 +407,70 @@ def bench_canon_shapes(steps, warmup):
     return rows
 
 
+COPY_LIB = os.path.join(ROOT, "tests", "copy_ceiling", "libcopy_ceiling.so")
+
+
+def bench_copy_ceiling(steps, warmup):
+    """Plain copies with the prefill kernels' access patterns (tests/copy_ceiling/copy_ceiling.hip): whole rows
+    (every lane 16 bytes, 2 KB per wave: the time-contiguous kernel without its arithmetic) and 32-row x 512-byte
+    tiles through buffer accesses (the channel-contiguous kernel without history, taps and LDS), at the metric
+    shape and at four times it, same buffer rotation as the kernels; and an empty launch.  The line through the
+    two sizes separates what a launch costs from the rate the data moves at."""
+    import torch
+    if not os.path.exists(COPY_LIB):
+        return None
+    lib = ctypes.CDLL(COPY_LIB)
+    lib.copy_rows.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.copy_tiles.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    lib.empty_launch.argtypes = [ctypes.c_void_p]
+    dev = "cuda:0"
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {"what": "plain streamed copies of bf16 [B, 3456, 1024] each way in the access patterns of the two prefill "
+                   "kernels, rotating buffers; intercept_us / GB/s_slope: the line through the two sizes"}
+    times = {}
+    for batch in (8, 32):
+        nbytes = batch * C * L * 2
+        nbuf = max(3, int(700e6 / (2 * nbytes)) + 1)
+        pool = torch.empty(2 * nbuf * nbytes, dtype=torch.uint8, device=dev)
+        pool.random_(0, 255)
+        src = [pool.data_ptr() + 2 * i * nbytes for i in range(nbuf)]
+        dst = [pool.data_ptr() + (2 * i + 1) * nbytes for i in range(nbuf)]
+
+        def rows(i):
+            if lib.copy_rows(src[i % nbuf], dst[i % nbuf], nbytes, stream):
+                raise RuntimeError("copy_rows failed")
+
+        def tiles(i):
+            if lib.copy_tiles(src[i % nbuf], dst[i % nbuf], batch, L, C * 2, stream):
+                raise RuntimeError("copy_tiles failed")
+
+        k = max(20, steps * 8 // batch)
+        times["rows", batch] = time_region(rows, k, warmup) * 1e3
+        times["tiles", batch] = time_region(tiles, k, warmup) * 1e3
+        # the copies copy: spot check of the last destination
+        torch.cuda.synchronize()
+        i = (k - 1) % nbuf
+        a = pool[2 * i * nbytes:(2 * i + 1) * nbytes]
+        b = pool[(2 * i + 1) * nbytes:(2 * i + 2) * nbytes]
+        if not torch.equal(a, b):
+            raise RuntimeError("copy_tiles did not copy")
+        del pool
+    for kind in ("rows", "tiles"):
+        t8, t32 = times[kind, 8], times[kind, 32]
+        per_entry = (t32 - t8) / 24.0
+        out[kind] = {"B8_us": round(t8, 3), "B32_us": round(t32, 3),
+                     "GB/s_slope": round(2 * C * L * 2 / (per_entry * 1e-6) / 1e9, 1),
+                     "intercept_us": round(t8 - 8 * per_entry, 3)}
+
+    def run64(stream_):
+        for _ in range(64):
+            lib.empty_launch(stream_)
+
+    graph = graph_of(run64)
+    out["empty_launch_us_hipgraph"] = round(time_region(lambda i: graph.replay(), max(4, steps // 16), 2) * 1e3 / 64, 3)
+    return out
+
+
 def bench_launch_floor(steps, warmup):
     """What one launch through this entry point costs when it moves next to nothing: canon_conv1d_update on a
     [1, 8] token (one wave), back to back on the stream every other leg uses."""
@@ -588,6 +652,7 @@ def main():
     if not args.no_extra:
         shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
         floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
+        ceiling = bench_copy_ceiling(args.steps, args.warmup)
         host_cost = bench_decode_host_cost()
 
     nbytes = prefill_bytes(B, C, L)
@@ -648,6 +713,10 @@ def main():
                     "to the reference's CPU path)"}
         out["decode"]["host_us_per_call"] = host_cost
         out["canon_shapes"] = shapes
+        out["copy_ceiling"] = ceiling
+        if ceiling:
+            out["roofline"]["frac_of_plain_copy"] = round(ceiling["rows"]["B8_us"] / (ms * 1e3), 4)
+            out["prefill_channel_last"]["frac_of_plain_tile_copy"] = round(ceiling["tiles"]["B8_us"] / (ms_blc * 1e3), 4)
         out["launch_floor"] = {
             "us_per_launch": round(floor_us[0], 3), "us_per_launch_hipgraph": round(floor_us[1], 3),
             "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what a launch "

@@ -541,3 +541,14 @@ def test_torch_operators_for_traced_graphs_have_shape_only_twins():
     # the state arguments of the decode operators are declared as written to
     assert "Tensor(a1!) conv_state" in str(ops.update.default._schema)
     assert "Tensor(a1!) conv_state" in str(ops.update_parts.default._schema)
+
+
+def test_copy_ceiling_library_exports_what_the_bench_times():
+    """tests/copy_ceiling (plain copies in the kernels' access patterns, timed by bench.py beside the kernels):
+    loads without a GPU and exports its three entry points."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "copy_ceiling", "libcopy_ceiling.so")
+    if not os.path.exists(path):
+        pytest.skip("not built (make -C tests/copy_ceiling)")
+    lib = ctypes.CDLL(path)
+    for name in ("copy_rows", "copy_tiles", "empty_launch"):
+        assert getattr(lib, name) is not None

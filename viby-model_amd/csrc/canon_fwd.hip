@@ -455,8 +455,103 @@ __device__ __forceinline__ void blc_rows_dispatch(const FwdArgs &a, const float 
     else blc_rows_buf<DT, W, R, MASK, BIG, VB, -1, -1, -1>(a, w, bias, hist, X, m, ro, voff, os, rows);
 }
 
-template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE>
-__device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t blk,
+// What a wave needs to request its slab: the plain kernel gets these as leading scalar arguments, which
+// arrive in registers with the wave (kernel-argument preload), so the slab is requested before the argument
+// block has been read; the other kernels take them from the block.
+struct BlcLead {
+    const char *x;
+    int64_t x_sb;         // elements
+    uint32_t xs;          // bytes between rows of x
+    uint32_t L, nvec;
+};
+
+// A wave's place in the launch and its view of x.
+template <int VB> struct BlcWave {
+    uint32_t b, lane, wv, wt, wc, cv0, nl, c0, voff, xs;
+    int64_t t0;
+    int rows;
+    bool active;
+    __amdgpu_buffer_rsrc_t rx;   // rows t0-3 .. t0+R-1 of the wave's 64 channel vectors
+};
+
+// Places the wave in tile (b, ct, tt).  Uses nothing but `h`.
+template <int DT, int R, int VB>
+__device__ __forceinline__ void blc_place(const BlcLead &h, const uint32_t b, const uint32_t ct, const uint32_t tt, BlcWave<VB> &g)
+{
+    constexpr int E = VB / Elem<DT>::bytes;
+    constexpr int BY = Elem<DT>::bytes;
+    constexpr int WT = kBlcWaves, WC = kBlcWC;
+    g.b = b;
+    g.lane = threadIdx.x & 63u;
+    g.wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    g.wt = g.wv / WC;
+    g.wc = g.wv - g.wt * WC;
+    g.cv0 = (ct * WC + g.wc) * 64u;                               // the wave's first channel vector
+    g.t0 = ((int64_t)tt * WT + g.wt) * R;
+    const int64_t left = (int64_t)h.L - g.t0;
+    const bool idle = g.cv0 >= h.nvec || left <= 0;               // wave uniform: nothing to do but the barrier
+    g.rows = idle ? 0 : (left >= R ? R : (int)left);
+    g.nl = idle ? 0u : (h.nvec - g.cv0 < 64u ? h.nvec - g.cv0 : 64u);   // lanes that hold channels
+    g.active = g.lane < g.nl;
+    const uint32_t cvl = g.cv0 + g.lane < h.nvec ? g.cv0 + g.lane : h.nvec - 1u;   // idle lanes shadow the last vector (taps, state)
+    g.c0 = cvl * E;
+    g.xs = h.xs;
+    // One buffer resource per tensor and wave: lanes by vector offset, rows by scalar offset.  The x resource
+    // starts three rows early.  Every access the wave issues lies inside the resource (rows past the end of
+    // the sequence are not loaded); only lanes without channels are sent out of range, by their vector offset.
+    const char *xw = h.x + ((int64_t)b * h.x_sb + (int64_t)g.cv0 * E) * BY + (g.t0 - 3) * (int64_t)h.xs;
+    const uint32_t xrec = idle ? 0u : (uint32_t)(R + 2) * h.xs + g.nl * VB;
+    g.rx = __builtin_amdgcn_make_buffer_rsrc((void *)xw, 0, (int)xrec, kBufFlags);
+    g.voff = g.active ? g.lane * VB : 0x80000000u;
+}
+
+// Requests the wave's slab and, for the first wave of a tile, the three rows before it.
+template <int DT, int W, int R, int VB>
+__device__ __forceinline__ void blc_request(const BlcLead &h, const BlcWave<VB> &g, typename VecIO<VB>::type (&X)[R],
+                                            typename VecIO<VB>::type (&H)[3])
+{
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // rows past the end of the sequence: the slab's last row again (loaded, never used)
+        const uint32_t rr = r < g.rows ? (uint32_t)r : (g.rows > 0 ? (uint32_t)(g.rows - 1) : 0u);
+        X[r] = BufIO<VB>::template load<kAuxStream>(g.rx, g.voff, (rr + 3u) * h.xs);
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j) H[j] = VecIO<VB>::zero();
+    if (g.wt == 0 && g.t0 > 0) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<kAuxPlain>(g.rx, g.voff, (uint32_t)j * h.xs);
+    }
+}
+
+// Where a block gets its argument block from.  ArgsHere: it was read at the start of the kernel.  ArgsLate: it
+// is read from the kernel-argument segment AFTER the slab has been requested (the plain kernel: the slab is
+// requested from preloaded scalars alone, so its loads are on their way while the argument block is read).
+// The empty asm is what orders the two: it may write memory, so the slab loads stay in front of it, and the
+// argument pointer comes out of it, so the argument loads stay behind it.
+struct ArgsHere {
+    static constexpr bool kLate = false;
+    const FwdArgs &a;
+    __device__ __forceinline__ const FwdArgs &get() const { return a; }
+};
+struct ArgsLate {
+    static constexpr bool kLate = true;
+    uint32_t offset;   // of the argument block in the kernel-argument segment
+    __device__ __forceinline__ FwdArgs get() const
+    {
+        typedef __attribute__((address_space(4))) const char *kernarg_ptr;
+        kernarg_ptr p = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr() + offset;
+        asm volatile("" : "+s"(p) : : "memory");
+        typedef __attribute__((address_space(4))) const FwdArgs *args_ptr;   // (aligned: scalar loads)
+        FwdArgs a;
+        __builtin_memcpy(&a, (args_ptr)p, sizeof(FwdArgs));
+        return a;
+    }
+};
+
+template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE, typename ARGS>
+__device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &h, const uint32_t tb, const uint32_t ct, const uint32_t tt,
                                                typename VecIO<VB>::type (*tail)[3][64],   // LDS: raw last three rows of each wave's slab
                                                uint32_t (*taps_lds)[64 * (VB / 2) * 5])   // LDS: taps and bias of each channel tile
 {
@@ -465,50 +560,25 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
     constexpr int WDT = MODE == TAPS_WIDE ? CANON_DTYPE_F32 : DT;   // weight type of the straight-line tap modes
     constexpr int WT = kBlcWaves, WC = kBlcWC;
     using V = VecIO<VB>;
-    using vec_t = typename V::type;
     static_assert(R >= 3, "a slab must hold the three rows the next slab needs");
-
-    // Block -> tile.  Workgroups are dealt to the eight XCDs (each with its own L2) in turn, block i to XCD
-    // i % 8.  The tiles are numbered so that `chunk` consecutive time tiles of one channel tile follow each
-    // other on ONE XCD: the three rows of history that the first wave of a tile re-reads were requested by
-    // the tile before it a moment earlier and come out of that L2 instead of memory.  The columns
-    // q = (b * ngroups + tg) * nct + ct (tg: a group of `chunk` time tiles) are dealt to the XCDs in turn,
-    // so the launch still sweeps memory in address order.
-    const uint32_t jq = blk >> 3;
-    const uint32_t jg = fdiv(jq, a.div_nseg);
-    const uint32_t q = jg * 8u + (blk & 7u);
-    if (q >= a.ntasks) return;   // whole block, before the barrier
-    const uint32_t qr = fdiv(q, a.div_nct);
-    const uint32_t ct = q - qr * a.nct;
-    const uint32_t b = fdiv(qr, a.div_ntt);
-    const uint32_t tt = (qr - b * a.nseg) * a.chunk + (jq - jg * a.chunk);
-    if (tt >= a.ntt) return;
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t wt = wv / WC, wc = wv - wt * WC;
-    const uint32_t cv0 = (ct * WC + wc) * 64u;                 // the wave's first channel vector
-    const int64_t t0 = ((int64_t)tt * WT + wt) * R;
-    const int64_t left = (int64_t)a.L - t0;
-    const bool idle = cv0 >= a.nvec || left <= 0;              // wave uniform: nothing to do but the barrier
-    const int rows = idle ? 0 : (left >= R ? R : (int)left);
-    const uint32_t nl = idle ? 0u : (a.nvec - cv0 < 64u ? a.nvec - cv0 : 64u);   // lanes that hold channels
-    const bool active = lane < nl;
-    const uint32_t cvl = cv0 + lane < a.nvec ? cv0 + lane : a.nvec - 1u;   // idle lanes shadow the last vector (taps, state)
-    const uint32_t c0 = cvl * E;
-
-    // One buffer resource per tensor and wave: lanes by vector offset, rows by scalar offset.  The x resource
-    // starts three rows early.
-    const uint32_t xs = (uint32_t)(a.x_sl * BY), os = (uint32_t)(a.o_sl * BY);
-    const char *xw = a.x + ((int64_t)b * a.x_sb + (int64_t)cv0 * E) * BY + (t0 - 3) * (int64_t)xs;
+    BlcWave<VB> wave;
+    typename V::type X[R], H[3];
+    blc_place<DT, R, VB>(h, tb, ct, tt, wave);
+    // the slab before the argument block where the block is still to be read; otherwise after the taps, which
+    // measured 0.4-0.7 us faster at B 8 than slab first
+    if constexpr (ARGS::kLate) blc_request<DT, W, R, VB>(h, wave, X, H);
+    const FwdArgs &a = args.get();
+    const uint32_t b = wave.b, lane = wave.lane, wv = wave.wv, wt = wave.wt, wc = wave.wc, cv0 = wave.cv0, nl = wave.nl, c0 = wave.c0;
+    const uint32_t voff = wave.voff, xs = wave.xs;
+    const int64_t t0 = wave.t0;
+    const int rows = wave.rows;
+    const bool active = wave.active;
+    const uint32_t os = (uint32_t)(a.o_sl * BY);
     char *ow = a.out + ((int64_t)b * a.o_sb + (int64_t)cv0 * E) * BY + t0 * (int64_t)os;
-    // Every access the wave issues lies inside the resources (rows past the end of the sequence are neither
-    // loaded nor stored); only lanes without channels are sent out of range, by their vector offset.
-    const uint32_t xrec = idle ? 0u : (uint32_t)(R + 2) * xs + nl * VB, orec = idle ? 0u : (uint32_t)(R - 1) * os + nl * VB;
-    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)xw, 0, (int)xrec, kBufFlags);
+    // (rows past the end of the sequence are not stored; lanes without channels are out of range)
+    const uint32_t orec = rows == 0 ? 0u : (uint32_t)(R - 1) * os + nl * VB;
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)ow, 0, (int)orec, kBufFlags);
-    const uint32_t voff = active ? lane * VB : 0x80000000u;
 
-    vec_t X[R], H[3];
     float m[R], mh[3];
     int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
@@ -534,25 +604,13 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
     } else if constexpr (MODE != TAPS_ANY) {
         fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
     }
+    if constexpr (!ARGS::kLate) blc_request<DT, W, R, VB>(h, wave, X, H);
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        // rows past the end of the sequence: the slab's last row again (loaded, never used)
-        const uint32_t rr = r < rows ? (uint32_t)r : (rows > 0 ? (uint32_t)(rows - 1) : 0u);
-        X[r] = BufIO<VB>::template load<kAuxStream>(rx, voff, (rr + 3u) * xs);
-        m[r] = 0.0f;
-    }
+    for (int r = 0; r < R; ++r) m[r] = 0.0f;
 #pragma unroll
     for (int j = 0; j < (SEQ ? R + 3 : 1); ++j) sq[j] = 0;
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
-        H[j] = V::zero();
-        mh[j] = 0.0f;
-    }
-    if (wt == 0 && t0 > 0) {
-#pragma unroll
-        for (int j = 0; j < 3; ++j)
-            if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<kAuxPlain>(rx, voff, (uint32_t)j * xs);
-    }
+    for (int j = 0; j < 3; ++j) mh[j] = 0.0f;
     if (rows > 0) {
         if constexpr (MODE == TAPS_ANY)
             fetch_taps<W, E>(a.weight, a.bias, a.w_sc, a.w_sk, a.w_dtype, a.w_vec != 0, c0, raw);
@@ -662,8 +720,9 @@ __device__ __forceinline__ void blc_block_body(const FwdArgs &a, const uint32_t 
 
 // The block's code once per tap layout (wave-uniform choice): the contiguous layouts are straight-line
 // loads, the general one branches on the run-time weight type between its loads and waits there.
-template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ = false, int VB = kBlcVecBytes>
-__device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
+template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ = false, int VB = kBlcVecBytes, typename ARGS>
+__device__ __forceinline__ void blc_block(const ARGS &a, const BlcLead &h, const uint32_t tap_mode, const uint32_t b,
+                                          const uint32_t ct, const uint32_t tt)
 {
     __shared__ typename VecIO<VB>::type tail[kBlcWaves * kBlcWC][3][64];
     // taps and bias of the block's channel tiles as fetched by its waves together: fp32 weights of 16-bit x are the
@@ -671,31 +730,74 @@ __device__ __forceinline__ void blc_block(const FwdArgs &a, const uint32_t blk)
     constexpr int kTapWordsLds = 64 * (VB / 2) * 5;
     __shared__ uint32_t taps_lds[kBlcWC][kTapWordsLds];
     if constexpr (W == 4) {
-        if (a.tap_mode == TAPS_SAME) {
-            blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_SAME>(a, blk, tail, taps_lds);
+        if (tap_mode == TAPS_SAME) {
+            blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_SAME>(a, h, b, ct, tt, tail, taps_lds);
             return;
         }
         if constexpr (DT != CANON_DTYPE_F32) {
-            if (a.tap_mode == TAPS_WIDE) {
-                blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_WIDE>(a, blk, tail, taps_lds);
+            if (tap_mode == TAPS_WIDE) {
+                blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_WIDE>(a, h, b, ct, tt, tail, taps_lds);
                 return;
             }
         }
     }
-    blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_ANY>(a, blk, tail, taps_lds);
+    blc_block_body<DT, W, R, MASK, BIG, SEQ, VB, TAPS_ANY>(a, h, b, ct, tt, tail, taps_lds);
 }
 
-template <int DT, int W, int R, bool MASK, bool BIG>
-__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const FwdArgs a)
+// Block -> tile.  Workgroups are dealt to the eight XCDs (each with its own L2) in turn, block i to XCD
+// i % 8.  The tiles are numbered so that `chunk` consecutive time tiles of one channel tile follow each
+// other on ONE XCD: the three rows of history that the first wave of a tile re-reads were requested by
+// the tile before it a moment earlier and come out of that L2 instead of memory.  The columns
+// q = (b * ngroups + tg) * nct + ct (tg: a group of `chunk` time tiles) are dealt to the XCDs in turn,
+// so the launch still sweeps memory in address order.
+//
+// ... with the blocks numbered in one dimension (block = (column group * chunk + tile of the group) * 8 + XCD)
+template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ = false, int VB = kBlcVecBytes>
+__device__ __forceinline__ void blc_block_linear(const FwdArgs &a, const uint32_t blk)
 {
-    blc_block<DT, W, R, MASK, BIG>(a, blockIdx.x);
+    const uint32_t jq = blk >> 3;
+    const uint32_t jg = fdiv(jq, a.div_nseg);
+    const uint32_t q = jg * 8u + (blk & 7u);
+    if (q >= a.ntasks) return;   // whole block, before the barrier
+    const uint32_t qr = fdiv(q, a.div_nct);
+    const uint32_t ct = q - qr * a.nct;
+    const uint32_t b = fdiv(qr, a.div_ntt);
+    const uint32_t tt = (qr - b * a.nseg) * a.chunk + (jq - jg * a.chunk);
+    if (tt >= a.ntt) return;
+    const BlcLead h = {a.x, a.x_sb, (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec};
+    blc_block<DT, W, R, MASK, BIG, SEQ, VB>(ArgsHere{a}, h, (uint32_t)a.tap_mode, b, ct, tt);
+}
+
+// ... and the same in the plain kernel from leading scalar arguments.  `chunk_m`: 2^32 / chunk rounded up (0 for
+// chunk 1), exact for the quotients of block numbers below 2^28 since chunk <= 8.  `packed`: chunk | tap mode
+// << 4 | s1 << 7 | s2 << 8 of the division by nct | s1 << 13 | s2 << 14 of that by ngroups.
+template <int DT, int W, int R, bool MASK, bool BIG>
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const char *x, int64_t x_sb, uint32_t xs, uint32_t L, uint32_t nvec,
+                                                                    uint32_t ncols, uint32_t nct, uint32_t nct_m, uint32_t ngroups,
+                                                                    uint32_t ngroups_m, uint32_t chunk_m, uint32_t packed,
+                                                                    const FwdArgs a)
+{
+    const uint32_t chunk = packed & 0xFu;
+    const uint32_t jq = blockIdx.x >> 3;
+    const uint32_t jg = chunk_m ? __umulhi(jq, chunk_m) : jq;
+    const uint32_t q = jg * 8u + (blockIdx.x & 7u);
+    if (q >= ncols) return;   // whole block, before the barrier
+    const uint32_t qr = fdiv(q, FastDiv{nct, nct_m, (packed >> 7) & 1u, (packed >> 8) & 31u});
+    const uint32_t ct = q - qr * nct;
+    const uint32_t b = fdiv(qr, FastDiv{ngroups, ngroups_m, (packed >> 13) & 1u, (packed >> 14) & 31u});
+    const uint32_t tt = (qr - b * ngroups) * chunk + (jq - jg * chunk);
+    if ((uint64_t)tt * (kBlcWaves * R) >= L) return;   // past the last time tile
+    const BlcLead h = {x, x_sb, xs, L, nvec};
+    // the argument block follows the fourteen leading dwords
+    static_assert(alignof(FwdArgs) == 8, "offset of the argument block in the kernel-argument segment");
+    blc_block<DT, W, R, MASK, BIG>(ArgsLate{56u}, h, (packed >> 4) & 3u, b, ct, tt);
 }
 
 // the same over packed variable-length sequences (seq_idx)
 template <int DT, int W, int R, bool MASK>
 __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_seq_kernel(const FwdArgs a)
 {
-    blc_block<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
+    blc_block_linear<DT, W, R, MASK, false, true, kBlcVecBytes>(a, blockIdx.x);
 }
 
 // fb1..fb3: the first blocks of parts 1..3 once more as leading scalars, which arrive in registers with the wave:
@@ -709,7 +811,7 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_parts_kernel(uint32
     const uint32_t first = p == 0 ? 0u : (p == 1 ? fb1 : (p == 2 ? fb2 : fb3));
     // a copy: its loads are issued together here, not one round after the other where the fields are used
     const FwdArgs a = m.part[p];
-    blc_block<DT, W, R, MASK, BIG>(a, blk - first);
+    blc_block_linear<DT, W, R, MASK, BIG>(a, blk - first);
 }
 
 // ---------------------------------------------------------------------------
@@ -889,8 +991,16 @@ template <int DT, int W, bool MASK, bool BIG> void launch_fwd_vec(const FwdPlan 
 {
     if (pl.kind == FWD_BCL_SHORT) hipLaunchKernelGGL((canon_fwd_bcl_short_kernel<DT, W, MASK>), dim3(pl.grid), dim3(256), 0, s, pl.args);
     else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, BIG>(pl, s);
-    else hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, pl.args);
+    else {
+        const FwdArgs &a = pl.args;
+        const uint32_t packed = a.chunk | (uint32_t)a.tap_mode << 4 | a.div_nct.s1 << 7 | a.div_nct.s2 << 8 | a.div_ntt.s1 << 13 | a.div_ntt.s2 << 14;
+        const uint32_t chunk_m = a.chunk > 1 ? (uint32_t)(((1ull << 32) + a.chunk - 1) / a.chunk) : 0u;
+        hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, a.x, a.x_sb,
+                           (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec, a.ntasks, a.nct, a.div_nct.m, a.nseg, a.div_ntt.m,
+                           chunk_m, packed, a);
+    }
 }
+
 
 template <int DT, int W> void launch_fwd_w(const FwdPlan &pl, hipStream_t s)
 {

@@ -869,6 +869,32 @@ __device__ __forceinline__ void decode_taps_contiguous(const TapWords<WDT, E> &r
     }
 }
 
+// Where a block gets its argument block from.  ArgsRead: it was read at the start of the kernel.  ArgsToRead: it
+// is read from the kernel-argument segment AFTER the block has requested its data from the kernel's leading
+// scalar arguments, which arrive in registers with the wave (kernel-argument preload): the data loads are on
+// their way while the argument block is read.  The empty asm is what orders the two: it may write memory, so
+// the data loads stay in front of it, and the argument pointer comes out of it, so the argument loads stay
+// behind it (left alone the compiler hoists them to the top of the kernel and waits for them there).
+template <typename A> struct ArgsRead {
+    static constexpr bool kLate = false;
+    const A &a;
+    __device__ __forceinline__ const A &get() const { return a; }
+};
+template <typename A> struct ArgsToRead {
+    static constexpr bool kLate = true;
+    uint32_t offset;   // of the argument block in the kernel-argument segment
+    __device__ __forceinline__ A get() const
+    {
+        typedef __attribute__((address_space(4))) const char *kernarg_ptr;
+        kernarg_ptr p = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr() + offset;
+        asm volatile("" : "+s"(p) : : "memory");
+        typedef __attribute__((address_space(4))) const A *args_ptr;   // (aligned: scalar loads)
+        A a;
+        __builtin_memcpy(&a, (args_ptr)p, sizeof(A));
+        return a;
+    }
+};
+
 template <typename Args>
 __device__ __forceinline__ uint32_t part_of_block(const PartTable<Args> &m, uint32_t blk)
 {

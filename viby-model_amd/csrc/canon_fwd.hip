@@ -525,30 +525,8 @@ __device__ __forceinline__ void blc_request(const BlcLead &h, const BlcWave<VB> 
     }
 }
 
-// Where a block gets its argument block from.  ArgsHere: it was read at the start of the kernel.  ArgsLate: it
-// is read from the kernel-argument segment AFTER the slab has been requested (the plain kernel: the slab is
-// requested from preloaded scalars alone, so its loads are on their way while the argument block is read).
-// The empty asm is what orders the two: it may write memory, so the slab loads stay in front of it, and the
-// argument pointer comes out of it, so the argument loads stay behind it.
-struct ArgsHere {
-    static constexpr bool kLate = false;
-    const FwdArgs &a;
-    __device__ __forceinline__ const FwdArgs &get() const { return a; }
-};
-struct ArgsLate {
-    static constexpr bool kLate = true;
-    uint32_t offset;   // of the argument block in the kernel-argument segment
-    __device__ __forceinline__ FwdArgs get() const
-    {
-        typedef __attribute__((address_space(4))) const char *kernarg_ptr;
-        kernarg_ptr p = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr() + offset;
-        asm volatile("" : "+s"(p) : : "memory");
-        typedef __attribute__((address_space(4))) const FwdArgs *args_ptr;   // (aligned: scalar loads)
-        FwdArgs a;
-        __builtin_memcpy(&a, (args_ptr)p, sizeof(FwdArgs));
-        return a;
-    }
-};
+using ArgsHere = ArgsRead<FwdArgs>;
+using ArgsLate = ArgsToRead<FwdArgs>;
 
 template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE, typename ARGS>
 __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &h, const uint32_t tb, const uint32_t ct, const uint32_t tt,

@@ -144,40 +144,75 @@ __device__ __forceinline__ void update_vec_body(const UpdArgs &a, const uint32_t
     }
 }
 
-template <int DT, int W, int S, int NB, bool POOL = false>
-__device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_t blk)
+// What a lane needs to request its token and its state rows.  The plain kernel gets these as leading scalar
+// arguments, which arrive in registers with the wave (kernel-argument preload), requests the data from them and
+// reads its argument block while those loads are on their way; the pool and multi-part kernels read the block
+// first and fill this from it.
+struct UpdLead {
+    const char *x;
+    char *state;
+    int64_t x_sb, s_sb;
+    uint32_t nthreads, nvec, B;
+    FastDiv div_nvec;
+};
+
+__device__ __forceinline__ UpdLead lead_of(const UpdArgs &a)
+{
+    return UpdLead{a.x, a.state, a.x_sb, a.s_sb, a.nthreads, a.nvec, a.B, a.div_nvec};
+}
+
+template <int DT, int W, int S, int NB, bool POOL = false, typename ARGS>
+__device__ __forceinline__ void update_vec_block(const ARGS &args, const UpdLead &h, const uint32_t blk)
 {
     constexpr int BY = Elem<DT>::bytes;
     constexpr int E = upd_lane_channels(BY, S);
     constexpr int ND = E * S * BY / 4;          // words of state per lane and batch entry
     constexpr int NX = (E * BY + 3) / 4;        // words of token / output
     static_assert(E * S * BY % 4 == 0, "a lane's piece of the state must be whole words");
+    static_assert(!(POOL && ARGS::kLate), "the pool indices are part of the argument block");
     const uint32_t tid = blk * 256u + threadIdx.x;
-    // the test reads a field of each 64-byte line of the arguments this kernel uses (the divisor is never 0,
-    // the flag never negative), so that all are requested together instead of one after the other
-    if ((tid >= a.nthreads) | (a.div_nvec.d == 0) | (a.w_vec < 0)) return;   // '|': one test, no short circuit
-    const uint32_t bg = fdiv(tid, a.div_nvec);
-    const uint32_t cv = tid - bg * a.nvec;
+    if (tid >= h.nthreads) return;
+    const uint32_t bg = fdiv(tid, h.div_nvec);
+    const uint32_t cv = tid - bg * h.nvec;
     const uint32_t c0 = cv * E;
 
     uint32_t X[NB][NX];
     uint32_t ST[NB][ND];
     uint32_t srow[NB];   // conv_state row of each batch entry
+    if constexpr (ARGS::kLate) {
 #pragma unroll
-    for (int n = 0; n < NB; ++n) {
-        const uint32_t b = bg * NB + n;
-        srow[n] = b;
-        if (b < a.B) {
-            // POOL: rows of a state pool (conv_state_indices); an entry whose index is outside the pool is skipped
-            // (nothing of it is read or written)
-            if constexpr (POOL) {
-                srow[n] = pool_row(a, b);
-                if (srow[n] == kSkipRow) continue;
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = bg * NB + n;
+            srow[n] = b;
+            if (b < h.B) {
+                const char *xp = h.x + ((int64_t)b * h.x_sb + c0) * BY;
+                if constexpr (E * BY == 2) X[n][0] = *(const uint16_t *)xp;
+                else load_words<NX>(xp, X[n]);
+                load_words<ND>(h.state + ((int64_t)b * h.s_sb + (int64_t)c0 * S) * BY, ST[n]);
             }
-            const char *xp = a.x + ((int64_t)b * a.x_sb + c0) * BY;
-            if constexpr (E * BY == 2) X[n][0] = *(const uint16_t *)xp;
-            else load_words<NX>(xp, X[n]);
-            load_words<ND>(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
+        }
+    }
+    const UpdArgs &a = args.get();
+    if constexpr (!ARGS::kLate) {
+        // the test reads a field of each 64-byte line of the arguments this kernel uses (the divisor is never 0,
+        // the flag never negative), so that all are requested together instead of one after the other
+        if ((a.div_nvec.d == 0) | (a.w_vec < 0)) return;   // '|': one test, no short circuit
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            const uint32_t b = bg * NB + n;
+            srow[n] = b;
+            if (b < a.B) {
+                // POOL: rows of a state pool (conv_state_indices); an entry whose index is outside the pool is
+                // skipped (nothing of it is read or written)
+                if constexpr (POOL) {
+                    srow[n] = pool_row(a, b);
+                    if (srow[n] == kSkipRow) continue;
+                }
+                const char *xp = a.x + ((int64_t)b * a.x_sb + c0) * BY;
+                if constexpr (E * BY == 2) X[n][0] = *(const uint16_t *)xp;
+                else load_words<NX>(xp, X[n]);
+                load_words<ND>(a.state + ((int64_t)srow[n] * a.s_sb + (int64_t)c0 * S) * BY, ST[n]);
+            }
         }
     }
     if constexpr (W == 4) {
@@ -195,17 +230,22 @@ __device__ __forceinline__ void update_vec_block(const UpdArgs &a, const uint32_
     update_vec_body<DT, W, S, NB, TAPS_ANY, POOL>(a, bg, c0, X, ST, srow);
 }
 
+// (the fourteen leading dwords; the argument block follows them in the kernel-argument segment)
 template <int DT, int W, int S, int NB>
-__global__ __launch_bounds__(256) void canon_update_vec_kernel(const UpdArgs a)
+__global__ __launch_bounds__(256) void canon_update_vec_kernel(const char *x, char *state, int64_t x_sb, int64_t s_sb,
+                                                               uint32_t nthreads, uint32_t nvec, uint32_t B, uint32_t div_m,
+                                                               uint32_t div_s1, uint32_t div_s2, const UpdArgs a)
 {
-    update_vec_block<DT, W, S, NB>(a, blockIdx.x);
+    static_assert(alignof(UpdArgs) == 8, "offset of the argument block in the kernel-argument segment");
+    const UpdLead h = {x, state, x_sb, s_sb, nthreads, nvec, B, FastDiv{nvec, div_m, div_s1, div_s2}};
+    update_vec_block<DT, W, S, NB>(ArgsToRead<UpdArgs>{56u}, h, blockIdx.x);
 }
 
 // the same with batch entry b using row conv_state_indices[b] of a state pool
 template <int DT, int W, int S, int NB>
 __global__ __launch_bounds__(256) void canon_update_vec_pool_kernel(const UpdArgs a)
 {
-    update_vec_block<DT, W, S, NB, true>(a, blockIdx.x);
+    update_vec_block<DT, W, S, NB, true>(ArgsRead<UpdArgs>{a}, lead_of(a), blockIdx.x);
 }
 
 // the token of one step given as several channel ranges (separate projections), one launch
@@ -220,7 +260,7 @@ __global__ __launch_bounds__(256) void canon_update_vec_parts_kernel(uint32_t fb
     const uint32_t p = (blk >= fb1 ? 1u : 0u) + (blk >= fb2 ? 1u : 0u) + (blk >= fb3 ? 1u : 0u);
     const uint32_t first = p == 0 ? 0u : (p == 1 ? fb1 : (p == 2 ? fb2 : fb3));
     const UpdArgs a = m.part[p];
-    update_vec_block<DT, W, S, NB>(a, blk - first);
+    update_vec_block<DT, W, S, NB>(ArgsRead<UpdArgs>{a}, lead_of(a), blk - first);
 }
 
 // decode update, any strides / state length / rounding mode: one thread per (b, c)
@@ -305,11 +345,16 @@ template <int DT, int W, int NB> void launch_update_vec_nb(const UpdPlan &pl, hi
         }
         return;
     }
-    switch (pl.args.S) {
-    case 3: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 3, NB>), g, b, 0, s, pl.args); break;
-    case 4: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 4, NB>), g, b, 0, s, pl.args); break;
-    default: hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, 8, NB>), g, b, 0, s, pl.args); break;
+    const UpdArgs &a = pl.args;
+#define CANON_UPD_LAUNCH(SS)                                                                                            \
+    hipLaunchKernelGGL((canon_update_vec_kernel<DT, W, SS, NB>), g, b, 0, s, a.x, a.state, a.x_sb, a.s_sb, a.nthreads,   \
+                       a.nvec, a.B, a.div_nvec.m, a.div_nvec.s1, a.div_nvec.s2, a)
+    switch (a.S) {
+    case 3: CANON_UPD_LAUNCH(3); break;
+    case 4: CANON_UPD_LAUNCH(4); break;
+    default: CANON_UPD_LAUNCH(8); break;
     }
+#undef CANON_UPD_LAUNCH
 }
 
 template <int DT, int W> void launch_update_vec_w(const UpdPlan &pl, hipStream_t s)

@@ -766,9 +766,14 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const char *
     const uint32_t tt = (qr - b * ngroups) * chunk + (jq - jg * chunk);
     if ((uint64_t)tt * (kBlcWaves * R) >= L) return;   // past the last time tile
     const BlcLead h = {x, x_sb, xs, L, nvec};
-    // the argument block follows the fourteen leading dwords
-    static_assert(alignof(FwdArgs) == 8, "offset of the argument block in the kernel-argument segment");
-    blc_block<DT, W, R, MASK, BIG>(ArgsLate{56u}, h, (packed >> 4) & 3u, b, ct, tt);
+    // the kernel-argument segment lays the arguments out like the members of a struct
+    struct Segment {
+        const char *x;
+        int64_t x_sb;
+        uint32_t xs, L, nvec, ncols, nct, nct_m, ngroups, ngroups_m, chunk_m, packed;
+        FwdArgs a;
+    };
+    blc_block<DT, W, R, MASK, BIG>(ArgsLate{(uint32_t)offsetof(Segment, a)}, h, (packed >> 4) & 3u, b, ct, tt);
 }
 
 // the same over packed variable-length sequences (seq_idx)

@@ -230,15 +230,21 @@ __device__ __forceinline__ void update_vec_block(const ARGS &args, const UpdLead
     update_vec_body<DT, W, S, NB, TAPS_ANY, POOL>(a, bg, c0, X, ST, srow);
 }
 
-// (the fourteen leading dwords; the argument block follows them in the kernel-argument segment)
 template <int DT, int W, int S, int NB>
 __global__ __launch_bounds__(256) void canon_update_vec_kernel(const char *x, char *state, int64_t x_sb, int64_t s_sb,
                                                                uint32_t nthreads, uint32_t nvec, uint32_t B, uint32_t div_m,
                                                                uint32_t div_s1, uint32_t div_s2, const UpdArgs a)
 {
-    static_assert(alignof(UpdArgs) == 8, "offset of the argument block in the kernel-argument segment");
+    // the kernel-argument segment lays the arguments out like the members of a struct
+    struct Segment {
+        const char *x;
+        char *state;
+        int64_t x_sb, s_sb;
+        uint32_t nthreads, nvec, B, div_m, div_s1, div_s2;
+        UpdArgs a;
+    };
     const UpdLead h = {x, state, x_sb, s_sb, nthreads, nvec, B, FastDiv{nvec, div_m, div_s1, div_s2}};
-    update_vec_block<DT, W, S, NB>(ArgsToRead<UpdArgs>{56u}, h, blockIdx.x);
+    update_vec_block<DT, W, S, NB>(ArgsToRead<UpdArgs>{(uint32_t)offsetof(Segment, a)}, h, blockIdx.x);
 }
 
 // the same with batch entry b using row conv_state_indices[b] of a state pool

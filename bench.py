@@ -574,17 +574,17 @@ def cpu_baseline(budget_s=10.0):
     w = (torch.randn(C, W, generator=g) * 0.02).bfloat16()
     bias = (torch.randn(C, generator=g) * 0.01).bfloat16()
     layer = EagerCanon(w, bias, False)
-    med, n = _median_time(lambda: layer.forward(x), budget_s, 50)
+    med, n = _median_time(lambda: layer.forward(x), 0.6 * budget_s, 300)
 
     cache = {}
     tok = torch.randn(DEC_B, 1, C, generator=g).bfloat16()
     layer.forward(tok, cache=cache, key=0)      # creates the 8-slot state the eager module keeps
-    med_dec, n_dec = _median_time(lambda: layer.forward(tok, cache=cache, key=0), budget_s / 4, 50)
+    med_dec, n_dec = _median_time(lambda: layer.forward(tok, cache=cache, key=0), budget_s / 4, 1000)
     dec_bytes = decode_bytes(DEC_B, C, 8)
 
     torch.set_num_threads(1)
     try:
-        med1, n1 = _median_time(lambda: layer.forward(x), budget_s / 2, 10)
+        med1, n1 = _median_time(lambda: layer.forward(x), budget_s / 2, 30)
     finally:
         torch.set_num_threads(cores)
     nbytes = prefill_bytes(B, C, L)

@@ -370,10 +370,14 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
 // the previous wave: each wave publishes the raw tail of its slab in LDS, one
 // barrier, the next wave picks it up -- only the first wave of a block reads
 // its history from memory, and the block order makes that a hit in the L2 of
-// its XCD (see blc_block_body).  The same barrier passes on the taps: the
+// its XCD (see blc_block_linear).  The same barrier passes on the taps: the
 // waves of a tile fetch a WT-th of its taps and bias each (every wave fetching
 // all of them cost 3 % at B = 32: 2.5 KB of L2 traffic per 8 KB of x).
-// All loads (slab, history, taps) are issued before the first wait.
+// All loads (slab, history, taps) are issued before the first wait on data.
+// The plain kernel requests slab and history before it has read its argument
+// block (from leading scalar arguments that arrive in registers), which takes
+// the read of the block out of the way: nothing at B 8, C 3456 unmasked,
+// 3 % with a mask, 5-22 % at C 640 / 960.
 // ---------------------------------------------------------------------------
 // One row of a slab: out = act(bias + taps . (history, x)) (+ residual), written through the wave's buffer
 // resource.  ACT / RES / EAGER: the activation flag, the residual mode and the rounding mode when they are

@@ -579,7 +579,8 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         const int rows = left >= R ? R : (left > 0 ? (int)left : 0);   // wave uniform
 
         // ---- all loads of the tile.  Requesting the next tile's rows while this one is worked on was measured
-        // twice (before, and after, this tile's rows are waited for): 3-4 % slower, 40 more registers.
+        // three times (before, and after, this tile's rows are waited for; with two register sets taken in turn
+        // and wait counts that leave the next tile's loads in flight): 3-5 % slower, 40-60 more registers.
         uint2 X[R], G[R], H[3];
 #pragma unroll
         for (int r = 0; r < R; ++r) {

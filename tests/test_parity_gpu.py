@@ -540,6 +540,25 @@ def test_time_contiguous_rows_off_the_16_byte_grid(cc, dtype):
                 assert_parity(got, want, exact=act is None, what=what, res=xm if res else None)
 
 
+def test_large_time_contiguous_launches_in_blocks_of_eight_waves(cc):
+    """Unmasked time-contiguous launches of 16384 waves or more run in blocks of eight waves: a last block that is
+    not full, rows off the 16-byte grid, rows of two segments; and the same rows with a mask (blocks of four)."""
+    g = torch.Generator().manual_seed(97)
+    for (B, C, L) in [(7, 2403, 1023), (2, 4211, 4100)]:
+        x = torch.randn(B, C, L, generator=g).bfloat16()
+        w = (torch.randn(C, 4, generator=g) * 0.3).bfloat16()
+        b = (torch.randn(C, generator=g) * 0.1).bfloat16()
+        mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
+        xg = x.to(DEV)
+        assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec", (B, C, L)
+        for m, res in ((None, True), (mask, "masked")):
+            want, want_state = co.conv1d_fwd(x, w, b, mask=m, residual=res, final_state_len=8)
+            got, state = run_fwd(cc, xg, w, b, mask=m, residual=res, S_out=8)
+            what = f"big/{B}x{C}x{L}/mask{m is not None}"
+            assert_parity(got, want, exact=True, what=what)
+            assert torch.equal(bits(state), bits(want_state)), what
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_short_time_contiguous_rows_share_a_wave(cc, dtype):
     """Rows of 1..32 whole vectors: 2..64 rows per wave (every power-of-two group size, vector counts on and

@@ -116,8 +116,9 @@ __device__ __forceinline__ void bcl_finish_vec(const FwdArgs &a, float *o, const
 // Measured at B 8, C 3456, L 1024, bf16: 20.3 -> 19.6 us, half of it from the preload and half from the
 // scalars sharing one line of the argument segment.  (The channel-contiguous prefill and the decode update
 // gained nothing from the same change, or lost: they take their arguments as one block.)
-// `wpb`: waves per block, 4 or 8 (the waves are independent; large unmasked launches run 0.5-1 % faster in blocks
-// of 8: 19.6 -> 19.5 us at B 8, 70.0 -> 69.1 us at B 32; 16 are 7 % slower, and with a mask 8 are 6-9 % slower).
+// `wpb`: waves per block, 1, 4 or 8 (the waves are independent; large unmasked launches run 0.5-1 % faster in
+// blocks of 8: 19.6 -> 19.5 us at B 8, 70.0 -> 69.1 us at B 32; 16 are 7 % slower; with a mask 8 are 6-9 % slower
+// and single waves 1-2 % faster than blocks of 4).
 template <int DT, int W, int U, bool MASK, bool BIG, bool EDGE = false>
 __global__ __launch_bounds__(64 * kBclMaxWaves) void canon_fwd_bcl_kernel(const char *x_base, int64_t x_sb, int64_t x_sc,
                                                                           uint32_t ntasks, uint32_t nseg, uint32_t C,

@@ -208,7 +208,7 @@ constexpr int kBwdHalfBlocksPerCU = CANON_BWD_HALF_BLOCKS;   // grid target of t
 // launch plans: what the validated arguments of one call turn into
 // ---------------------------------------------------------------------------
 // waves per block of the time-contiguous prefill: 4, or 8 in unmasked launches of at least kBclBigLaunch waves (64
-// per CU); with a mask blocks of 8 measured 6-9 % slower
+// per CU); with a mask 1 (blocks of 8 measured 6-9 % slower, of 1 1-2 % faster than of 4)
 constexpr int kBclMaxWaves = 8;
 constexpr uint32_t kBclBigLaunch = 16384;
 

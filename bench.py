@@ -61,7 +61,13 @@ def decode_bytes(b, c, s, esize=2, wsize=2):
 CLOCK_RAMP_S = 0.03   # untimed load before the warm-up steps: the first ~10 ms after idle run ~1 % slower (clocks ramping)
 
 
-def time_region(fn, steps, warmup, ramp=True):
+REGIONS = 9           # back-to-back timed regions of `steps` launches each; the median region is the figure reported
+
+
+def time_region(fn, steps, warmup, ramp=True, regions=REGIONS, stats=None):
+    """ms per step: `regions` timed regions of exactly `steps` steps each, one after the other on the launch stream,
+    each bracketed by events; the MEDIAN region is returned (a single region of 20 launches is 0.4 ms: one
+    scheduling hiccup of the host moves it by several percent).  `stats`, a dict, receives min / max / regions."""
     import torch
     t_end = time.perf_counter() + (CLOCK_RAMP_S if ramp else 0.0)
     i = 0
@@ -72,13 +78,19 @@ def time_region(fn, steps, warmup, ramp=True):
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(regions + 1)]
+    events[0].record()
+    k = 0
+    for r in range(regions):
+        for _ in range(steps):
+            fn(k)
+            k += 1
+        events[r + 1].record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps  # ms per step
+    times = sorted(events[r].elapsed_time(events[r + 1]) / steps for r in range(regions))
+    if stats is not None:
+        stats.update({"regions": regions, "min_ms_per_step": round(times[0], 6), "max_ms_per_step": round(times[-1], 6)})
+    return times[len(times) // 2]  # ms per step
 
 
 def graph_of(run):
@@ -98,9 +110,9 @@ def graph_of(run):
 
 
 def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None, rounding=0, with_mask=False,
-                  as_graph=False):
+                  as_graph=False, act=0, stats=None):
     """One prefill launch per step over `nbuf` rotating buffer pairs.  shape: (B, C, L), the metric's by default;
-    dtype: torch.bfloat16 by default; rounding: 0 fused, 1 the eager module's rounding points; with_mask: a
+    dtype: torch.bfloat16 by default; rounding: 0 fused, 1 the eager module's rounding points; act: 1 = SiLU; with_mask: a
     right-padded padding mask of x's type and the masked residual (what CanonLayer passes); as_graph: the launches
     of one pass over the buffer pairs replayed as a HIP graph (for kernels shorter than the few microseconds this
     host needs to issue a launch from Python: back-to-back launches would measure the host)."""
@@ -131,7 +143,7 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None
         x.copy_(torch.randn(x.shape, generator=g, device=dev))
         xs.append(x)
         outs.append(o)
-        params.append(cc._fill_fwd(x, o, w, bias, mask, None, None, 0, 1, rounding))
+        params.append(cc._fill_fwd(x, o, w, bias, mask, None, None, act, 1, rounding))
     plan = _lib.lib().canon_conv1d_fwd_plan(ctypes.byref(params[0])).decode()
     fwd = _lib.lib().canon_conv1d_fwd
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -149,9 +161,9 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None
                 if rc:
                     _lib.check(rc, "canon_conv1d_fwd")
         graph = graph_of(one_pass)
-        ms = time_region(lambda i: graph.replay(), max(20, 4 * steps // nbuf), 3, ramp) / nbuf
+        ms = time_region(lambda i: graph.replay(), max(20, 4 * steps // nbuf), 3, ramp, stats=stats) / nbuf
         return ms, plan
-    ms = time_region(step, steps, warmup, ramp)
+    ms = time_region(step, steps, warmup, ramp, stats=stats)
     return ms, plan
 
 
@@ -375,34 +387,52 @@ def bench_backward(steps, warmup, nbuf, layout="channel_last"):
     return ms, plan, ws.numel()
 
 
+def _shape_row(what, shape, dtype, masked, steps, warmup, act=0):
+    """One shape in both layouts.  us_per_step (and the rates derived from it) is always the HIP-graph figure: the
+    launches of one pass over the buffer pairs replayed as a graph, i.e. device time without the host's launch cost
+    (the shortest of these kernels finish faster than Python issues the next launch).  us_per_step_host_issued,
+    launches issued one by one from Python, is a side column."""
+    import torch
+    esize = 4 if dtype == torch.float32 else 2
+    nbytes = prefill_bytes(*shape, esize, esize) + (shape[0] * shape[2] * esize if masked else 0)
+    nbuf = max(3, min(48, int(700e6 / nbytes) + 1))
+    row = {"workload": f"{what}: {'fp32' if esize == 4 else 'bf16'} x[{shape[0]},{shape[1]},{shape[2]}]", "bytes": nbytes}
+    for layout, key in (("bcl", "time_contiguous"), ("blc", "channel_last")):
+        ms_host, plan = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked, act=act)
+        ms, _ = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked, as_graph=True, act=act)
+        row[key] = {"kernel": plan, "us_per_step": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "us_per_step_host_issued": round(ms_host * 1e3, 3)}
+    return row
+
+
 def bench_canon_shapes(steps, warmup):
     """The other shapes the Canon layers are called with (reference: causal-conv1d-mps/bench.py:89-164 benches
     Canon A/C, B and D): C = 640 (A, C), 960 (B), 3456 (D) at B8 L1024 bf16 in both layouts, the fp32 B1 C640
     case of configuration 1, and the masked B16 calls of configuration 5's prefill.  These are small: a launch
-    moves 5-60 MB, so part of each figure is the cost of a launch itself (see launch_floor), and the shortest
-    finish faster than Python can issue the next one: each is timed as a HIP graph of one pass over its buffer
-    pairs (us_per_step_hipgraph) and as launches issued one by one from Python (us_per_step_host_issued); us_per_step
-    is the smaller of the two (a slow host inflates the second, few replays of a short graph the first)."""
+    moves 5-60 MB, so part of each figure is the cost of a launch itself (see launch_floor)."""
     import torch
-    rows = []
     cases = [("configs[1] Canon-A/C", (8, 640, 1024), torch.bfloat16, False),
              ("configs[1] Canon-B", (8, 960, 1024), torch.bfloat16, False),
              ("configs[0] Canon-A fp32", (1, 640, 1024), torch.float32, False),
              ("configs[4] prefill Canon-A/C, padding mask", (16, 640, 1024), torch.bfloat16, True),
              ("configs[4] prefill Canon-B, padding mask", (16, 960, 1024), torch.bfloat16, True),
              ("configs[4] prefill Canon-D, padding mask", (16, 3456, 1024), torch.bfloat16, True)]
-    for what, shape, dtype, masked in cases:
-        esize = 4 if dtype == torch.float32 else 2
-        nbytes = prefill_bytes(*shape, esize, esize) + (shape[0] * shape[2] * esize if masked else 0)
-        nbuf = max(3, min(48, int(700e6 / nbytes) + 1))
-        row = {"workload": f"{what}: {'fp32' if esize == 4 else 'bf16'} x[{shape[0]},{shape[1]},{shape[2]}]", "bytes": nbytes}
-        for layout, key in (("bcl", "time_contiguous"), ("blc", "channel_last")):
-            ms_host, plan = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked)
-            ms, _ = bench_prefill(layout, steps, warmup, nbuf, shape=shape, dtype=dtype, with_mask=masked, as_graph=True)
-            ms_graph, ms = ms, min(ms, ms_host)
-            row[key] = {"kernel": plan, "us_per_step": round(ms * 1e3, 3), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
-                        "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                        "us_per_step_hipgraph": round(ms_graph * 1e3, 3), "us_per_step_host_issued": round(ms_host * 1e3, 3)}
+    return [_shape_row(what, shape, dtype, masked, steps, warmup) for what, shape, dtype, masked in cases]
+
+
+def bench_silu(steps, warmup):
+    """configs[1] with its optional SiLU (every Canon scenario of the reference's own bench runs with
+    activation=True, causal-conv1d-mps/bench.py:106-123, 236-246): C = 640 and 3456 at B8 L1024 bf16, both
+    layouts, and next to each the same launch without the activation, timed the same way in the same run."""
+    import torch
+    rows = []
+    for what, shape in (("configs[1] Canon-A/C, SiLU", (8, 640, 1024)), ("configs[1] Canon-D, SiLU", (8, 3456, 1024))):
+        row = _shape_row(what, shape, torch.bfloat16, False, steps, warmup, act=1)
+        plain = _shape_row(what, shape, torch.bfloat16, False, steps, warmup, act=0)
+        for key in ("time_contiguous", "channel_last"):
+            row[key]["us_per_step_no_activation"] = plain[key]["us_per_step"]
+            row[key]["silu_cost"] = round(row[key]["us_per_step"] / plain[key]["us_per_step"] - 1.0, 4)
         rows.append(row)
     return rows
 
@@ -539,6 +569,63 @@ def bench_decode_host_cost(calls=5000):
                         "8-slot state; the layer step includes the token mask and nn.Module.__call__" % calls}
 
 
+def bench_config5(steps=128):
+    """configs[4]: the Viby-shaped 18-layer bf16 model (tests/viby_harness.py, a restatement of the reference
+    forward, model/model.py:1115-1157, 1308-1327) with random weights: prefill of B16 x L1024 token ids, then
+    `steps` greedy tokens through the conv caches.  Timed with the HIP Canon layers and with the Canon layers
+    switched off (everything else identical), the decode both as a Python loop that launches kernel by kernel and
+    with the whole step captured once as a HIP graph (causal_conv1d.canon.GraphedDecodeStep) and replayed per
+    token: the difference between the two models is what the 72 Canon calls per forward cost."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from viby_harness import VibyShaped, generate_graphed, init_weights, viby_config
+    from causal_conv1d.canon import CanonLayer
+
+    class NoCanon(torch.nn.Module):
+        def forward(self, x, attention_mask=None, cache=None, layer_idx=None):
+            return x
+
+    dev = "cuda:0"
+    cfg = viby_config()
+    Bm, Tm = 16, 1024
+    ids = torch.randint(0, cfg.vocab_size, (Bm, Tm), generator=torch.Generator().manual_seed(5)).to(dev)
+    out = {"workload": f"configs[4]: 18 layers, hidden 640, 4 q / 1 kv heads of 160, FFN 1728, vocab 25600, Canon A-D, "
+                       f"bf16, random weights; prefill B{Bm} x L{Tm}, then {steps} greedy steps; wall clock around "
+                       f"torch.cuda.synchronize()"}
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        r = fn()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, r
+
+    for name, factory in (("hip_canon", lambda C, n: CanonLayer(C, cfg, n)), ("canon_off", lambda C, n: NoCanon())):
+        model = init_weights(VibyShaped(cfg, factory), 11, torch.bfloat16, dev)
+        with torch.no_grad():
+            model.generate(ids[:2, :64], 2)                      # warm-up: library, allocator
+            generate_graphed(model, ids[:2, :64], 3)
+            mask = torch.ones(Bm, Tm, dtype=torch.int64, device=dev)
+            t_prefill = min(timed(lambda: model.forward(ids, model.new_cache(), mask))[0] for _ in range(3))
+            t_loop, _ = timed(lambda: model.generate(ids, steps))
+            t_graph, _ = timed(lambda: generate_graphed(model, ids, steps))
+        out[name] = {"prefill_ms": round(t_prefill * 1e3, 2),
+                     "prefill_plus_decode_python_loop_s": round(t_loop, 4),
+                     "prefill_plus_decode_hipgraph_s": round(t_graph, 4),
+                     "decode_ms_per_token_python_loop": round((t_loop - t_prefill) / (steps - 1) * 1e3, 3),
+                     "decode_ms_per_token_hipgraph": round((t_graph - t_prefill) / (steps - 1) * 1e3, 3)}
+        del model
+        torch.cuda.empty_cache()
+    h, o = out["hip_canon"], out["canon_off"]
+    out["canon_share"] = {
+        "prefill": round(1.0 - o["prefill_ms"] / h["prefill_ms"], 4),
+        "decode_python_loop": round(1.0 - o["decode_ms_per_token_python_loop"] / h["decode_ms_per_token_python_loop"], 4),
+        "decode_hipgraph": round(1.0 - o["decode_ms_per_token_hipgraph"] / h["decode_ms_per_token_hipgraph"], 4),
+        "what": "1 - time with the Canon layers off / time with the HIP Canon layers: under the graph it is device time "
+                "(72 update launches per token), in the Python loop mostly the host's cost of issuing them"}
+    return out
+
+
 def _cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -632,12 +719,13 @@ def main():
         del src, dst
 
     nbuf = 6  # 6 x 113 MB = 680 MB of distinct traffic between reuses
-    ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf)
+    head_stats, blc_stats = {}, {}
+    ms, plan = bench_prefill("bcl", args.steps, args.warmup, nbuf, stats=head_stats)
     # right after the headline leg (clocks are up) and short: its launches of the same kernel hardly move that
     # kernel's average duration in a profile of this command
     ms_warm, _ = bench_prefill("bcl", max(20, args.steps // 10), 5, 1, ramp=False)
     ms_copy = bench_copy(args.steps, args.warmup, nbuf)
-    ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf)
+    ms_blc, plan_blc = bench_prefill("blc", args.steps, args.warmup, nbuf, stats=blc_stats)
     if not args.no_extra:
         ms_blc_eager, plan_blc_eager = bench_prefill("blc", args.steps, args.warmup, nbuf, rounding=1)
     ms_parts, plan_parts = bench_prefill_parts(args.steps, args.warmup, nbuf)
@@ -651,6 +739,8 @@ def main():
     ms_bwd_t, plan_bwd_t, ws_bwd_t = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4, "time_contiguous")
     if not args.no_extra:
         shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
+        silu = bench_silu(max(50, args.steps // 2), max(5, args.warmup // 2))
+        config5 = bench_config5()
         floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
         ceiling = bench_copy_ceiling(args.steps, args.warmup)
         host_cost = bench_decode_host_cost()
@@ -660,7 +750,9 @@ def main():
     out = {
         "metric": "Canon conv1d HBM GB/s (prefill B8 L1024 C3456 bf16); decode us/step B256",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms, 6), "timing": dict(head_stats, what="ms_per_step is the median of `regions` back-to-back "
+                                                    "timed regions of exactly `steps` launches each (HIP events)"),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: prefill bf16 x[B=8,C=3456,L=1024] time-contiguous, width 4, "
                                "bias, residual fused, no activation", "kernel": plan,
@@ -672,7 +764,7 @@ def main():
         "prefill_same_buffers": {"ms_per_step": round(ms_warm, 6), "GB/s": round(nbytes / (ms_warm * 1e-3) / 1e9, 1),
                                  "what": "the headline launch repeated on ONE buffer pair (113 MB, inside the 256 MB "
                                          "Infinity Cache): a cache rate, reported beside the HBM rate, never as it"},
-        "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6),
+        "prefill_channel_last": {"kernel": plan_blc, "ms_per_step": round(ms_blc, 6), "timing": blc_stats,
                                  "GB/s": round(nbytes / (ms_blc * 1e-3) / 1e9, 1),
                                  "frac_of_hbm_peak": round(nbytes / (ms_blc * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "prefill_channel_last_parts": {"workload": "gate, up as two [8,1024,1728] tensors, one launch, no cat",
@@ -713,6 +805,8 @@ def main():
                     "to the reference's CPU path)"}
         out["decode"]["host_us_per_call"] = host_cost
         out["canon_shapes"] = shapes
+        out["prefill_silu"] = silu
+        out["config5"] = config5
         out["copy_ceiling"] = ceiling
         if ceiling:
             out["roofline"]["frac_of_plain_copy"] = round(ceiling["rows"]["B8_us"] / (ms * 1e3), 4)

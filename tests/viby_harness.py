@@ -243,29 +243,15 @@ def generate_graphed(model: VibyShaped, ids: torch.Tensor, steps: int, capture=T
         tok.copy_(lg.argmax(dim=-1)[:, None])
         cache.pos_t.add_(1)
 
-    # warm-up on a side stream (library handles, allocator), then put every carried state back
-    sites = [name for name in ("a", "b", "c", "d") if hasattr(cache, f"canon_cache_{name}")]
-    saved = {name: [t.clone() for t in getattr(cache, f"canon_cache_{name}")] for name in sites}
     tok0 = tok.clone()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        step()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    for name in sites:
-        for t, old in zip(getattr(cache, f"canon_cache_{name}"), saved[name]):
-            t.copy_(old)
-    tok.copy_(tok0)
-    cache.pos_t.fill_(T)
-
     graph = None
     if capture == "compile":
         step = torch.compile(step, fullgraph=True, **(compile_kwargs or {}))
     elif capture:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
+        # the package's helper: warm-up on a side stream, every carried state put back, capture
+        from causal_conv1d.canon import GraphedDecodeStep
+        # (the K / V row the warm-up writes at position T is written again, with the same values, by the first replay)
+        graph = GraphedDecodeStep(step, cache, state=[tok, cache.pos_t, out_logits])
     toks, logits = [tok0[:, 0].clone()], [logits0]
     for _ in range(steps - 1):
         if graph is not None:

@@ -155,13 +155,18 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None
             _lib.check(rc, "canon_conv1d_fwd")
 
     if as_graph:
-        def one_pass(stream_):
-            for r in refs:
-                rc = fwd(r, stream_)
-                if rc:
-                    _lib.check(rc, "canon_conv1d_fwd")
-        graph = graph_of(one_pass)
-        ms = time_region(lambda i: graph.replay(), max(20, 4 * steps // nbuf), 3, ramp, stats=stats) / nbuf
+        # at least 48 launches per replay, so that what a replay itself costs (about 10 us) is spread thin
+        passes = max(1, -(-48 // nbuf))
+
+        def some_passes(stream_):
+            for _ in range(passes):
+                for r in refs:
+                    rc = fwd(r, stream_)
+                    if rc:
+                        _lib.check(rc, "canon_conv1d_fwd")
+        graph = graph_of(some_passes)
+        nodes = passes * nbuf
+        ms = time_region(lambda i: graph.replay(), max(5, steps // nodes), 2, ramp, stats=stats) / nodes
         return ms, plan
     ms = time_region(step, steps, warmup, ramp, stats=stats)
     return ms, plan
@@ -453,6 +458,9 @@ def bench_copy_ceiling(steps, warmup):
     lib.copy_rows.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     lib.copy_tiles.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
     lib.empty_launch.argtypes = [ctypes.c_void_p]
+    lib.copy_tile_shape.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+                                    ctypes.c_int, ctypes.c_void_p]
+    shapes = ["32x512B_8B_lanes", "16x512B_8B_lanes", "16x1KB_16B_lanes", "32x1KB_16B_lanes", "64x256B_16B_lanes"]
     dev = "cuda:0"
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {"what": "plain streamed copies of bf16 [B, 3456, 1024] each way in the access patterns of the two prefill "
@@ -477,6 +485,15 @@ def bench_copy_ceiling(steps, warmup):
         k = max(20, steps * 8 // batch)
         times["rows", batch] = time_region(rows, k, warmup) * 1e3
         times["tiles", batch] = time_region(tiles, k, warmup) * 1e3
+        for code, name in enumerate(shapes):
+            def shaped(i, code=code):
+                if lib.copy_tile_shape(src[i % nbuf], dst[i % nbuf], batch, L, C * 2, code, stream):
+                    raise RuntimeError("copy_tile_shape failed")
+            pool[nbytes:2 * nbytes].zero_()
+            times[name, batch] = time_region(shaped, k, warmup) * 1e3
+            torch.cuda.synchronize()
+            if not torch.equal(pool[:nbytes], pool[nbytes:2 * nbytes]):
+                raise RuntimeError(f"copy_tile_shape {name} did not copy")
         # the copies copy: spot check of the last destination
         torch.cuda.synchronize()
         i = (k - 1) % nbuf
@@ -485,12 +502,19 @@ def bench_copy_ceiling(steps, warmup):
         if not torch.equal(a, b):
             raise RuntimeError("copy_tiles did not copy")
         del pool
-    for kind in ("rows", "tiles"):
+    def line(kind):
         t8, t32 = times[kind, 8], times[kind, 32]
         per_entry = (t32 - t8) / 24.0
-        out[kind] = {"B8_us": round(t8, 3), "B32_us": round(t32, 3),
-                     "GB/s_slope": round(2 * C * L * 2 / (per_entry * 1e-6) / 1e9, 1),
-                     "intercept_us": round(t8 - 8 * per_entry, 3)}
+        return {"B8_us": round(t8, 3), "B32_us": round(t32, 3),
+                "GB/s_slope": round(2 * C * L * 2 / (per_entry * 1e-6) / 1e9, 1),
+                "intercept_us": round(t8 - 8 * per_entry, 3)}
+
+    for kind in ("rows", "tiles"):
+        out[kind] = line(kind)
+    out["tile_shapes"] = dict({name: line(name) for name in shapes},
+                              what="the channel-contiguous tensor copied in other tile shapes (rows x bytes per block of "
+                                   "four waves, bytes per lane), blocks in address order, stores written through: no "
+                                   "decomposition streams faster than the kernel's own by more than a few percent")
 
     def run64(stream_):
         for _ in range(64):

@@ -224,7 +224,8 @@ typedef struct canon_conv1d_bwd_params {
     const void *initial_state;      /* [batch, channels, initial_len] or NULL: the forward's initial_state (the chunked
                                        continuation of model/model.py:647-659 as one differentiable call); its last
                                        W-1 entries enter z as the inputs before t = 0 and dweight with them.  Not with
-                                       seq_idx.  Such calls take the strided kernel. */
+                                       seq_idx.  Channel-contiguous tensors keep their vector kernel with it;
+                                       time-contiguous ones take the strided kernel. */
     int64_t init_stride_b, init_stride_c, init_stride_s;
     int32_t initial_len;            /* >= W-1 when initial_state != NULL */
     int32_t reserved1;
@@ -234,7 +235,7 @@ typedef struct canon_conv1d_bwd_params {
     const void *dfinal_state;       /* [batch, channels, final_len] in x_dtype, or NULL: the gradient that arrives through
                                        the forward's final_state (the last final_len entries of initial_state ++ xm):
                                        added to dxm of the last steps and, where the state reaches back before t = 0,
-                                       to dinitial_state.  Such calls take the strided kernel. */
+                                       to dinitial_state.  Kernel choice as for initial_state. */
     int64_t dfinal_stride_b, dfinal_stride_c, dfinal_stride_s;
     int32_t final_len;              /* >= 1 when dfinal_state != NULL */
     int32_t reserved2;

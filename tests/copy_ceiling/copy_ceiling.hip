@@ -5,8 +5,11 @@
 //   copy_rows   every lane 16 bytes, a wave two vectors per lane = 2 KB of one row, streamed accesses:
 //               the time-contiguous kernel without its arithmetic
 //   copy_tiles  [B, L, rowbytes] memory in tiles of 32 rows x 512 bytes: 8 bytes per lane, 8 rows per wave,
-//               4 waves per block, buffer accesses, consecutive time tiles of a column on one XCD:
-//               the channel-contiguous kernel without history, taps, LDS and arithmetic
+//               4 waves per block, buffer accesses, consecutive time tiles of a column on one XCD, stores written
+//               through from 64 MB of traffic: the channel-contiguous kernel without history, taps, LDS and arithmetic
+//   copy_tile_shape  the same memory in other tile shapes (16 x 512 B, 16 x 1 KB and 32 x 1 KB with 16-byte lanes,
+//               64 x 256 B with 16-byte lanes and four rows per instruction), blocks in address order: would another
+//               decomposition of the channel-contiguous tensor stream faster?
 //   empty_launch  a kernel of one wave that does nothing
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -30,8 +33,9 @@ struct Tiles {
     char *out;
     uint32_t ncols, nct, ntt, L, rowbytes;
 };
+constexpr uint64_t kThroughBytes = 64ull << 20;   // traffic from which the channel-contiguous prefill writes its stores through
 
-__global__ __launch_bounds__(256) void copy_tiles_kernel(const Tiles g)
+template <int AUXS> __global__ __launch_bounds__(256) void copy_tiles_kernel(const Tiles g)
 {
     constexpr uint32_t R = 8, WT = 4, VB = 8;
     // block = (column group * ntt + time tile) * 8 + XCD; column = (batch entry, channel tile)
@@ -55,7 +59,59 @@ __global__ __launch_bounds__(256) void copy_tiles_kernel(const Tiles g)
 #pragma unroll
     for (uint32_t r = 0; r < R; ++r) v[r] = __builtin_amdgcn_raw_buffer_load_b64(ri, (int)voff, (int)(r * g.rowbytes), 2);
 #pragma unroll
-    for (uint32_t r = 0; r < R; ++r) __builtin_amdgcn_raw_buffer_store_b64(v[r], ro, (int)voff, (int)(r * g.rowbytes), 2);
+    for (uint32_t r = 0; r < R; ++r) __builtin_amdgcn_raw_buffer_store_b64(v[r], ro, (int)voff, (int)(r * g.rowbytes), AUXS);
+}
+
+// Tiles of R * WT * (64 / LPR) rows x LPR * VB bytes: a lane moves VB bytes, LPR lanes cover one row of the tile, a
+// load instruction 64 / LPR rows, a wave R instructions, a block WT waves.  Blocks in address order (channel tile
+// fastest, then time tile, then batch entry); stores written through like the kernel's in large launches.
+template <int VB, int R, int WT, int LPR>
+__global__ __launch_bounds__(64 * WT) void copy_shape_kernel(const Tiles g)
+{
+    constexpr uint32_t RPI = 64 / LPR, WB = LPR * VB;           // rows per instruction, tile width in bytes
+    const uint32_t ct = blockIdx.x % g.nct, r0 = blockIdx.x / g.nct, tt = r0 % g.ntt, b = r0 / g.ntt;
+    const uint32_t wt = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    const uint32_t cbase = ct * WB;
+    const uint32_t t0 = (tt * WT + wt) * R * RPI;
+    if (t0 >= g.L) return;
+    const uint32_t width = g.rowbytes - cbase < WB ? g.rowbytes - cbase : WB;
+    const uint32_t rows = g.L - t0 < R * RPI ? g.L - t0 : R * RPI;
+    const size_t base = ((size_t)b * g.L + t0) * g.rowbytes + cbase;
+    const uint32_t nrec = (rows - 1u) * g.rowbytes + width;
+    __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc((void *)(g.in + base), 0, (int)nrec, 0x00020000);
+    __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)(g.out + base), 0, (int)nrec, 0x00020000);
+    const uint32_t col = (lane % LPR) * VB;
+    const uint32_t voff = col < width ? col + (lane / LPR) * g.rowbytes : 0x80000000u;
+    if constexpr (VB == 8) {
+        u32x2 v[R];
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r) v[r] = __builtin_amdgcn_raw_buffer_load_b64(ri, (int)voff, (int)(r * RPI * g.rowbytes), 2);
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r) __builtin_amdgcn_raw_buffer_store_b64(v[r], ro, (int)voff, (int)(r * RPI * g.rowbytes), 2 | 16);
+    } else {
+        u32x4 v[R];
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r) v[r] = __builtin_amdgcn_raw_buffer_load_b128(ri, (int)voff, (int)(r * RPI * g.rowbytes), 2);
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r) __builtin_amdgcn_raw_buffer_store_b128(v[r], ro, (int)voff, (int)(r * RPI * g.rowbytes), 2 | 16);
+    }
+}
+
+template <int VB, int R, int WT, int LPR>
+static int launch_shape(const void *in, void *out, uint32_t batch, uint32_t rows, uint32_t rowbytes, hipStream_t stream)
+{
+    Tiles g;
+    g.in = (const char *)in;
+    g.out = (char *)out;
+    g.nct = (rowbytes + LPR * VB - 1) / (LPR * VB);
+    g.ntt = (rows + R * WT * (64 / LPR) - 1) / (R * WT * (64 / LPR));
+    g.L = rows;
+    g.rowbytes = rowbytes;
+    g.ncols = batch * g.nct;
+    const uint64_t grid = (uint64_t)batch * g.nct * g.ntt;
+    if (grid >= (1ull << 31)) return 1;
+    hipLaunchKernelGGL((copy_shape_kernel<VB, R, WT, LPR>), dim3((uint32_t)grid), dim3(64 * WT), 0, stream, g);
+    return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
 __global__ void empty_kernel() {}
@@ -89,8 +145,27 @@ __attribute__((visibility("default"))) int copy_tiles(const void *in, void *out,
     const uint64_t grid = (ncols + 7) / 8 * 8 * g.ntt;
     if (grid >= (1ull << 31)) return 1;
     g.ncols = (uint32_t)ncols;
-    hipLaunchKernelGGL(copy_tiles_kernel, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
+    if (2ull * batch * rows * rowbytes >= kThroughBytes) hipLaunchKernelGGL(copy_tiles_kernel<2 | 16>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
+    else hipLaunchKernelGGL(copy_tiles_kernel<2>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
     return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// shape: 0 = 32 rows x 512 B (8-byte lanes, the kernel's tile), 1 = 16 x 512 B (8-byte lanes), 2 = 16 x 1 KB and
+// 3 = 32 x 1 KB (16-byte lanes), 4 = 64 x 256 B (16-byte lanes, four rows per instruction)
+__attribute__((visibility("default"))) int copy_tile_shape(const void *in, void *out, uint32_t batch, uint32_t rows,
+                                                           uint32_t rowbytes, int shape, void *stream)
+{
+    if (rowbytes % 16 || ((uintptr_t)in | (uintptr_t)out) % 16 || batch == 0 || rows == 0 || rowbytes == 0) return 1;
+    if ((uint64_t)rowbytes * 40 >= (1ull << 31)) return 1;   // rows are 32-bit offsets inside a wave's resource
+    hipStream_t s = (hipStream_t)stream;
+    switch (shape) {
+    case 0: return launch_shape<8, 8, 4, 64>(in, out, batch, rows, rowbytes, s);
+    case 1: return launch_shape<8, 4, 4, 64>(in, out, batch, rows, rowbytes, s);
+    case 2: return launch_shape<16, 4, 4, 64>(in, out, batch, rows, rowbytes, s);
+    case 3: return launch_shape<16, 8, 4, 64>(in, out, batch, rows, rowbytes, s);
+    case 4: return launch_shape<16, 4, 4, 16>(in, out, batch, rows, rowbytes, s);
+    default: return 1;
+    }
 }
 
 __attribute__((visibility("default"))) int empty_launch(void *stream)

@@ -306,6 +306,20 @@ int plan_update(const canon_conv1d_update_params *p, UpdPlan *plan)
         return fail(CANON_ERR_INVALID_ARGUMENT, "x, out, conv_state and weight must not be NULL");
     if (p->token_mask && !valid_mask_dtype(p->mask_dtype))
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
+    if (!empty) {
+        // The state is rewritten in place while other threads still read the token and write the output: neither
+        // may lie inside it.  (With a state pool of unstated size the rows the call touches are not known here.)
+        const int xb = elem_bytes(p->x_dtype);
+        const int64_t srows = p->conv_state_indices ? p->state_rows : p->batch;
+        if (srows > 0) {
+            const Extent es = extent_of(p->conv_state, srows, p->channels, p->state_len, p->state_stride_b, p->state_stride_c,
+                                        p->state_stride_s, xb);
+            const Extent ex = extent_of(p->x, p->batch, p->channels, 1, p->x_stride_b, p->x_stride_c, 0, xb);
+            const Extent eo = extent_of(p->out, p->batch, p->channels, 1, p->out_stride_b, p->out_stride_c, 0, xb);
+            if ((ex.lo < es.hi && es.lo < ex.hi && (ex.dense || es.dense)) || (eo.lo < es.hi && es.lo < eo.hi && (eo.dense || es.dense)))
+                return fail(CANON_ERR_INVALID_ARGUMENT, "x and out must not overlap conv_state, which is updated in place");
+        }
+    }
 
     UpdArgs &a = plan->args;
     memset(&a, 0, sizeof(a));

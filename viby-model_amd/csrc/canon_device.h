@@ -869,7 +869,8 @@ __device__ __forceinline__ void decode_taps_contiguous(const TapWords<WDT, E> &r
     }
 }
 
-// Where a block gets its argument block from.  ArgsRead: it was read at the start of the kernel.  ArgsToRead: it
+// Where a block gets its argument block from.  ArgsRead: it was read at the start of the kernel (what every
+// kernel does when the library is built with -DCANON_NO_LATE_ARGS).  ArgsToRead: it
 // is read from the kernel-argument segment AFTER the block has requested its data from the kernel's leading
 // scalar arguments, which arrive in registers with the wave (kernel-argument preload): the data loads are on
 // their way while the argument block is read.  The empty asm is what orders the two: it may write memory, so
@@ -894,6 +895,12 @@ template <typename A> struct ArgsToRead {
         return a;
     }
 };
+
+// A kernel's leading scalar arguments are listed once, as X(type, name) entries of a macro, and expanded with these
+// two into its signature and into the struct that mirrors its kernel-argument segment: the offset of the argument
+// block that follows them cannot drift from the signature.
+#define CANON_LEAD_PARAM(type, name) type name,
+#define CANON_LEAD_FIELD(type, name) type name;
 
 template <typename Args>
 __device__ __forceinline__ uint32_t part_of_block(const PartTable<Args> &m, uint32_t blk)

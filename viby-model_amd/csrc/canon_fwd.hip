@@ -374,11 +374,12 @@ __global__ __launch_bounds__(256) void canon_fwd_bcl_short_kernel(const FwdArgs 
 // its XCD (see blc_block_linear).  The same barrier passes on the taps: the
 // waves of a tile fetch a WT-th of its taps and bias each (every wave fetching
 // all of them cost 3 % at B = 32: 2.5 KB of L2 traffic per 8 KB of x).
-// All loads (slab, history, taps) are issued before the first wait on data.
-// The plain kernel requests slab and history before it has read its argument
+// All loads (history, slab, taps) are issued before the first wait on data.
+// The plain kernel requests history and slab before it has read its argument
 // block (from leading scalar arguments that arrive in registers), which takes
-// the read of the block out of the way: nothing at B 8, C 3456 unmasked,
-// 3 % with a mask, 5-22 % at C 640 / 960.
+// the read of the block out of the way: 3 % with a mask, 5-22 % at C 640 /
+// 960.  In large launches it requests the taps even before those, through
+// two pointers it reads ahead of the block (see blc_block_body).
 // ---------------------------------------------------------------------------
 // One row of a slab: out = act(bias + taps . (history, x)) (+ residual), written through the wave's buffer
 // resource.  ACT / RES / EAGER: the activation flag, the residual mode and the rounding mode when they are
@@ -511,17 +512,13 @@ __device__ __forceinline__ void blc_place(const BlcLead &h, const uint32_t b, co
     g.voff = g.active ? g.lane * VB : 0x80000000u;
 }
 
-// Requests the wave's slab and, for the first wave of a tile, the three rows before it.
+// Requests, for the first wave of a tile, the three rows before its slab, and then the wave's slab.  (The history
+// rows first: they are hits in the L2 of the block's XCD and come back before the slab, whose loads no longer wait
+// in front of them: B 8, C 960 6.7 -> 6.4 us; gate / up as two tensors at B 8 20.7 -> 20.4 us.)
 template <int DT, int W, int R, int VB>
 __device__ __forceinline__ void blc_request(const BlcLead &h, const BlcWave<VB> &g, typename VecIO<VB>::type (&X)[R],
                                             typename VecIO<VB>::type (&H)[3])
 {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        // rows past the end of the sequence: the slab's last row again (loaded, never used)
-        const uint32_t rr = r < g.rows ? (uint32_t)r : (g.rows > 0 ? (uint32_t)(g.rows - 1) : 0u);
-        X[r] = BufIO<VB>::template load<kAuxStream>(g.rx, g.voff, (rr + 3u) * h.xs);
-    }
 #pragma unroll
     for (int j = 0; j < 3; ++j) H[j] = VecIO<VB>::zero();
     if (g.wt == 0 && g.t0 > 0) {
@@ -529,10 +526,22 @@ __device__ __forceinline__ void blc_request(const BlcLead &h, const BlcWave<VB> 
         for (int j = 0; j < 3; ++j)
             if (j >= 3 - (W - 1)) H[j] = BufIO<VB>::template load<kAuxPlain>(g.rx, g.voff, (uint32_t)j * h.xs);
     }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // rows past the end of the sequence: the slab's last row again (loaded, never used)
+        const uint32_t rr = r < g.rows ? (uint32_t)r : (g.rows > 0 ? (uint32_t)(g.rows - 1) : 0u);
+        X[r] = BufIO<VB>::template load<kAuxStream>(g.rx, g.voff, (rr + 3u) * h.xs);
+    }
 }
 
 using ArgsHere = ArgsRead<FwdArgs>;
-using ArgsLate = ArgsToRead<FwdArgs>;
+// ... with the two pointers the taps are fetched through, which the plain kernel receives among its leading
+// scalars: the taps are requested BEFORE the slab, from registers, and wait neither for the slab in front of them
+// in the queue nor for a read of the argument block (a round trip of its own: with the taps requested after it, a
+// wave's taps arrived later than its slab)
+struct ArgsLate : ArgsToRead<FwdArgs> {
+    const void *weight, *bias;
+};
 
 template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE, typename ARGS>
 __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &h, const uint32_t tb, const uint32_t ct, const uint32_t tt,
@@ -550,7 +559,37 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
     blc_place<DT, R, VB>(h, tb, ct, tt, wave);
     // the slab before the argument block where the block is still to be read; otherwise after the taps, which
     // measured 0.4-0.7 us faster at B 8 than slab first
-    if constexpr (ARGS::kLate) blc_request<DT, W, R, VB>(h, wave, X, H);
+    constexpr bool kShare = MODE != TAPS_ANY && kBlcWaves > 1;
+    constexpr int NW = TapWords<WDT, E>::NW, NB = TapWords<WDT, E>::NB;   // words per lane
+    constexpr int PW = NW / WT > 0 ? NW / WT : 1, PB = (NB + WT - 1) / WT;   // words per thread
+    static_assert(!kShare || NW % WT == 0, "taps of a lane split evenly over the waves of a tile");
+    uint32_t tpw[PW], tpb[PB];
+    // The waves that share a channel tile fetch its taps and bias together, each a contiguous WT-th of them, and
+    // pass them on through LDS with the hand-over of the slab tails (one barrier for both).
+    auto fetch_shared_taps = [&](const void *weight, const void *bias, uint32_t nvec_row) {
+        constexpr int WBY = Elem<WDT>::bytes;
+        const uint32_t g = wave.wt * 64u + wave.lane;                 // thread within the tile's group of waves
+        const uint32_t ctile = wave.cv0 < nvec_row ? wave.cv0 * E : 0u;     // first channel of the tile
+        const uint32_t cleft = wave.cv0 < nvec_row ? nvec_row * E - ctile : 0u;
+        const uint32_t wbytes = (cleft < 64u * E ? cleft : 64u * E) * 4u * WBY;
+        const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)weight + (int64_t)ctile * 4 * WBY), 0, (int)wbytes, kBufFlags);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)(bias ? bias : weight) + (int64_t)ctile * WBY), 0, (int)(wbytes / 4u), kBufFlags);
+        buf_load_words<PW>(rw, g * (PW * 4u), tpw);
+        // (words past the tile's bias are out of range of the resource and read zero)
+        buf_load_words<PB>(rb, g * (PB * 4u) < 64u * NB * 4u ? g * (PB * 4u) : 0x80000000u, tpb);
+    };
+    // Where the argument block is still to be read the slab is requested ahead of it.  Small launches request the
+    // taps last: every block of the launch reads the same few lines of taps at the same moment, and a slab queued
+    // behind those loads is late (B 8, C 640 / 960: 5.4 / 6.8 us slab first, 6.2 / 7.6 us taps first).  Large
+    // launches request the taps FIRST, through two pointers read on their own ahead of the block (B 8 / 32, C 3456:
+    // 20.5 -> 20.0 / 73.6 -> 73.0 us; with a mask at B 16: 38.2 -> 38.0 us).
+    constexpr bool kTapsFirst = ARGS::kLate && BIG && kShare;
+    if constexpr (ARGS::kLate) {
+        if constexpr (kTapsFirst) {
+            fetch_shared_taps(args.weight, args.bias, h.nvec);
+        }
+        blc_request<DT, W, R, VB>(h, wave, X, H);
+    }
     const FwdArgs &a = args.get();
     const uint32_t b = wave.b, lane = wave.lane, wv = wave.wv, wt = wave.wt, wc = wave.wc, cv0 = wave.cv0, nl = wave.nl, c0 = wave.c0;
     const uint32_t voff = wave.voff, xs = wave.xs;
@@ -567,24 +606,9 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
     int32_t sq[SEQ ? R + 3 : 1];   // sequence index of rows t0-3 .. t0+R-1
     RawTaps<E> raw;
     TapWords<WDT, E> tw;
-    // The waves that share a channel tile fetch its taps and bias together, each a contiguous WT-th of them, and
-    // pass them on through LDS with the hand-over of the slab tails (one barrier for both).
-    constexpr bool kShare = MODE != TAPS_ANY && WT > 1;
-    constexpr int NW = TapWords<WDT, E>::NW, NB = TapWords<WDT, E>::NB;   // words per lane
-    constexpr int PW = NW / WT > 0 ? NW / WT : 1, PB = (NB + WT - 1) / WT;   // words per thread
-    static_assert(!kShare || NW % WT == 0, "taps of a lane split evenly over the waves of a tile");
-    uint32_t tpw[PW], tpb[PB];
     const uint32_t g = wt * 64u + lane;                         // thread within the tile's group of waves
     if constexpr (kShare) {
-        constexpr int WBY = Elem<WDT>::bytes;
-        const uint32_t ctile = cv0 < a.nvec ? cv0 * E : 0u;     // first channel of the tile
-        const uint32_t cleft = cv0 < a.nvec ? a.C - ctile : 0u;
-        const uint32_t wbytes = (cleft < 64u * E ? cleft : 64u * E) * 4u * WBY;
-        const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.weight + (int64_t)ctile * 4 * WBY), 0, (int)wbytes, kBufFlags);
-        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)(a.bias ? a.bias : a.weight) + (int64_t)ctile * WBY), 0, (int)(wbytes / 4u), kBufFlags);
-        buf_load_words<PW>(rw, g * (PW * 4u), tpw);
-        // (words past the tile's bias are out of range of the resource and read zero)
-        buf_load_words<PB>(rb, g * (PB * 4u) < 64u * NB * 4u ? g * (PB * 4u) : 0x80000000u, tpb);
+        if constexpr (!kTapsFirst) fetch_shared_taps(a.weight, a.bias, a.nvec);
     } else if constexpr (MODE != TAPS_ANY) {
         fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
     }
@@ -754,14 +778,24 @@ __device__ __forceinline__ void blc_block_linear(const FwdArgs &a, const uint32_
     blc_block<DT, W, R, MASK, BIG, SEQ, VB>(ArgsHere{a}, h, (uint32_t)a.tap_mode, b, ct, tt);
 }
 
-// ... and the same in the plain kernel from leading scalar arguments.  `chunk_m`: 2^32 / chunk rounded up (0 for
-// chunk 1), exact for the quotients of block numbers below 2^28 since chunk <= 8.  `packed`: chunk | tap mode
-// << 4 | s1 << 7 | s2 << 8 of the division by nct | s1 << 13 | s2 << 14 of that by ngroups.
+// ... and the same in the plain kernel from leading scalar arguments: fourteen dwords, the most that arrive in
+// registers.  CANON_BLC_LEAD lists them once, for the kernel's signature and for the struct that mirrors the
+// kernel-argument segment (the argument block behind them is read through its offset in that struct).
+// `chunk_m`: 2^32 / chunk rounded up (0 for chunk 1), exact for the quotients of block numbers below 2^28 since
+// chunk <= 8.  `packed`: chunk | tap mode << 4 | s1 << 7 | s2 << 8 of the division by nct | s1 << 13 | s2 << 14 of
+// that by ngroups.
+#define CANON_BLC_LEAD(X)                                                                                            \
+    X(const char *, x) X(int64_t, x_sb) X(uint32_t, xs) X(uint32_t, L) X(uint32_t, nvec) X(uint32_t, ncols)         \
+    X(uint32_t, nct) X(uint32_t, nct_m) X(uint32_t, ngroups) X(uint32_t, ngroups_m) X(uint32_t, chunk_m)            \
+    X(uint32_t, packed)
+struct BlcSegment {
+    CANON_BLC_LEAD(CANON_LEAD_FIELD)
+    FwdArgs a;
+};
+static_assert(offsetof(BlcSegment, a) == 14 * 4, "fourteen leading dwords, then the argument block");
+
 template <int DT, int W, int R, bool MASK, bool BIG>
-__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const char *x, int64_t x_sb, uint32_t xs, uint32_t L, uint32_t nvec,
-                                                                    uint32_t ncols, uint32_t nct, uint32_t nct_m, uint32_t ngroups,
-                                                                    uint32_t ngroups_m, uint32_t chunk_m, uint32_t packed,
-                                                                    const FwdArgs a)
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(CANON_BLC_LEAD(CANON_LEAD_PARAM) const FwdArgs a)
 {
     const uint32_t chunk = packed & 0xFu;
     const uint32_t jq = blockIdx.x >> 3;
@@ -774,14 +808,26 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(const char *
     const uint32_t tt = (qr - b * ngroups) * chunk + (jq - jg * chunk);
     if ((uint64_t)tt * (kBlcWaves * R) >= L) return;   // past the last time tile
     const BlcLead h = {x, x_sb, xs, L, nvec};
-    // the kernel-argument segment lays the arguments out like the members of a struct
-    struct Segment {
-        const char *x;
-        int64_t x_sb;
-        uint32_t xs, L, nvec, ncols, nct, nct_m, ngroups, ngroups_m, chunk_m, packed;
-        FwdArgs a;
-    };
-    blc_block<DT, W, R, MASK, BIG>(ArgsLate{(uint32_t)offsetof(Segment, a)}, h, (packed >> 4) & 3u, b, ct, tt);
+#ifdef CANON_NO_LATE_ARGS
+    // build switch: the argument block read the ordinary way, at the top of the kernel (for a toolchain whose
+    // kernel-argument segment is not laid out like BlcSegment: costs speed, not correctness)
+    blc_block<DT, W, R, MASK, BIG>(ArgsHere{a}, h, (packed >> 4) & 3u, b, ct, tt);
+    return;
+#endif
+    ArgsLate late;
+    late.offset = (uint32_t)offsetof(BlcSegment, a);
+    late.weight = late.bias = nullptr;
+    if constexpr (BIG) {
+        // Large launches fetch the taps before the slab, through these two pointers, which are read on their own
+        // ahead of the argument block (nothing orders the two loads: the compiler issues them at the top of the
+        // kernel, under the tile arithmetic).
+        typedef __attribute__((address_space(4))) const char *kernarg_ptr;
+        typedef __attribute__((address_space(4))) const uintptr_t *word_ptr;
+        kernarg_ptr base = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr() + offsetof(BlcSegment, a);
+        late.weight = (const void *)*(word_ptr)(base + offsetof(FwdArgs, weight));
+        late.bias = (const void *)*(word_ptr)(base + offsetof(FwdArgs, bias));
+    }
+    blc_block<DT, W, R, MASK, BIG>(late, h, (packed >> 4) & 3u, b, ct, tt);
 }
 
 // the same over packed variable-length sequences (seq_idx)

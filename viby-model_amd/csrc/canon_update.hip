@@ -230,21 +230,26 @@ __device__ __forceinline__ void update_vec_block(const ARGS &args, const UpdLead
     update_vec_body<DT, W, S, NB, TAPS_ANY, POOL>(a, bg, c0, X, ST, srow);
 }
 
+// The leading scalars (fourteen dwords: they arrive in registers) listed once, for the kernel's signature and for the
+// struct that mirrors the kernel-argument segment, through which the argument block behind them is read late.
+#define CANON_UPD_LEAD(X)                                                                                         \
+    X(const char *, x) X(char *, state) X(int64_t, x_sb) X(int64_t, s_sb) X(uint32_t, nthreads) X(uint32_t, nvec) \
+    X(uint32_t, B) X(uint32_t, div_m) X(uint32_t, div_s1) X(uint32_t, div_s2)
+struct UpdSegment {
+    CANON_UPD_LEAD(CANON_LEAD_FIELD)
+    UpdArgs a;
+};
+static_assert(offsetof(UpdSegment, a) == 14 * 4, "fourteen leading dwords, then the argument block");
+
 template <int DT, int W, int S, int NB>
-__global__ __launch_bounds__(256) void canon_update_vec_kernel(const char *x, char *state, int64_t x_sb, int64_t s_sb,
-                                                               uint32_t nthreads, uint32_t nvec, uint32_t B, uint32_t div_m,
-                                                               uint32_t div_s1, uint32_t div_s2, const UpdArgs a)
+__global__ __launch_bounds__(256) void canon_update_vec_kernel(CANON_UPD_LEAD(CANON_LEAD_PARAM) const UpdArgs a)
 {
-    // the kernel-argument segment lays the arguments out like the members of a struct
-    struct Segment {
-        const char *x;
-        char *state;
-        int64_t x_sb, s_sb;
-        uint32_t nthreads, nvec, B, div_m, div_s1, div_s2;
-        UpdArgs a;
-    };
     const UpdLead h = {x, state, x_sb, s_sb, nthreads, nvec, B, FastDiv{nvec, div_m, div_s1, div_s2}};
-    update_vec_block<DT, W, S, NB>(ArgsToRead<UpdArgs>{(uint32_t)offsetof(Segment, a)}, h, blockIdx.x);
+#ifdef CANON_NO_LATE_ARGS
+    update_vec_block<DT, W, S, NB>(ArgsRead<UpdArgs>{a}, h, blockIdx.x);
+#else
+    update_vec_block<DT, W, S, NB>(ArgsToRead<UpdArgs>{(uint32_t)offsetof(UpdSegment, a)}, h, blockIdx.x);
+#endif
 }
 
 // the same with batch entry b using row conv_state_indices[b] of a state pool

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 7
+#define CANON_CONV1D_ABI_VERSION 8
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -319,6 +319,16 @@ int canon_conv1d_abi_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *canon_conv1d_last_error(void);
 
+/*
+ * Optional set-up of the CURRENT device, once per GPU and process: loads the library's code objects onto it and
+ * looks up the address of that GPU's copy of the static scratch buffer (see canon_conv1d_bwd_static), which is
+ * where the runtime does its one-time allocations.  Without it the first launch of each kernel family on a device
+ * does the same work by itself.  Call it (or make one warm-up call of every entry point you use) BEFORE capturing
+ * launches into a HIP graph and before a section of the program that must not allocate.  Has no counterpart in
+ * the reference (its Metal library is built and cached on first use, causal_conv1d_mps.mm:35-104).
+ */
+int canon_conv1d_init(void);
+
 /* Enqueue on `stream` (a hipStream_t; NULL = the default stream). */
 int canon_conv1d_fwd(const canon_conv1d_fwd_params *p, void *stream);
 int canon_conv1d_update(const canon_conv1d_update_params *p, void *stream);
@@ -346,7 +356,10 @@ int canon_conv1d_update_parts(const canon_conv1d_update_params *p, const canon_c
  * CANON_CONV1D_STATIC_SCRATCH_BYTES that is part of the library's device image
  * (every GPU the library runs on holds its own copy until the process ends).
  * Nothing is allocated or freed, by the library or by the runtime on its
- * behalf.  A problem whose scratch exceeds the buffer is rejected with
+ * behalf, once the device is set up (canon_conv1d_init, or one earlier call
+ * of this function on the GPU: the first one makes the runtime load the
+ * library's code object, which allocates).  A problem whose scratch exceeds
+ * the buffer is rejected with
  * CANON_ERR_UNSUPPORTED (the metric shape, bf16 [8, 3456, 1024], needs 2.2 MB).
  * All calls on one GPU share that GPU's buffer: calls that overlap in time on
  * one GPU (different streams, different threads) race and must be serialised
@@ -369,6 +382,9 @@ int64_t canon_conv1d_update_bwd_workspace_bytes(const canon_conv1d_update_bwd_pa
  * assert that a layout takes the fast path.
  */
 const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p);
+/* Waves per block of that launch (time-contiguous rows: 8 in unmasked launches of at least 16384 waves, 1 with a
+ * mask, else 4; 4 for the other vector kernels and the strided one), 0 for an empty problem, -1 if rejected. */
+int canon_conv1d_fwd_plan_waves(const canon_conv1d_fwd_params *p);
 const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p);
 const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p);   /* "bwd_blc_vec" | "bwd_bcl_vec" | "bwd_generic" */
 /* "blc_vec_parts" / "update_vec_parts" (one launch) or "per_part" (one launch per part) */

@@ -122,6 +122,22 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     assert plan(fwd_params(C=128, x_stride_b=4096 * 1024, x_stride_c=1024)) == "bcl_vec"
 
 
+def test_fwd_plan_waves_per_block():
+    """Waves per block of the time-contiguous prefill: 1 with a padding mask, 4 in small unmasked launches, 8 from
+    16384 waves; the other kernels run blocks of four."""
+    waves = lambda p: _lib.lib().canon_conv1d_fwd_plan_waves(ctypes.byref(p))
+    assert waves(fwd_params()) == 8                                        # 8 * 3456 rows = 27648 waves
+    assert waves(fwd_params(B=4)) == 4                                     # 13824 waves
+    assert waves(fwd_params(B=4, C=4096)) == 8                             # exactly 16384
+    assert waves(fwd_params(B=4, C=4095)) == 4
+    assert waves(fwd_params(mask=FAKE_STATE, mask_dtype=2, mask_stride_b=1024, mask_stride_l=1)) == 1
+    assert waves(fwd_params(B=32, mask=FAKE_STATE, mask_dtype=4, mask_stride_b=1024, mask_stride_l=1)) == 1
+    assert waves(fwd_params(layout="blc")) == 4
+    assert waves(fwd_params(L=64)) == 4                                    # rows sharing waves
+    assert waves(fwd_params(B=0)) == 0
+    assert waves(fwd_params(width=9)) == -1
+
+
 def test_fwd_validation_messages():
     cases = [
         (dict(struct_size=8), "struct_size"),
@@ -196,7 +212,10 @@ def test_update_plan_and_validation():
     for over, needle in [(dict(S=2), "state_len"), (dict(width=7), "width"),
                          (dict(cache_seqlens=FAKE_STATE + 2), "4-byte aligned"),
                          (dict(conv_state_indices=FAKE_STATE + 1), "4-byte aligned"),
-                         (dict(conv_state=0), "NULL"), (dict(struct_size=4), "struct_size")]:
+                         (dict(conv_state=0), "NULL"), (dict(struct_size=4), "struct_size"),
+                         # the state is rewritten in place: neither the token nor the output may lie inside it
+                         (dict(x=FAKE_STATE + 4096), "overlap"), (dict(out=FAKE_STATE), "overlap"),
+                         (dict(conv_state=FAKE_X - 64), "overlap")]:
         if "S" in over:
             p = update_params(S=over["S"])
         else:
@@ -550,5 +569,5 @@ def test_copy_ceiling_library_exports_what_the_bench_times():
     if not os.path.exists(path):
         pytest.skip("not built (make -C tests/copy_ceiling)")
     lib = ctypes.CDLL(path)
-    for name in ("copy_rows", "copy_tiles", "empty_launch"):
+    for name in ("copy_rows", "copy_tiles", "copy_tile_shape", "empty_launch"):
         assert getattr(lib, name) is not None

@@ -187,3 +187,49 @@ def test_unmodified_model_call_pattern():
                 assert torch.equal(bits(y), bits(want))
             else:
                 assert (y.float().cpu() - want.float()).abs().max() <= 2 ** -7 * want.float().abs().max()
+
+
+def test_prepared_decode_call_agrees_with_the_checked_path():
+    """The decode fast path (a signature seen once is launched from a prepared argument block): second and later
+    calls with a mask that grew, a token that is a non-contiguous view, and a trainable bias under autograd give
+    what the fully checked path gives, and the table of signatures never grows beyond its limit."""
+    import causal_conv1d as cc
+    from oracle import canon_oracle as co
+    torch.manual_seed(9)
+    B, C, dtype = 5, 96, torch.bfloat16
+    w = (torch.randn(C, 4) * 0.3).to(dtype)
+    b = (torch.randn(C) * 0.1).to(dtype)
+    layer = make_layer(C, 4, w, b, False, dtype, "fused")
+    cache = types.SimpleNamespace()
+    state_ref = torch.zeros(B, C, 8, dtype=dtype)
+    with torch.no_grad():
+        for step, width in enumerate([3, 4, 9, 9, 17]):           # the mask's length changes from call to call
+            wide = torch.randn(B, 3, 2 * C).to(dtype)
+            tok = wide[:, 1:2, ::2] if step % 2 else wide[:, 1:2, :C].contiguous()   # strided view / dense token
+            mask = torch.ones(B, width, dtype=torch.int64)
+            mask[step % B, -1] = 0
+            got = layer(tok.to(DEV) if tok.is_contiguous() else wide.to(DEV)[:, 1:2, ::2], attention_mask=mask.to(DEV),
+                        cache=cache, layer_idx=0)
+            xt = tok[:, 0] * mask[:, -1:].to(dtype)
+            want = tok[:, 0] + co.conv1d_update(xt.contiguous(), state_ref, w, b)   # the residual is the unmasked token
+            assert torch.equal(bits(cache.canon_cache_a[0]), bits(state_ref)), step
+            assert_parity(got[:, 0], want.to(dtype), exact=False, what=f"step {step}", res=tok[:, 0])
+    # a frozen weight with a trainable bias takes the autograd path, not the prepared launch
+    layer.weight.requires_grad_(False)
+    layer.bias_param.requires_grad_(True)
+    tok = torch.randn(B, 1, C).to(dtype).to(DEV)
+    y = layer(tok, attention_mask=None, cache=types.SimpleNamespace(), layer_idx=0)
+    assert y.requires_grad
+    y.float().sum().backward()
+    assert layer.bias_param.grad is not None and torch.isfinite(layer.bias_param.grad.float()).all()
+    # the table keeps its size: new signatures push the oldest ones out
+    known = cc._known_updates()
+    with torch.no_grad():
+        for n in range(cc._KNOWN_UPDATES_MAX + 8):
+            x = torch.zeros(1, 2 + 2 * n, dtype=dtype, device=DEV)
+            st = torch.zeros(1, 2 + 2 * n, 3, dtype=dtype, device=DEV)
+            wt = torch.zeros(2 + 2 * n, 4, dtype=dtype, device=DEV)
+            cc.causal_conv1d_update(x, st, wt)
+            cc.causal_conv1d_update(x, st, wt)
+    assert len(known) == cc._KNOWN_UPDATES_MAX
+    torch.cuda.synchronize()

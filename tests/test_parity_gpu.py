@@ -9,7 +9,7 @@ import itertools
 import pytest
 import torch
 
-from helpers import assert_parity, bits, right_padded_mask
+from helpers import assert_parity, bits, right_padded_mask, ulp_diff
 from oracle import canon_oracle as co
 
 pytestmark = pytest.mark.gpu
@@ -386,6 +386,71 @@ def test_eager_rounding_matches_eager_module(cc, dtype, act):
         assert_parity(got, want, exact=(not act and dtype != torch.float32), what="eager step", res=xt[:, 0])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_eager_rounding_with_silu_vs_the_c_oracle_in_both_layouts(cc, dtype, capsys):
+    """rounding='eager' with SiLU and a residual against the C oracle's round_mode = 1 (rounds after the conv, after
+    the activation and at the store), in the vector kernels of both layouts and with a padding mask: within one
+    unit in the last place of the output itself (the GPU divides and exponentiates in fp32 like libm but not
+    with libm's code), and the share of outputs that are bit equal is printed."""
+    g = torch.Generator().manual_seed(131)
+    B, C, L = 3, 264, 520
+    x = torch.randn(B, C, L, generator=g).to(dtype)
+    w = (torch.randn(C, 4, generator=g) * 0.4).to(dtype)
+    b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+    mask = right_padded_mask([520, 300, 7], L)
+    for m, res in ((None, False), (None, "unmasked"), (mask, "masked")):
+        want, want_state = co.conv1d_fwd(x, w, b, activation="silu", mask=m, residual=res, final_state_len=8, round_mode=1)
+        for name, xg in layouts(x):
+            assert cc.kernel_plan_fwd(xg, w.to(DEV), rounding="eager") == f"{name}_vec"
+            got, state = run_fwd(cc, xg, w, b, act="silu", mask=m, residual=res, S_out=8, rounding="eager")
+            assert torch.equal(bits(state), bits(want_state))
+            d = ulp_diff(got, want)
+            equal = (d == 0).float().mean().item()
+            # the eager mode rounds the activation before the residual is added, so what reaches the sum is a
+            # storage-type value on both sides: one step of it apart at most, which the sum's rounding may keep
+            xm = x if m is None else x * m.unsqueeze(1).to(dtype)
+            assert_parity(got, want, exact=False, what=f"eager silu/{name}/res{res}", res=xm if res else None)
+            with capsys.disabled():
+                print(f"\n[eager rounding + SiLU, {str(dtype)[6:]}, {name}, residual {res}] bit equal {equal * 100:.2f} %, "
+                      f"largest distance {d.max().item()} ulp of the output")
+
+
+def test_silu_with_residual_literal_ulp_distance(cc, capsys):
+    """The optional-activation variant at configuration 2's largest shape: SiLU and a residual, one rounding.  The
+    bar of this repository measures the 1 ulp against the larger of the output and the residual term (the sum
+    cancels).  Reported here as well: the literal distance in units of the OUTPUT's last place, which is large
+    exactly where x + silu(conv) cancels, and the same distance for the oracle evaluated with float32 libm against
+    float64: any two correct evaluations of the activation differ there."""
+    import numpy as np
+    g = torch.Generator().manual_seed(3456)
+    B, C, L = 8, 3456, 1024
+    x = torch.randn(B, C, L, generator=g).bfloat16()
+    w = (torch.randn(C, 4, generator=g) * 0.02).bfloat16()
+    b = (torch.randn(C, generator=g) * 0.01).bfloat16()
+    want = co.conv1d_fwd(x, w, b, activation="silu", residual=1)
+    # the same in float64 (exact products and sums of bf16 values up to the activation)
+    xd, wd = x.double(), w.double()
+    xp = torch.nn.functional.pad(xd, (3, 0))
+    z = b.double()[None, :, None] + sum(wd[None, :, k, None] * xp[:, :, k:k + L] for k in range(4))
+    ref64 = (xd + z / (1 + torch.exp(-z))).bfloat16()
+    for name, xg in layouts(x):
+        got = run_fwd(cc, xg, w, b, act="silu", residual=True)
+        assert_parity(got, want, exact=False, what=f"silu+residual/{name}", res=x)
+        d = ulp_diff(got, want)
+        d64 = ulp_diff(want, ref64)
+        hist = np.bincount(d.flatten().numpy().clip(max=3), minlength=4)
+        worst = d.max().item()
+        at = tuple(int(i) for i in (d == worst).nonzero()[0])
+        with capsys.disabled():
+            print(f"\n[SiLU + residual, bf16 [8,3456,1024], {name}] literal distance to the oracle in ulp of the output: "
+                  f"0: {hist[0]}, 1: {hist[1]}, 2: {hist[2]}, >= 3: {hist[3]} elements; largest {worst} at {at} where "
+                  f"out = {want[at].item():.3e}, x = {x[at].item():.3e} (the sum cancels); the oracle itself is up to "
+                  f"{d64.max().item()} ulp from a float64 evaluation")
+        # away from cancellation (|out| at least half of |x|) the literal distance is within one ulp
+        plain = want.float().abs() >= 0.5 * x.float().abs()
+        assert d[plain].max().item() <= 1
+
+
 def test_errors_surface(cc):
     x = torch.randn(2, 8, 16, device=DEV)
     w = torch.randn(8, 4, device=DEV)
@@ -542,7 +607,7 @@ def test_time_contiguous_rows_off_the_16_byte_grid(cc, dtype):
 
 def test_large_time_contiguous_launches_in_blocks_of_eight_waves(cc):
     """Unmasked time-contiguous launches of 16384 waves or more run in blocks of eight waves: a last block that is
-    not full, rows off the 16-byte grid, rows of two segments; and the same rows with a mask (blocks of four)."""
+    not full, rows off the 16-byte grid, rows of two segments; and the same rows with a mask (single-wave blocks)."""
     g = torch.Generator().manual_seed(97)
     for (B, C, L) in [(7, 2403, 1023), (2, 4211, 4100)]:
         x = torch.randn(B, C, L, generator=g).bfloat16()
@@ -551,6 +616,10 @@ def test_large_time_contiguous_launches_in_blocks_of_eight_waves(cc):
         mask = right_padded_mask(torch.randint(1, L + 1, (B,), generator=g).tolist(), L)
         xg = x.to(DEV)
         assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec", (B, C, L)
+        # the three regimes of the block size: eight waves here, one with a mask, four in a small launch
+        assert cc.kernel_plan_fwd_waves(xg, w.to(DEV)) == 8, (B, C, L)
+        assert cc.kernel_plan_fwd_waves(xg, w.to(DEV), attention_mask=mask.to(DEV)) == 1
+        assert cc.kernel_plan_fwd_waves(xg[:1, :512], w[:512].to(DEV)) == 4
         for m, res in ((None, True), (mask, "masked")):
             want, want_state = co.conv1d_fwd(x, w, b, mask=m, residual=res, final_state_len=8)
             got, state = run_fwd(cc, xg, w, b, mask=m, residual=res, S_out=8)

@@ -118,3 +118,76 @@ def test_static_scratch_backward_rejects_what_does_not_fit():
     rc = L.canon_conv1d_bwd_static(ctypes.byref(p), None)
     assert rc == _lib.ERR_UNSUPPORTED
     assert "static buffer holds 8388608" in L.canon_conv1d_last_error().decode()
+
+
+def _problem(_lib, shape, seed):
+    """One channel-contiguous bf16 problem with its argument block (workspace fields unset)."""
+    g = torch.Generator().manual_seed(seed)
+    B, C, T = shape
+    x = torch.randn(B, T, C, generator=g).bfloat16().to(DEV).transpose(1, 2)
+    dout = torch.randn(B, T, C, generator=g).bfloat16().to(DEV).transpose(1, 2)
+    weight = (torch.randn(C, 4, generator=g) * 0.3).bfloat16().to(DEV)
+    bias = (torch.randn(C, generator=g) * 0.1).bfloat16().to(DEV)
+    dx = torch.empty_like(x)
+    dweight = torch.empty(C, 4, dtype=torch.float32, device=DEV)
+    dbias = torch.empty(C, dtype=torch.float32, device=DEV)
+    p = _params(_lib, x, dout, dx, weight, bias, None, dweight, dbias, 1, 1)
+    return p, (x, dout, weight, bias), (dx, dweight, dbias)
+
+
+def test_static_scratch_backward_allocates_nothing_after_the_device_is_set_up():
+    """Free device memory as the driver reports it is the same before and after calls of the static-scratch entry
+    point, once canon_conv1d_init has set the device up (the code objects and the scratch array are in place)."""
+    from causal_conv1d import _lib
+    L = _lib.lib()
+    assert L.canon_conv1d_init() == 0, L.canon_conv1d_last_error().decode()
+    assert L.canon_conv1d_init() == 0                       # idempotent
+    p, keep, outs = _problem(_lib, (4, 640, 512), 11)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # one warm-up call: whatever the runtime sets up at a kernel's first launch is in place after it
+    assert L.canon_conv1d_bwd_static(ctypes.byref(p), stream) == 0, L.canon_conv1d_last_error().decode()
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert L.canon_conv1d_bwd_static(ctypes.byref(p), stream) == 0, L.canon_conv1d_last_error().decode()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"free device memory changed by {free0 - free1} bytes across calls that must not allocate"
+
+
+def test_static_scratch_backward_captured_in_a_hip_graph_replays_exactly():
+    """The call recorded into a HIP graph (what it exists for) and replayed several times, with eager work and
+    synchronisations in between and the inputs rewritten before every replay: each replay equals
+    canon_conv1d_bwd on the same inputs bit for bit."""
+    from causal_conv1d import _lib
+    L = _lib.lib()
+    assert L.canon_conv1d_init() == 0
+    p, (x, dout, weight, bias), (dx, dweight, dbias) = _problem(_lib, (3, 960, 384), 12)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                           # warm-up outside the capture
+        assert L.canon_conv1d_bwd_static(ctypes.byref(p), ctypes.c_void_p(side.cuda_stream)) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = L.canon_conv1d_bwd_static(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, L.canon_conv1d_last_error().decode()
+    g = torch.Generator(device=DEV).manual_seed(13)
+    for replay in range(3):
+        x.copy_(torch.randn(x.shape, generator=g, device=DEV))          # new inputs in the captured buffers
+        dout.copy_(torch.randn(dout.shape, generator=g, device=DEV))
+        for t in (dx, dweight, dbias):
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (dx, dweight, dbias)]
+        # the reference: the workspace call, launched eagerly on the same inputs
+        want = [torch.full_like(t, float("nan")) for t in (dx, dweight, dbias)]
+        q = _params(_lib, x, dout, want[0], weight, bias, None, want[1], want[2], 1, 1)
+        nbytes = L.canon_conv1d_bwd_workspace_bytes(ctypes.byref(q))
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+        q.workspace, q.workspace_bytes = workspace.data_ptr(), nbytes
+        assert L.canon_conv1d_bwd(ctypes.byref(q), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+        torch.cuda.synchronize()
+        _same(got, want)

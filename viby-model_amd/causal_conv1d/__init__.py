@@ -39,7 +39,9 @@ __all__ = [
     "causal_conv1d_update_parts",
     "short_conv_fused",
     "short_conv_update",
+    "prepare_device",
     "kernel_plan_fwd",
+    "kernel_plan_fwd_waves",
     "kernel_plan_update",
     "kernel_plan_fwd_parts",
     "kernel_plan_update_parts",
@@ -505,7 +507,8 @@ def causal_conv1d_update(
     # prepared argument block with only the five addresses filled in.
     if cache_seqlens is None and conv_state_indices is None and not (
             torch.is_grad_enabled() and (x.requires_grad or weight.requires_grad or conv_state.requires_grad
-                                         or (bias is not None and bias.requires_grad))):
+                                         or (bias is not None and bias.requires_grad)
+                                         or (token_mask is not None and token_mask.requires_grad))):
         key = (x.shape, x.stride(), x.dtype, x.device, conv_state.shape, conv_state.stride(), conv_state.dtype,
                conv_state.device, weight.shape, weight.stride(), weight.dtype, weight.device,
                None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device),
@@ -581,10 +584,10 @@ def causal_conv1d_update(
                                             act, res, rnd)
     else:
         out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
-        if (key is not None and not squeeze_back and out.numel() and len(_known_updates()) < _KNOWN_UPDATES_MAX
+        if (key is not None and not squeeze_back and out.numel()
                 and (bias is None or (bias.dtype == weight.dtype and bias.is_contiguous()))):
             # the call went through: remember its signature with an argument block whose sizes, strides and flags are set
-            _known_updates()[key] = _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd)
+            _remember_update(key, _fill_update(x2, out, conv_state, weight, bias, token_mask, act, res, rnd))
     return out.unsqueeze(-1) if squeeze_back else out
 
 
@@ -602,8 +605,8 @@ def _canon_decode_step(x: torch.Tensor, conv_state: torch.Tensor, taps: torch.Te
     key = (x.shape, x.stride(), x.dtype, x.device, conv_state.shape, conv_state.stride(), conv_state.dtype,
            conv_state.device, taps.shape, taps.stride(), taps.dtype, taps.device,
            None if bias is None else (bias.shape, bias.stride(), bias.dtype, bias.device),
-           None if attention_mask is None else (attention_mask.shape[0], attention_mask.stride(1), attention_mask.dtype,
-                                                attention_mask.device),
+           None if attention_mask is None else (attention_mask.dim(), attention_mask.shape[0], attention_mask.stride(1),
+                                                attention_mask.dtype, attention_mask.device),
            activation, rounding)
     known = _known_updates()
     p = known.get(key)
@@ -611,11 +614,10 @@ def _canon_decode_step(x: torch.Tensor, conv_state: torch.Tensor, taps: torch.Te
         token_mask = attention_mask[:, -1] if attention_mask is not None else None
         y = causal_conv1d_update(x[:, 0], conv_state, taps, bias, activation=activation, token_mask=token_mask,
                                  residual="unmasked", rounding=rounding)
-        if y.numel() and len(known) < _KNOWN_UPDATES_MAX and (
-                bias is None or (bias.dtype == taps.dtype and bias.is_contiguous())):
+        if y.numel() and (bias is None or (bias.dtype == taps.dtype and bias.is_contiguous())):
             # x[:, 0] and a contiguous (batch, dim) output: the strides of every later call with this signature
-            known[key] = _fill_update(x[:, 0], y, conv_state, taps, bias, token_mask, _activation_flag(activation),
-                                      _residual_mode("unmasked"), _round_mode(rounding))
+            _remember_update(key, _fill_update(x[:, 0], y, conv_state, taps, bias, token_mask, _activation_flag(activation),
+                                               _residual_mode("unmasked"), _round_mode(rounding)))
         return y.unsqueeze(1)
     out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
     p.x, p.out, p.conv_state, p.weight = x.data_ptr(), out.data_ptr(), conv_state.data_ptr(), taps.data_ptr()
@@ -641,6 +643,15 @@ def _known_updates() -> dict:
     except AttributeError:
         _update_tls.known = {}
         return _update_tls.known
+
+
+def _remember_update(key, block) -> None:
+    """Keep at most _KNOWN_UPDATES_MAX signatures per thread: the oldest one makes room (a model has a handful of
+    distinct decode calls; a program that keeps producing new ones must not lose the fast path for good)."""
+    known = _known_updates()
+    if len(known) >= _KNOWN_UPDATES_MAX:
+        known.pop(next(iter(known)))
+    known[key] = block
 
 
 def _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
@@ -1139,6 +1150,27 @@ def kernel_plan_fwd(x, weight, bias=None, activation=None, attention_mask=None, 
     if name is None:
         _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_fwd")
     return name.decode()
+
+
+def kernel_plan_fwd_waves(x, weight, bias=None, activation=None, attention_mask=None, residual=False,
+                          rounding="fused") -> int:
+    """Waves per block of the launch ``causal_conv1d_fn`` would make (1, 4 or 8 for time-contiguous rows, else 4)."""
+    out = torch.empty_like(x)
+    p = _fill_fwd(x, out, weight, _prep_bias(weight, bias), attention_mask, None, None,
+                  _activation_flag(activation), _residual_mode(residual), _round_mode(rounding))
+    n = _lib.lib().canon_conv1d_fwd_plan_waves(ctypes.byref(p))
+    if n < 0:
+        _lib.check(_lib.ERR_INVALID_ARGUMENT, "kernel_plan_fwd_waves")
+    return n
+
+
+def prepare_device(device=None) -> None:
+    """Set the library up on ``device`` (default: the current one): loads its code objects and resolves the static
+    scratch buffer, so that nothing of that is left to the first launches.  Call it before capturing launches
+    into a HIP graph or entering a section that must not allocate device memory."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().canon_conv1d_init(), "prepare_device")
 
 
 def kernel_plan_update(x, conv_state, weight, bias=None, activation=None, residual=False, rounding="fused") -> str:

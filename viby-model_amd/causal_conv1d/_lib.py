@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -120,7 +120,9 @@ EXPORTS = (
     "canon_conv1d_last_error",
     "canon_conv1d_fwd",
     "canon_conv1d_update",
+    "canon_conv1d_init",
     "canon_conv1d_fwd_plan",
+    "canon_conv1d_fwd_plan_waves",
     "canon_conv1d_update_plan",
     "canon_conv1d_bwd",
     "canon_conv1d_bwd_static",
@@ -154,6 +156,10 @@ def lib() -> ctypes.CDLL:
         L.canon_conv1d_fwd.argtypes = [ctypes.POINTER(FwdParams), _vp]
         L.canon_conv1d_update.restype = ctypes.c_int
         L.canon_conv1d_update.argtypes = [ctypes.POINTER(UpdateParams), _vp]
+        L.canon_conv1d_init.restype = ctypes.c_int
+        L.canon_conv1d_init.argtypes = []
+        L.canon_conv1d_fwd_plan_waves.restype = ctypes.c_int
+        L.canon_conv1d_fwd_plan_waves.argtypes = [ctypes.POINTER(FwdParams)]
         L.canon_conv1d_fwd_plan.restype = ctypes.c_char_p
         L.canon_conv1d_fwd_plan.argtypes = [ctypes.POINTER(FwdParams)]
         L.canon_conv1d_update_plan.restype = ctypes.c_char_p

@@ -124,7 +124,8 @@ class CanonLayer(nn.Module):
             if state is None:
                 state = torch.zeros(B, D, self._state_len(), dtype=x.dtype, device=x.device)
                 slot[layer_idx] = state
-            if torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad or state.requires_grad):
+            if torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad or state.requires_grad
+                                            or (self.bias_param is not None and self.bias_param.requires_grad)):
                 y = causal_conv1d_update(x[:, 0], state, self._taps(), self.bias_param, activation=act,
                                          token_mask=token_mask[:, -1] if token_mask is not None else None,
                                          residual="unmasked", rounding=self.rounding)

@@ -861,37 +861,54 @@ CANON_API int64_t canon_conv1d_bwd_workspace_bytes(const canon_conv1d_bwd_params
 constexpr int64_t kStaticScratchBytes = CANON_CONV1D_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
+// Device address of the current GPU's copy, looked up once per device (by canon_conv1d_init, else by the first
+// call of canon_conv1d_bwd_static on that GPU: the lookup makes the runtime load this file's code object, which
+// is when the array's memory is allocated).
+static int static_scratch(const char *who, void **out)
+{
+    constexpr int kMaxDevices = 64;
+    static void *ptr_of_device[kMaxDevices];
+    static std::mutex lookup;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(CANON_ERR_UNSUPPORTED, "%s: device %d", who, dev);
+    std::lock_guard<std::mutex> hold(lookup);
+    if (!ptr_of_device[dev]) {
+        void *q = nullptr;
+        e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !q) return fail(CANON_ERR_LAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+        ptr_of_device[dev] = q;
+    }
+    *out = ptr_of_device[dev];
+    return CANON_OK;
+}
+
+CANON_API int canon_conv1d_init(void)
+{
+    void *ptr;
+    const int rc = static_scratch("canon_conv1d_init", &ptr);
+    if (rc != CANON_OK) return rc;
+    const hipError_t loaded[3] = {preload_fwd(), preload_update(), preload_bwd()};
+    for (hipError_t e : loaded)
+        if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "canon_conv1d_init: loading the kernels: %s", hipGetErrorString(e));
+    return CANON_OK;
+}
+
 CANON_API int canon_conv1d_bwd_static(const canon_conv1d_bwd_params *p, void *stream)
 {
     if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(canon_conv1d_bwd_params))
         return fail(CANON_ERR_INVALID_ARGUMENT, "struct_size %u does not match this library's canon_conv1d_bwd_params (%zu)",
                     p->struct_size, sizeof(canon_conv1d_bwd_params));
-    // device address of this GPU's copy, looked up once per device
-    constexpr int kMaxDevices = 64;
-    static void *ptr_of_device[kMaxDevices];
-    static std::mutex lookup;
-    int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return fail(CANON_ERR_LAUNCH, "canon_conv1d_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
-    if (dev < 0 || dev >= kMaxDevices) return fail(CANON_ERR_UNSUPPORTED, "canon_conv1d_bwd_static: device %d", dev);
     void *ptr;
-    {
-        std::lock_guard<std::mutex> hold(lookup);
-        if (!ptr_of_device[dev]) {
-            void *q = nullptr;
-            e = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
-            if (e != hipSuccess || !q)
-                return fail(CANON_ERR_LAUNCH, "canon_conv1d_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
-            ptr_of_device[dev] = q;
-        }
-        ptr = ptr_of_device[dev];
-    }
+    int rc = static_scratch("canon_conv1d_bwd_static", &ptr);
+    if (rc != CANON_OK) return rc;
     canon_conv1d_bwd_params q = *p;
     q.workspace = ptr;
     q.workspace_bytes = kStaticScratchBytes;
     BwdPlan pl;
-    int rc = plan_bwd(&q, &pl, false);
+    rc = plan_bwd(&q, &pl, false);
     if (rc != CANON_OK) return rc;
     if (pl.workspace_bytes > kStaticScratchBytes)
         return fail(CANON_ERR_UNSUPPORTED,
@@ -942,6 +959,14 @@ CANON_API const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p)
     if (pl.kind == FWD_BLC && pl.args.seq) return "blc_vec_seq";
     if (pl.kind == FWD_BCL_SHORT) return "bcl_vec_short";
     return pl.kind == FWD_BCL ? "bcl_vec" : pl.kind == FWD_BLC ? "blc_vec" : "generic";
+}
+
+CANON_API int canon_conv1d_fwd_plan_waves(const canon_conv1d_fwd_params *p)
+{
+    FwdPlan pl;
+    if (plan_fwd(p, &pl) != CANON_OK) return -1;
+    if (pl.grid == 0) return 0;
+    return pl.kind == FWD_BCL ? (int)pl.wpb : 4;
 }
 
 CANON_API const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p)

@@ -1344,6 +1344,13 @@ void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s)
                            pl.args.dweight, pl.args.dbias, pl.args.C, pl.args.ngroups, pl.args.W);
 }
 
+// Asking for a kernel's attributes makes the runtime load this file's code object onto the current device.
+hipError_t preload_bwd()
+{
+    hipFuncAttributes attr;
+    return hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&canon_zero_kernel));
+}
+
 void launch_zero(float *p, uint32_t n, hipStream_t s)
 {
     if (n) hipLaunchKernelGGL(canon_zero_kernel, dim3((n + 255) / 256), dim3(256), 0, s, p, n);

@@ -264,6 +264,11 @@ void launch_update_parts(const UpdPartsPlan &pp, int x_dtype, hipStream_t s);
 void launch_bwd(const BwdPlan &pl, int x_dtype, hipStream_t s);          // dx + partial sets, then the reduction
 void launch_update_bwd(const UpdBwdPlan &pl, int x_dtype, hipStream_t s);   // dx, dstate + partial sets, then the reduction
 void launch_zero(float *p, uint32_t n, hipStream_t s);                    // fill kernel (graph-capture safe)
+// Make the runtime load this translation unit's code object onto the current device now (it would otherwise do so
+// at the unit's first launch): hipSuccess or the runtime's error.
+hipError_t preload_fwd();
+hipError_t preload_update();
+hipError_t preload_bwd();
 
 }  // namespace canon
 #endif  // CANON_PLAN_H

@@ -425,6 +425,13 @@ template <int DT> void launch_update_parts_t(const UpdPartsPlan &pp, hipStream_t
 
 }  // namespace
 
+// Asking for a kernel's attributes makes the runtime load this file's code object onto the current device.
+hipError_t preload_update()
+{
+    hipFuncAttributes attr;
+    return hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&(canon_update_generic_kernel<CANON_DTYPE_F32>)));
+}
+
 void launch_update(const UpdPlan &pl, int x_dtype, hipStream_t s)
 {
     switch (x_dtype) {

@@ -602,9 +602,9 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
             return CANON_OK;
         }
     }
-    // channel-contiguous tensors: 8-byte groups of channels per lane
-    const int E8 = 8 / elem_bytes(p->x_dtype);
-    const bool ptrs8 = (((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & 7u) == 0;
+    // channel-contiguous tensors: a group of kBwdVecBytes of adjacent channels per lane
+    const int E8 = kBwdVecBytes / elem_bytes(p->x_dtype);
+    const bool ptrs8 = (((uintptr_t)p->x | (uintptr_t)p->dout | (uintptr_t)p->dx) & (uintptr_t)(kBwdVecBytes - 1)) == 0;
     const bool vec = !packed && a.x_sc == 1 && a.g_sc == 1 && a.d_sc == 1 && a.C % E8 == 0 && a.x_sl != 1 &&
                      a.x_sb % E8 == 0 && a.x_sl % E8 == 0 && a.g_sb % E8 == 0 && a.g_sl % E8 == 0 &&
                      a.d_sb % E8 == 0 && a.d_sl % E8 == 0 && ptrs8;

@@ -295,47 +295,31 @@ __global__ __launch_bounds__(256) void canon_bwd_walk_kernel(const BwdArgs a)
 // x and dout are read once and dx is written once: streamed (non-temporal) accesses, as in the forward kernels
 // (measured at B 8, C 3456, L 1024, bf16: 40.7 -> 37.8 us channel-contiguous, 33.6 -> 30.9 us time-contiguous).
 constexpr bool kBwdStream = true;
-template <int DT> __device__ __forceinline__ void unpack_half(const uint2 &v, float *f)
-{
-    if constexpr (DT == CANON_DTYPE_F32) {
-        f[0] = bits_f(v.x);
-        f[1] = bits_f(v.y);
-    } else {
-        unpack2<DT>(v.x, f[0], f[1]);
-        unpack2<DT>(v.y, f[2], f[3]);
-    }
-}
-
-template <int DT> __device__ __forceinline__ uint2 pack_half(const float *f)
-{
-    if constexpr (DT == CANON_DTYPE_F32) return make_uint2(f_bits(f[0]), f_bits(f[1]));
-    else return make_uint2(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]));
-}
+using BV = VecIO<kBwdVecBytes>;
+using BVT = BV::type;   // a lane's piece of one row
+template <int DT> __device__ __forceinline__ void unpack_half(const BVT &v, float *f) { BV::template unpack<DT>(v, f); }
+template <int DT> __device__ __forceinline__ BVT pack_half(const float *f) { return BV::template pack<DT>(f); }
 
 // One raw row -> the bits of xm = x * mask in the storage type (zero when the row does not exist)
 template <int DT, bool MASK>
-__device__ __forceinline__ uint2 bwd_mask_row(const uint2 &raw, float m, bool exists)
+__device__ __forceinline__ BVT bwd_mask_row(const BVT &raw, float m, bool exists)
 {
-    uint2 v = raw;
+    constexpr int E = kBwdVecBytes / Elem<DT>::bytes;
+    BVT v = raw;
     if constexpr (MASK) {
       // m is the same for the whole wave and 1 for every valid token of a padded batch: x * 1 is x, bit for bit
       if (m != 1.0f) {
-        if constexpr (DT == CANON_DTYPE_F32) {
-            v.x = f_bits(bits_f(raw.x) * m);
-            v.y = f_bits(bits_f(raw.y) * m);
-        } else {
-            float f[4];
-            unpack_half<DT>(raw, f);
+        float f[E];
+        unpack_half<DT>(raw, f);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                f[e] *= m;
-                if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(f[e]));   // see mul_round
-            }
-            v = pack_half<DT>(f);
+        for (int e = 0; e < E; ++e) {
+            f[e] *= m;
+            if constexpr (DT == CANON_DTYPE_F16) asm volatile("" : "+v"(f[e]));   // see mul_round
         }
+        v = pack_half<DT>(f);
       }
     }
-    if (!exists) v = make_uint2(0, 0);
+    if (!exists) v = BV::zero();
     return v;
 }
 
@@ -366,8 +350,8 @@ __device__ __forceinline__ void bwd_dz(const float (*w)[W], const float *bias, c
 // (slot t - fin_first for t >= fin_first = L - S_out) and get that slot's gradient, read at `fin` (the lane's
 // first channel of slot 0) where it is needed: at most S_out steps per sequence.
 template <int DT, int W, bool MASK, bool ACT, bool FULL, bool FIN, int R, int E>
-__device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W], const float *bias, const uint2 *X,
-                                          const uint2 *H, const uint2 *G, const float *mm, const float (*dzh)[E],
+__device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W], const float *bias, const BVT *X,
+                                          const BVT *H, const BVT *G, const float *mm, const float (*dzh)[E],
                                           float (*dzf)[E], float (*dw)[W], float *dbs, char *dxp, int64_t ds, int rows,
                                           bool active, const char *fin = nullptr, int64_t fin_first_row = 0)
 {
@@ -431,7 +415,7 @@ __device__ __forceinline__ void bwd_sweep(const BwdArgs &a, const float (*w)[W],
 #pragma unroll
             for (int e = 0; e < E; ++e) o[e] += g[e];
         }
-        if ((FULL || r < rows) && active) VecIO<8>::store<kBwdStream>(dxp + r * ds, pack_half<DT>(o));
+        if ((FULL || r < rows) && active) BV::store<kBwdStream>(dxp + r * ds, pack_half<DT>(o));
         if (r > 0) {
             // slide the window one step back: the new oldest row is r - 4
 #pragma unroll
@@ -452,15 +436,15 @@ template <int DT, int W, bool MASK, bool ACT, bool STATES>
 __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
 {
     constexpr int BY = Elem<DT>::bytes;
-    constexpr int E = 8 / BY;
+    constexpr int E = kBwdVecBytes / BY;
     constexpr int R = kBwdSlab, NW = kBwdWaves;
     // With an activation: tailx / headdz, two barriers per tile (dz of a slab's head needs the previous
     // wave's tail first).  Without one dz IS dout, so the head is handed over as raw rows (headg) together
     // with the tail, one barrier per tile, both double-buffered (a fast wave publishes the next tile while
     // a slow one still reads this one).
-    __shared__ uint2 tailx[ACT ? 1 : 2][NW][3][64];            // last three xm rows of each wave's slab (storage bits)
+    __shared__ BVT tailx[ACT ? 1 : 2][NW][3][64];            // last three xm rows of each wave's slab (storage bits)
     __shared__ float headdz[ACT ? NW : 1][3][ACT ? E : 1][64];  // dz of the first three steps of each wave's slab
-    __shared__ uint2 headg[2][ACT ? 1 : NW][3][64];            // ACT == false: the first three dout rows of each slab
+    __shared__ BVT headg[2][ACT ? 1 : NW][3][64];            // ACT == false: the first three dout rows of each slab
     __shared__ float red[NW - 1][5 * E][64];      // dweight / dbias sums of waves 1..3
     // mask entries of steps t_chunk-3 .. t_chunk+chunk+2 as floats.  Staged once per block: inside the
     // time loop (after the first store to dx) the compiler can no longer use scalar loads for them, and
@@ -510,38 +494,38 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
     if constexpr (!ACT) {
         // no activation: the three dz after the chunk are three rows of dout, kept by the last wave
         const int64_t te = t_chunk + (int64_t)a.chunk;
-        uint2 GE[3];
+        BVT GE[3];
 #pragma unroll
-        for (int j = 0; j < 3; ++j) GE[j] = make_uint2(0, 0);
+        for (int j = 0; j < 3; ++j) GE[j] = BV::zero();
         if (wv == NW - 1) {
 #pragma unroll
             for (int j = 0; j < 3; ++j)
-                if (te + j <= Lm1) GE[j] = *(const uint2 *)(gb + (te + j) * gs);
+                if (te + j <= Lm1) GE[j] = BV::load<false>(gb + (te + j) * gs);
         }
         decode_taps<DT, W, E>(rawt, a.w_dtype, a.w_vec != 0, a.bias != nullptr, w, bias);
 #pragma unroll
         for (int j = 0; j < 3; ++j) unpack_half<DT>(GE[j], dzf[j]);
     } else {
         const int64_t te = t_chunk + (int64_t)a.chunk;   // first step after the chunk (at least 32)
-        uint2 XE[6], GE[3];
+        BVT XE[6], GE[3];
         float me[6];
 #pragma unroll
         for (int j = 0; j < 6; ++j) {
-            XE[j] = make_uint2(0, 0);
+            XE[j] = BV::zero();
             me[j] = 1.0f;
         }
 #pragma unroll
-        for (int j = 0; j < 3; ++j) GE[j] = make_uint2(0, 0);
+        for (int j = 0; j < 3; ++j) GE[j] = BV::zero();
         if (wv == NW - 1 && te <= Lm1) {
 #pragma unroll
             for (int j = 0; j < 6; ++j) {
                 const int64_t t = te - 3 + j;
-                XE[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+                XE[j] = BV::load<false>(xb + (t < Lm1 ? t : Lm1) * xs);
             }
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
                 const int64_t t = te + j;
-                GE[j] = *(const uint2 *)(gb + (t < Lm1 ? t : Lm1) * gs);
+                GE[j] = BV::load<false>(gb + (t < Lm1 ? t : Lm1) * gs);
             }
             if constexpr (MASK) {
 #pragma unroll
@@ -581,20 +565,20 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
         // ---- all loads of the tile.  Requesting the next tile's rows while this one is worked on was measured
         // three times (before, and after, this tile's rows are waited for; with two register sets taken in turn
         // and wait counts that leave the next tile's loads in flight): 3-5 % slower, 40-60 more registers.
-        uint2 X[R], G[R], H[3];
+        BVT X[R], G[R], H[3];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t t = t0 + r < Lm1 ? t0 + r : Lm1;
-            X[r] = VecIO<8>::load<kBwdStream>(xb + t * xs);
-            G[r] = VecIO<8>::load<kBwdStream>(gb + t * gs);
+            X[r] = BV::load<kBwdStream>(xb + t * xs);
+            G[r] = BV::load<kBwdStream>(gb + t * gs);
         }
 #pragma unroll
-        for (int j = 0; j < 3; ++j) H[j] = make_uint2(0, 0);
+        for (int j = 0; j < 3; ++j) H[j] = BV::zero();
         if (wv == 0) {
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
                 const int64_t t = t0 - 3 + j;
-                if (t >= 0) H[j] = *(const uint2 *)(xb + (t < Lm1 ? t : Lm1) * xs);
+                if (t >= 0) H[j] = BV::load<false>(xb + (t < Lm1 ? t : Lm1) * xs);
             }
         }
         float mm[R + 3];   // mask of steps t0-3 .. t0+R-1
@@ -651,7 +635,7 @@ __global__ __launch_bounds__(256) void canon_bwd_blc_kernel(const BwdArgs a)
 #pragma unroll
             for (int j = 0; j < 3; ++j) {
                 tailx[pb][wv][j][lane] = X[R - 3 + j];
-                headg[pb][wv][j][lane] = j < rows ? G[j] : make_uint2(0, 0);
+                headg[pb][wv][j][lane] = j < rows ? G[j] : BV::zero();
             }
             __syncthreads();
             if (wv > 0) {

@@ -344,6 +344,32 @@ template <> struct VecIO<8> {
     }
 };
 
+template <> struct VecIO<4> {
+    using type = uint32_t;
+    static __device__ __forceinline__ type zero() { return 0u; }
+    template <bool NT> static __device__ __forceinline__ type load(const void *p)
+    {
+        const uint32_t *q = (const uint32_t *)p;
+        if constexpr (NT) return __builtin_nontemporal_load(q);
+        else return *q;
+    }
+    template <bool NT> static __device__ __forceinline__ void store(void *p, const type &v)
+    {
+        if constexpr (NT) __builtin_nontemporal_store(v, (uint32_t *)p);
+        else *(uint32_t *)p = v;
+    }
+    template <int DT> static __device__ __forceinline__ void unpack(const type &v, float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) f[0] = bits_f(v);
+        else unpack2<DT>(v, f[0], f[1]);
+    }
+    template <int DT> static __device__ __forceinline__ type pack(const float *f)
+    {
+        if constexpr (DT == CANON_DTYPE_F32) return f_bits(f[0]);
+        else return pack2<DT>(f[0], f[1]);
+    }
+};
+
 // Buffer accesses: address = resource base + vector offset + scalar offset, the sum checked against the
 // resource's size (measured on this hardware: the scalar offset counts; an access beyond the size loads zeros
 // and stores nothing).  A resource therefore spans every row its wave touches, and lanes that must not access

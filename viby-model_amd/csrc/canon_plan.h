@@ -185,6 +185,10 @@ constexpr int kBlcVecBytes = 8;   // bytes per lane and access: 8 measured 4-9 %
 #define CANON_BWD_SLAB 8
 #endif
 constexpr int kBwdSlab = CANON_BWD_SLAB;    // time steps per wave and tile
+#ifndef CANON_BWD_VEC_BYTES
+#define CANON_BWD_VEC_BYTES 8
+#endif
+constexpr int kBwdVecBytes = CANON_BWD_VEC_BYTES;   // bytes per lane and row in the channel-contiguous backward
 constexpr int kBwdWaves = 4;
 constexpr int kBwdMaxChunk = 32 * kBwdSlab * kBwdWaves;   // most time steps one block of the channel-contiguous backward walks
 enum FwdKind { FWD_BCL, FWD_BCL_SHORT, FWD_BLC, FWD_GENERIC };

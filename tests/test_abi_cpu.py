@@ -105,6 +105,14 @@ def test_fwd_plan_picks_the_vector_kernels_for_dense_layouts():
     # ragged channel counts, misaligned base pointers -> strided kernel
     assert plan(fwd_params(C=3457, layout="blc")) == "generic"
     assert plan(fwd_params(x=FAKE_X + 2)) == "generic"
+    # the channel-contiguous kernel takes the tap addresses (48 bits each), the batch stride in lane vectors (32 bits)
+    # and the number of channel tiles (16 bits) among its leading scalar arguments: beyond those, the strided kernel
+    assert plan(fwd_params(layout="blc", weight=FAKE_W | 1 << 48)) == "generic"
+    assert plan(fwd_params(layout="blc", bias=FAKE_W + 4096)) == "blc_vec"
+    assert plan(fwd_params(layout="blc", bias=1 << 50)) == "generic"
+    assert plan(fwd_params(B=1, C=65535 * 256, L=8, layout="blc")) == "blc_vec"
+    assert plan(fwd_params(B=1, C=65536 * 256, L=8, layout="blc")) == "generic"
+    assert plan(fwd_params(B=2, C=8, L=8, layout="blc", x_stride_b=4 << 32, out_stride_b=4 << 32)) == "generic"
     # the eager module's rounding points are register arithmetic: the same kernels
     assert plan(fwd_params(round_mode=1)) == "bcl_vec"
     assert plan(fwd_params(round_mode=1, layout="blc")) == "blc_vec"

@@ -183,6 +183,10 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     const bool blc_ok = ptr8_ok && a.x_sc == 1 && a.o_sc == 1 && a.C % EB == 0 &&
                         a.x_sb % EB == 0 && a.x_sl % EB == 0 && a.o_sb % EB == 0 && a.o_sl % EB == 0 &&
                         a.x_sl != 1 &&
+                        // the plain kernel receives the batch stride in lane vectors, the tile count in sixteen bits and
+                        // the tap addresses in 48 bits among its leading scalar arguments
+                        a.x_sb >= 0 && (uint64_t)(a.x_sb / EB) < (1ull << 32) && (a.C / EB + 63) / 64 < (1u << 16) &&
+                        (((uintptr_t)p->weight | (uintptr_t)p->bias) >> 48) == 0 &&
                         // rows are addressed by 32-bit scalar offsets inside a wave's buffer resource
                         a.x_sl > 0 && a.o_sl > 0 &&
                         (uint64_t)(kBlcRows + 3) * (uint64_t)a.x_sl * elem_bytes(p->x_dtype) + 64 * kBlcVecBytes < (1ull << 31) &&
@@ -245,9 +249,11 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
         const uint32_t nct = (nvec + 64 * kBlcWC - 1) / (64 * kBlcWC);          // channel tiles per row
         const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
         // `group` consecutive time tiles of a channel tile run back to back on one XCD (see blc_block_body): the
-        // fewest equal groups of at most kBlcGroup tiles
-        const uint32_t ngroups = (ntt + kBlcGroup - 1) / kBlcGroup;
-        const uint32_t group = (ntt + ngroups - 1) / ngroups;
+        // largest power of two up to kBlcGroup (the kernel divides by it with a shift) that leaves at most an
+        // eighth of the block slots of a sequence without a tile (such blocks return at once)
+        uint32_t group = kBlcGroup;
+        while (group > 1 && (uint64_t)((ntt + group - 1) / group * group - ntt) * 8 > ntt) group /= 2;
+        const uint32_t ngroups = (ntt + group - 1) / group;
         const uint64_t ncols = (uint64_t)a.B * ngroups * nct;
         const uint64_t nblocks = (ncols + 7) / 8 * 8 * group;
         if (nblocks < (1ull << 31) - 8) {

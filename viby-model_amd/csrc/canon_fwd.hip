@@ -536,9 +536,9 @@ __device__ __forceinline__ void blc_request(const BlcLead &h, const BlcWave<VB> 
 
 using ArgsHere = ArgsRead<FwdArgs>;
 // ... with the two pointers the taps are fetched through, which the plain kernel receives among its leading
-// scalars: the taps are requested BEFORE the slab, from registers, and wait neither for the slab in front of them
-// in the queue nor for a read of the argument block (a round trip of its own: with the taps requested after it, a
-// wave's taps arrived later than its slab)
+// scalars: large launches request the taps BEFORE the slab, from registers, so that they wait neither for the slab
+// in front of them in the queue nor for a read of the argument block (a round trip of its own: with the taps
+// requested after it, a wave's taps arrived later than its slab)
 struct ArgsLate : ArgsToRead<FwdArgs> {
     const void *weight, *bias;
 };
@@ -579,15 +579,15 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
         buf_load_words<PB>(rb, g * (PB * 4u) < 64u * NB * 4u ? g * (PB * 4u) : 0x80000000u, tpb);
     };
     // Where the argument block is still to be read the slab is requested ahead of it.  Small launches request the
-    // taps last: every block of the launch reads the same few lines of taps at the same moment, and a slab queued
-    // behind those loads is late (B 8, C 640 / 960: 5.4 / 6.8 us slab first, 6.2 / 7.6 us taps first).  Large
-    // launches request the taps FIRST, through two pointers read on their own ahead of the block (B 8 / 32, C 3456:
-    // 20.5 -> 20.0 / 73.6 -> 73.0 us; with a mask at B 16: 38.2 -> 38.0 us).
+    // taps last, behind the read of the argument block: every block of the launch reads the same few lines of taps
+    // at the same moment, and whatever shares the path to L2 with those loads is late (B 8, C 640 / 960: 5.0 / 6.4 us
+    // with the taps last, 5.7 / 7.6 us with the taps at once, before or after the slab).  Large launches request
+    // the taps FIRST, through the two addresses among the kernel's leading arguments (B 8 / 32, C 3456: 20.5 -> 19.9
+    // / 73.6 -> 72.9 us; with a mask at B 16: 38.2 -> 37.8 us; through two pointers read from the argument segment
+    // ahead of the block instead: 20.0 / 73.1 / 38.0 us).
     constexpr bool kTapsFirst = ARGS::kLate && BIG && kShare;
     if constexpr (ARGS::kLate) {
-        if constexpr (kTapsFirst) {
-            fetch_shared_taps(args.weight, args.bias, h.nvec);
-        }
+        if constexpr (kTapsFirst) fetch_shared_taps(args.weight, args.bias, h.nvec);
         blc_request<DT, W, R, VB>(h, wave, X, H);
     }
     const FwdArgs &a = args.get();
@@ -781,13 +781,16 @@ __device__ __forceinline__ void blc_block_linear(const FwdArgs &a, const uint32_
 // ... and the same in the plain kernel from leading scalar arguments: fourteen dwords, the most that arrive in
 // registers.  CANON_BLC_LEAD lists them once, for the kernel's signature and for the struct that mirrors the
 // kernel-argument segment (the argument block behind them is read through its offset in that struct).
-// `chunk_m`: 2^32 / chunk rounded up (0 for chunk 1), exact for the quotients of block numbers below 2^28 since
-// chunk <= 8.  `packed`: chunk | tap mode << 4 | s1 << 7 | s2 << 8 of the division by nct | s1 << 13 | s2 << 14 of
-// that by ngroups.
-#define CANON_BLC_LEAD(X)                                                                                            \
-    X(const char *, x) X(int64_t, x_sb) X(uint32_t, xs) X(uint32_t, L) X(uint32_t, nvec) X(uint32_t, ncols)         \
-    X(uint32_t, nct) X(uint32_t, nct_m) X(uint32_t, ngroups) X(uint32_t, ngroups_m) X(uint32_t, chunk_m)            \
-    X(uint32_t, packed)
+//   x_sbv    batch stride of x in lane vectors (kBlcVecBytes)
+//   packed   log2(chunk) | tap mode << 2 | s1 << 4 | s2 << 5 of the division by nct | s1 << 10 | s2 << 11 of that
+//            by ngroups | nct << 16 (the planner keeps nct below 2^16 and chunk a power of two)
+//   w_lo, b_lo, wb_hi   weight and bias addresses: low words, and the two high words' low halves (device addresses
+//            have 48 bits; checked on the host).  With them in registers the taps are requested without a read of
+//            the argument block in front of them.
+#define CANON_BLC_LEAD(X)                                                                                              \
+    X(const char *, x) X(uint32_t, x_sbv) X(uint32_t, xs) X(uint32_t, L) X(uint32_t, nvec) X(uint32_t, ncols)        \
+    X(uint32_t, nct_m) X(uint32_t, ngroups) X(uint32_t, ngroups_m) X(uint32_t, packed) X(uint32_t, w_lo)             \
+    X(uint32_t, b_lo) X(uint32_t, wb_hi)
 struct BlcSegment {
     CANON_BLC_LEAD(CANON_LEAD_FIELD)
     FwdArgs a;
@@ -797,37 +800,28 @@ static_assert(offsetof(BlcSegment, a) == 14 * 4, "fourteen leading dwords, then 
 template <int DT, int W, int R, bool MASK, bool BIG>
 __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(CANON_BLC_LEAD(CANON_LEAD_PARAM) const FwdArgs a)
 {
-    const uint32_t chunk = packed & 0xFu;
+    const uint32_t lg = packed & 3u, nct = packed >> 16;
     const uint32_t jq = blockIdx.x >> 3;
-    const uint32_t jg = chunk_m ? __umulhi(jq, chunk_m) : jq;
+    const uint32_t jg = jq >> lg;
     const uint32_t q = jg * 8u + (blockIdx.x & 7u);
     if (q >= ncols) return;   // whole block, before the barrier
-    const uint32_t qr = fdiv(q, FastDiv{nct, nct_m, (packed >> 7) & 1u, (packed >> 8) & 31u});
+    const uint32_t qr = fdiv(q, FastDiv{nct, nct_m, (packed >> 4) & 1u, (packed >> 5) & 31u});
     const uint32_t ct = q - qr * nct;
-    const uint32_t b = fdiv(qr, FastDiv{ngroups, ngroups_m, (packed >> 13) & 1u, (packed >> 14) & 31u});
-    const uint32_t tt = (qr - b * ngroups) * chunk + (jq - jg * chunk);
+    const uint32_t b = fdiv(qr, FastDiv{ngroups, ngroups_m, (packed >> 10) & 1u, (packed >> 11) & 31u});
+    const uint32_t tt = ((qr - b * ngroups) << lg) + (jq - (jg << lg));
     if ((uint64_t)tt * (kBlcWaves * R) >= L) return;   // past the last time tile
-    const BlcLead h = {x, x_sb, xs, L, nvec};
+    const BlcLead h = {x, (int64_t)x_sbv * (kBlcVecBytes / Elem<DT>::bytes), xs, L, nvec};
 #ifdef CANON_NO_LATE_ARGS
     // build switch: the argument block read the ordinary way, at the top of the kernel (for a toolchain whose
     // kernel-argument segment is not laid out like BlcSegment: costs speed, not correctness)
-    blc_block<DT, W, R, MASK, BIG>(ArgsHere{a}, h, (packed >> 4) & 3u, b, ct, tt);
+    blc_block<DT, W, R, MASK, BIG>(ArgsHere{a}, h, (packed >> 2) & 3u, b, ct, tt);
     return;
 #endif
     ArgsLate late;
     late.offset = (uint32_t)offsetof(BlcSegment, a);
-    late.weight = late.bias = nullptr;
-    if constexpr (BIG) {
-        // Large launches fetch the taps before the slab, through these two pointers, which are read on their own
-        // ahead of the argument block (nothing orders the two loads: the compiler issues them at the top of the
-        // kernel, under the tile arithmetic).
-        typedef __attribute__((address_space(4))) const char *kernarg_ptr;
-        typedef __attribute__((address_space(4))) const uintptr_t *word_ptr;
-        kernarg_ptr base = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr() + offsetof(BlcSegment, a);
-        late.weight = (const void *)*(word_ptr)(base + offsetof(FwdArgs, weight));
-        late.bias = (const void *)*(word_ptr)(base + offsetof(FwdArgs, bias));
-    }
-    blc_block<DT, W, R, MASK, BIG>(late, h, (packed >> 4) & 3u, b, ct, tt);
+    late.weight = (const void *)((uint64_t)w_lo | (uint64_t)(wb_hi & 0xFFFFu) << 32);
+    late.bias = (const void *)((uint64_t)b_lo | (uint64_t)(wb_hi >> 16) << 32);
+    blc_block<DT, W, R, MASK, BIG>(late, h, (packed >> 2) & 3u, b, ct, tt);
 }
 
 // the same over packed variable-length sequences (seq_idx)
@@ -1030,11 +1024,15 @@ template <int DT, int W, bool MASK, bool BIG> void launch_fwd_vec(const FwdPlan 
     else if (pl.kind == FWD_BCL) launch_bcl<DT, W, MASK, BIG>(pl, s);
     else {
         const FwdArgs &a = pl.args;
-        const uint32_t packed = a.chunk | (uint32_t)a.tap_mode << 4 | a.div_nct.s1 << 7 | a.div_nct.s2 << 8 | a.div_ntt.s1 << 13 | a.div_ntt.s2 << 14;
-        const uint32_t chunk_m = a.chunk > 1 ? (uint32_t)(((1ull << 32) + a.chunk - 1) / a.chunk) : 0u;
-        hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, a.x, a.x_sb,
-                           (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec, a.ntasks, a.nct, a.div_nct.m, a.nseg, a.div_ntt.m,
-                           chunk_m, packed, a);
+        uint32_t lg = 0;
+        while ((1u << lg) < a.chunk) ++lg;
+        const uint32_t packed = lg | (uint32_t)a.tap_mode << 2 | a.div_nct.s1 << 4 | a.div_nct.s2 << 5 | a.div_ntt.s1 << 10 |
+                                a.div_ntt.s2 << 11 | a.nct << 16;
+        const uint64_t wp = (uint64_t)(uintptr_t)a.weight, bp = (uint64_t)(uintptr_t)a.bias;
+        hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, a.x,
+                           (uint32_t)(a.x_sb / (kBlcVecBytes / Elem<DT>::bytes)), (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec,
+                           a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp, (uint32_t)bp,
+                           (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a);
     }
 }
 

@@ -61,14 +61,16 @@ def decode_bytes(b, c, s, esize=2, wsize=2):
 CLOCK_RAMP_S = 0.03   # untimed load before the warm-up steps: the first ~10 ms after idle run ~1 % slower (clocks ramping)
 
 
+PREFILL_ACT = 0       # activation of the prefill legs (0 none, 1 SiLU: --activation silu)
 REGIONS = 9           # back-to-back timed regions of `steps` launches each; the median region is the figure reported
 
 
-def time_region(fn, steps, warmup, ramp=True, regions=REGIONS, stats=None):
+def time_region(fn, steps, warmup, ramp=True, regions=None, stats=None):
     """ms per step: `regions` timed regions of exactly `steps` steps each, one after the other on the launch stream,
     each bracketed by events; the MEDIAN region is returned (a single region of 20 launches is 0.4 ms: one
     scheduling hiccup of the host moves it by several percent).  `stats`, a dict, receives min / max / regions."""
     import torch
+    regions = regions or REGIONS
     t_end = time.perf_counter() + (CLOCK_RAMP_S if ramp else 0.0)
     i = 0
     while time.perf_counter() < t_end and i < 1500:   # bounded both ways: launches are slow under a profiler
@@ -110,7 +112,7 @@ def graph_of(run):
 
 
 def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None, rounding=0, with_mask=False,
-                  as_graph=False, act=0, stats=None):
+                  as_graph=False, act=None, stats=None):
     """One prefill launch per step over `nbuf` rotating buffer pairs.  shape: (B, C, L), the metric's by default;
     dtype: torch.bfloat16 by default; rounding: 0 fused, 1 the eager module's rounding points; act: 1 = SiLU; with_mask: a
     right-padded padding mask of x's type and the masked residual (what CanonLayer passes); as_graph: the launches
@@ -122,6 +124,7 @@ def bench_prefill(layout, steps, warmup, nbuf, ramp=True, shape=None, dtype=None
     dev = "cuda:0"
     Bx, Cx, Lx = shape or (B, C, L)
     dtype = dtype or torch.bfloat16
+    act = PREFILL_ACT if act is None else act
     g = torch.Generator(device=dev).manual_seed(0)
     w = (torch.randn(Cx, W, generator=g, device=dev) * 0.02).to(dtype)
     bias = (torch.randn(Cx, generator=g, device=dev) * 0.01).to(dtype)
@@ -192,7 +195,7 @@ def bench_ragged(layout, steps, warmup, nbuf, batch=32):
         else:
             x = torch.randn(batch, L, C, generator=g, device=dev).bfloat16().transpose(1, 2)
         o = torch.empty_like(x)
-        p = cc._fill_fwd(x, o, w, bias, mask, None, None, 0, 1, 0)
+        p = cc._fill_fwd(x, o, w, bias, mask, None, None, PREFILL_ACT, 1, 0)
         keep.append((x, o, p))
         refs.append(ctypes.byref(p))
     fwd = _lib.lib().canon_conv1d_fwd
@@ -237,7 +240,7 @@ def bench_prefill_parts(steps, warmup, nbuf):
     for _ in range(nbuf):
         xs = [torch.randn(B, L, C // 2, generator=g, device=dev).bfloat16().transpose(1, 2) for _ in range(2)]
         outs = [torch.empty_like(x) for x in xs]
-        p = cc._fill_fwd(xs[0], outs[0], w, bias, None, None, None, 0, 1, 0)
+        p = cc._fill_fwd(xs[0], outs[0], w, bias, None, None, None, PREFILL_ACT, 1, 0)
         p.channels = C
         p.x = p.out = None
         arr = cc._part_array(xs, outs)
@@ -715,6 +718,7 @@ def cpu_baseline(budget_s=10.0):
 
 
 def main():
+    global REGIONS, PREFILL_ACT
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
@@ -723,6 +727,13 @@ def main():
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the legs that run the headline kernels on other shapes (canon_shapes, launch_floor, "
                          "host cost, eager rounding): a profile of the command then has one workload per kernel name")
+    ap.add_argument("--regions", type=int, default=REGIONS,
+                    help="timed regions of --steps launches per leg; the median is reported (profiles use 1)")
+    ap.add_argument("--activation", choices=("none", "silu"), default="none",
+                    help="silu: the prefill legs run with the optional SiLU (for a profile of that variant; the metric is "
+                         "quoted without it)")
+    ap.add_argument("--copy-ceiling", action="store_true", help="with --no-extra: run the plain-copy leg all the same")
+    ap.add_argument("--no-config5", action="store_true", help="skip the whole-model leg (configs[4])")
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="also run this many plain device-to-device copies of one x-sized buffer "
                          "(a kernel of known traffic to scale profiler byte counters by)")
@@ -733,6 +744,8 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    REGIONS = max(1, args.regions)
+    PREFILL_ACT = 1 if args.activation == "silu" else 0
 
     if args.calibration_copies:
         src = torch.empty(B * C * L, dtype=torch.bfloat16, device="cuda:0").normal_()
@@ -761,10 +774,13 @@ def main():
 
     us_dbwd, dbwd_bytes, ws_dbwd = bench_decode_backward(max(50, args.steps), max(5, args.warmup))
     ms_bwd_t, plan_bwd_t, ws_bwd_t = bench_backward(max(20, args.steps // 3), max(4, args.warmup // 3), 4, "time_contiguous")
+    ceiling = None
+    if args.no_extra and args.copy_ceiling:
+        ceiling = bench_copy_ceiling(args.steps, args.warmup)
     if not args.no_extra:
         shapes = bench_canon_shapes(max(50, args.steps // 2), max(5, args.warmup // 2))
         silu = bench_silu(max(50, args.steps // 2), max(5, args.warmup // 2))
-        config5 = bench_config5()
+        config5 = None if args.no_config5 else bench_config5()
         floor_us = bench_launch_floor(max(200, args.steps), max(20, args.warmup))
         ceiling = bench_copy_ceiling(args.steps, args.warmup)
         host_cost = bench_decode_host_cost()
@@ -779,7 +795,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: prefill bf16 x[B=8,C=3456,L=1024] time-contiguous, width 4, "
-                               "bias, residual fused, no activation", "kernel": plan,
+                               "bias, residual fused, " + ("SiLU" if PREFILL_ACT else "no activation"), "kernel": plan,
                    "storage": "bf16", "accumulate": "f32", "rotating_buffer_pairs": nbuf},
         "tokens_per_s": round(B * L / (ms * 1e-3)),
         "device_copy_same_bytes": {"ms_per_step": round(ms_copy, 6),
@@ -830,7 +846,8 @@ def main():
         out["decode"]["host_us_per_call"] = host_cost
         out["canon_shapes"] = shapes
         out["prefill_silu"] = silu
-        out["config5"] = config5
+        if config5 is not None:
+            out["config5"] = config5
         out["copy_ceiling"] = ceiling
         if ceiling:
             out["roofline"]["frac_of_plain_copy"] = round(ceiling["rows"]["B8_us"] / (ms * 1e3), 4)
@@ -840,6 +857,8 @@ def main():
             "what": "canon_conv1d_update on a [1, 8] token (one wave), back to back on the same stream: what a launch "
                     "costs before it moves any data, issued one by one from Python (host and device side together) "
                     "and as 64 nodes of a HIP graph (the device side alone)"}
+    if args.no_extra and ceiling:
+        out["copy_ceiling"] = ceiling
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -387,7 +387,8 @@ const char *canon_conv1d_fwd_plan(const canon_conv1d_fwd_params *p);
 int canon_conv1d_fwd_plan_waves(const canon_conv1d_fwd_params *p);
 const char *canon_conv1d_update_plan(const canon_conv1d_update_params *p);
 const char *canon_conv1d_bwd_plan(const canon_conv1d_bwd_params *p);   /* "bwd_blc_vec" | "bwd_bcl_vec" | "bwd_generic" */
-/* "blc_vec_parts" / "update_vec_parts" (one launch) or "per_part" (one launch per part) */
+/* "blc_vec_pair" (two dense tensors of one shape: one launch of the single-tensor code), "blc_vec_parts" /
+ * "update_vec_parts" (one launch over a table of parts) or "per_part" (one launch per part) */
 const char *canon_conv1d_fwd_parts_plan(const canon_conv1d_fwd_params *p, const canon_conv1d_part *parts, int32_t nparts);
 const char *canon_conv1d_update_parts_plan(const canon_conv1d_update_params *p, const canon_conv1d_part *parts,
                                            int32_t nparts);

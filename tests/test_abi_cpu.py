@@ -496,7 +496,8 @@ def test_parts_plan_and_validation():
 
     # Canon-B (q, k, v) and Canon-D (gate, up), separate tensors and slices of one projection output
     assert fplan(fwd_params(C=960, layout="blc"), make_parts([640, 160, 160])) == "blc_vec_parts"
-    assert fplan(fwd_params(C=3456, layout="blc"), make_parts([1728, 1728])) == "blc_vec_parts"
+    assert fplan(fwd_params(C=3456, layout="blc"), make_parts([1728, 1728])) == "blc_vec_pair"       # equal and dense
+    assert fplan(fwd_params(C=3456, layout="blc"), make_parts([1728, 1728], row=3456)) == "blc_vec_parts"   # views of one tensor
     assert fplan(fwd_params(C=960, layout="blc"), make_parts([640, 160, 160], row=960)) == "blc_vec_parts"
     assert fplan(fwd_params(C=960, layout="blc", x=None, out=None), make_parts([640, 160, 160])) == "blc_vec_parts"
     # one launch per part: time-contiguous parts, a single part, other widths, channel counts off the vector size

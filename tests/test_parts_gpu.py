@@ -48,7 +48,9 @@ def test_prefill_parts_one_launch(cc, dims, dtype):
                              initial_state=init if use_state else None, final_state_len=8 if use_state else None)
         want_out, want_state = want if use_state else (want, None)
         xs = blc_parts(x, list(dims), how)
-        assert cc.kernel_plan_fwd_parts(xs, w.to(DEV)) == "blc_vec_parts"
+        # two dense tensors of one shape take the pair launch, everything else the launch over a table of parts
+        pair = len(dims) == 2 and dims[0] == dims[1] and how == "separate"
+        assert cc.kernel_plan_fwd_parts(xs, w.to(DEV)) == ("blc_vec_pair" if pair else "blc_vec_parts")
         fs = torch.full((B, C, 8), float("nan"), dtype=dtype, device=DEV) if use_state else None
         r = cc.causal_conv1d_fn_parts(xs, w.to(DEV), b.to(DEV), activation=act, residual="masked",
                                       attention_mask=None if m is None else m.to(DEV),
@@ -81,9 +83,21 @@ def test_prefill_parts_metric_shape(cc):
     w = (torch.randn(C, 4, generator=g) * 0.02).bfloat16()
     want = co.conv1d_fwd(x, w, None, residual=1)
     xs = blc_parts(x, dims, "separate")
-    assert cc.kernel_plan_fwd_parts(xs, w.to(DEV)) == "blc_vec_parts"
+    assert cc.kernel_plan_fwd_parts(xs, w.to(DEV)) == "blc_vec_pair"
     outs = cc.causal_conv1d_fn_parts(xs, w.to(DEV), residual=True)
     assert_parity(torch.cat([o.contiguous() for o in outs], dim=1), want, exact=True, what="parts/metric")
+    # the same launch size with everything on: bias, padding mask, fp32 taps, final states (a large launch fetches its
+    # taps ahead of everything else, through the addresses among its leading arguments)
+    b = (torch.randn(C, generator=g) * 0.1).bfloat16()
+    mask = right_padded_mask([1024, 1000, 517, 3, 1024, 64, 999, 1], L)
+    for wt in (w, w.float()):
+        want, want_state = co.conv1d_fwd(x, wt, b.to(wt.dtype), mask=mask, residual=1, final_state_len=3)
+        outs, fs = cc.causal_conv1d_fn_parts(xs, wt.to(DEV), b.to(wt.dtype).to(DEV), residual="masked",
+                                             attention_mask=mask.to(DEV), return_final_states=True)
+        assert_parity(torch.cat([o.contiguous() for o in outs], dim=1), want, exact=True, what=f"parts/metric/full/{wt.dtype}")
+        assert torch.equal(bits(fs), bits(want_state)), wt.dtype
+    # views into one projection output are not dense: the launch over a table of parts
+    assert cc.kernel_plan_fwd_parts(blc_parts(x, dims, "sliced"), w.to(DEV)) == "blc_vec_parts"
 
 
 def test_prefill_parts_fall_back_to_one_launch_per_part(cc):

@@ -1185,7 +1185,8 @@ def kernel_plan_update(x, conv_state, weight, bias=None, activation=None, residu
 
 
 def kernel_plan_fwd_parts(xs, weight, bias=None, activation=None, attention_mask=None, residual=False) -> str:
-    """'blc_vec_parts' if ``causal_conv1d_fn_parts`` would run these parts as one launch, else 'per_part'."""
+    """'blc_vec_pair' (two dense tensors of one shape) or 'blc_vec_parts' if ``causal_conv1d_fn_parts`` would run
+    these parts as one launch, else 'per_part'."""
     xs = list(xs)
     outs = [torch.empty_like(x) for x in xs]
     p = _fill_fwd(xs[0], outs[0], weight, _prep_bias(weight, bias), attention_mask, None, None,

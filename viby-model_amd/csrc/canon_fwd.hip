@@ -541,7 +541,13 @@ using ArgsHere = ArgsRead<FwdArgs>;
 // requested after it, a wave's taps arrived later than its slab)
 struct ArgsLate : ArgsToRead<FwdArgs> {
     const void *weight, *bias;
+    uint32_t part;   // pair kernel: which of the two tensors the block works on (0 in the plain kernel)
 };
+// which of a pair's two parts the block works on; part 1 finds its taps, bias, output and states at fixed distances
+// from part 0's, whose argument block the launch carries
+template <typename ARGS> __device__ __forceinline__ uint32_t pair_part(const ARGS &) { return 0u; }
+__device__ __forceinline__ uint32_t pair_part(const ArgsLate &l) { return l.part; }
+__device__ __forceinline__ const void *shifted(const void *p, int64_t bytes) { return p ? (const void *)((const char *)p + bytes) : nullptr; }
 
 template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE, typename ARGS>
 __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &h, const uint32_t tb, const uint32_t ct, const uint32_t tt,
@@ -586,18 +592,23 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
     // / 73.6 -> 72.9 us; with a mask at B 16: 38.2 -> 37.8 us; through two pointers read from the argument segment
     // ahead of the block instead: 20.0 / 73.1 / 38.0 us).
     constexpr bool kTapsFirst = ARGS::kLate && BIG && kShare;
+    constexpr int64_t kWBY = Elem<WDT>::bytes;
+    const uint32_t part = pair_part(args);
     if constexpr (ARGS::kLate) {
-        if constexpr (kTapsFirst) fetch_shared_taps(args.weight, args.bias, h.nvec);
+        if constexpr (kTapsFirst)
+            fetch_shared_taps(shifted(args.weight, (int64_t)(part * h.nvec) * (E * 4 * kWBY)),
+                              shifted(args.bias, (int64_t)(part * h.nvec) * (E * kWBY)), h.nvec);
         blc_request<DT, W, R, VB>(h, wave, X, H);
     }
     const FwdArgs &a = args.get();
+    const uint32_t cshift = part ? a.pair_c : 0u;   // the block's channels in tensors that cover both parts of a pair
     const uint32_t b = wave.b, lane = wave.lane, wv = wave.wv, wt = wave.wt, wc = wave.wc, cv0 = wave.cv0, nl = wave.nl, c0 = wave.c0;
     const uint32_t voff = wave.voff, xs = wave.xs;
     const int64_t t0 = wave.t0;
     const int rows = wave.rows;
     const bool active = wave.active;
     const uint32_t os = (uint32_t)(a.o_sl * BY);
-    char *ow = a.out + ((int64_t)b * a.o_sb + (int64_t)cv0 * E) * BY + t0 * (int64_t)os;
+    char *ow = a.out + (part ? a.pair_out_shift : 0) + ((int64_t)b * a.o_sb + (int64_t)cv0 * E) * BY + t0 * (int64_t)os;
     // (rows past the end of the sequence are not stored; lanes without channels are out of range)
     const uint32_t orec = rows == 0 ? 0u : (uint32_t)(R - 1) * os + nl * VB;
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void *)ow, 0, (int)orec, kBufFlags);
@@ -608,7 +619,8 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
     TapWords<WDT, E> tw;
     const uint32_t g = wt * 64u + lane;                         // thread within the tile's group of waves
     if constexpr (kShare) {
-        if constexpr (!kTapsFirst) fetch_shared_taps(a.weight, a.bias, a.nvec);
+        if constexpr (!kTapsFirst)
+            fetch_shared_taps(shifted(a.weight, (int64_t)cshift * (4 * kWBY)), shifted(a.bias, (int64_t)cshift * kWBY), a.nvec);
     } else if constexpr (MODE != TAPS_ANY) {
         fetch_taps_contiguous<WDT, E>(a.weight, a.bias, c0, tw);
     }
@@ -681,7 +693,7 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
             if (j < 3 - (W - 1)) continue;
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
+                hist[j][e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(cshift + c0 + e) * a.i_sc + (int64_t)(a.S_in - 3 + j) * a.i_ss);
         }
     }
     float w[E][W], bias[E];
@@ -703,7 +715,7 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
     }
 
     if (a.fin && active && t0 + rows == (int64_t)a.L) {
-        const char *xb = a.x + ((int64_t)b * a.x_sb + c0) * BY;
+        const char *xb = h.x + ((int64_t)b * h.x_sb + c0) * BY;
         for (int slot = 0; slot < a.S_out; ++slot) {
             const int64_t t = (int64_t)a.L - a.S_out + slot;
             float v[E];
@@ -719,11 +731,11 @@ __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &
             } else if (a.init && a.S_in + t >= 0) {
 #pragma unroll
                 for (int e = 0; e < E; ++e)
-                    v[e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
+                    v[e] = load1<DT>(a.init, b * a.i_sb + (int64_t)(cshift + c0 + e) * a.i_sc + (a.S_in + t) * a.i_ss);
             }
 #pragma unroll
             for (int e = 0; e < E; ++e)
-                store1<DT>(a.fin, b * a.f_sb + (int64_t)(c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
+                store1<DT>(a.fin, b * a.f_sb + (int64_t)(cshift + c0 + e) * a.f_sc + slot * a.f_ss, v[e]);
         }
     }
 }
@@ -821,8 +833,50 @@ __global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_kernel(CANON_BLC_LE
     late.offset = (uint32_t)offsetof(BlcSegment, a);
     late.weight = (const void *)((uint64_t)w_lo | (uint64_t)(wb_hi & 0xFFFFu) << 32);
     late.bias = (const void *)((uint64_t)b_lo | (uint64_t)(wb_hi >> 16) << 32);
+    late.part = 0u;
     blc_block<DT, W, R, MASK, BIG>(late, h, (packed >> 2) & 3u, b, ct, tt);
 }
+
+// Two tensors of the same shape, each dense ([B, L, C] with nothing between rows or sequences), in ONE launch of the
+// plain kernel's code: Canon-D's gate and up where they are.  The columns of part 1 follow those of part 0; a block
+// picks its tensor from two leading pointers, and the row and batch strides, which the plain kernel receives,
+// follow from nvec and L.  `a` is part 0's argument block; part 1's taps, bias, output and states lie at the
+// distances a.pair_c / a.pair_out_shift from part 0's (see blc_block_body).  Only for taps the straight-line
+// modes cover (the planner sees to that), and not in a build with -DCANON_NO_LATE_ARGS, which plans no such launch.
+#ifndef CANON_NO_LATE_ARGS
+#define CANON_BLC_PAIR_LEAD(X)                                                                                         \
+    X(const char *, x0) X(const char *, x1) X(uint32_t, L) X(uint32_t, nvec) X(uint32_t, ncols) X(uint32_t, nct_m)     \
+    X(uint32_t, ngroups) X(uint32_t, ngroups_m) X(uint32_t, packed) X(uint32_t, w_lo) X(uint32_t, b_lo) X(uint32_t, wb_hi)
+struct BlcPairSegment {
+    CANON_BLC_PAIR_LEAD(CANON_LEAD_FIELD)
+    FwdArgs a;
+};
+static_assert(offsetof(BlcPairSegment, a) == 14 * 4, "fourteen leading dwords, then the argument block");
+
+template <int DT, int W, int R, bool MASK, bool BIG>
+__global__ __launch_bounds__(kBlcThreads) void canon_fwd_blc_pair_kernel(CANON_BLC_PAIR_LEAD(CANON_LEAD_PARAM) const FwdArgs a)
+{
+    const uint32_t lg = packed & 3u, nct = packed >> 16;
+    const uint32_t jq = blockIdx.x >> 3;
+    const uint32_t jg = jq >> lg;
+    uint32_t q = jg * 8u + (blockIdx.x & 7u);
+    if (q >= 2u * ncols) return;   // whole block, before the barrier
+    const uint32_t part = q >= ncols ? 1u : 0u;
+    q -= part * ncols;
+    const uint32_t qr = fdiv(q, FastDiv{nct, nct_m, (packed >> 4) & 1u, (packed >> 5) & 31u});
+    const uint32_t ct = q - qr * nct;
+    const uint32_t b = fdiv(qr, FastDiv{ngroups, ngroups_m, (packed >> 10) & 1u, (packed >> 11) & 31u});
+    const uint32_t tt = ((qr - b * ngroups) << lg) + (jq - (jg << lg));
+    if ((uint64_t)tt * (kBlcWaves * R) >= L) return;   // past the last time tile
+    const BlcLead h = {part ? x1 : x0, (int64_t)L * nvec * (kBlcVecBytes / Elem<DT>::bytes), nvec * (uint32_t)kBlcVecBytes, L, nvec};
+    ArgsLate late;
+    late.offset = (uint32_t)offsetof(BlcPairSegment, a);
+    late.weight = (const void *)((uint64_t)w_lo | (uint64_t)(wb_hi & 0xFFFFu) << 32);
+    late.bias = (const void *)((uint64_t)b_lo | (uint64_t)(wb_hi >> 16) << 32);
+    late.part = part;
+    blc_block<DT, W, R, MASK, BIG>(late, h, (packed >> 2) & 3u, b, ct, tt);
+}
+#endif  // CANON_NO_LATE_ARGS
 
 // the same over packed variable-length sequences (seq_idx)
 template <int DT, int W, int R, bool MASK>
@@ -1077,8 +1131,38 @@ void launch_blc_parts(const PartTable<FwdArgs> &m, uint32_t grid, hipStream_t s)
                        m.first_block[1], m.first_block[2], m.first_block[3], m);
 }
 
+#ifndef CANON_NO_LATE_ARGS
+template <int DT, bool MASK, bool BIG> void launch_blc_pair(const FwdPartsPlan &pp, hipStream_t s)
+{
+    FwdArgs a = pp.part[0].args;
+    a.pair_out_shift = (int64_t)((intptr_t)pp.part[1].args.out - (intptr_t)pp.part[0].args.out);
+    a.pair_c = a.C;
+    uint32_t lg = 0;
+    while ((1u << lg) < a.chunk) ++lg;
+    const uint32_t packed = lg | (uint32_t)a.tap_mode << 2 | a.div_nct.s1 << 4 | a.div_nct.s2 << 5 | a.div_ntt.s1 << 10 |
+                            a.div_ntt.s2 << 11 | a.nct << 16;
+    const uint64_t wp = (uint64_t)(uintptr_t)a.weight, bp = (uint64_t)(uintptr_t)a.bias;
+    hipLaunchKernelGGL((canon_fwd_blc_pair_kernel<DT, 4, kBlcRows, MASK, BIG>), dim3(pp.grid), dim3(kBlcThreads), 0, s, a.x,
+                       pp.part[1].args.x, a.L, a.nvec, a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp,
+                       (uint32_t)bp, (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a);
+}
+#endif
+
 template <int DT> void launch_fwd_parts_t(const FwdPartsPlan &pp, hipStream_t s)
 {
+#ifndef CANON_NO_LATE_ARGS
+    if (pp.pair) {
+        const bool mask = pp.part[0].args.mask != nullptr, nt = pp.part[0].args.nt != 0;
+        if (mask) {
+            if (nt) launch_blc_pair<DT, true, true>(pp, s);
+            else launch_blc_pair<DT, true, false>(pp, s);
+        } else {
+            if (nt) launch_blc_pair<DT, false, true>(pp, s);
+            else launch_blc_pair<DT, false, false>(pp, s);
+        }
+        return;
+    }
+#endif
     if (!pp.single) {
         for (int i = 0; i < pp.n; ++i)
             if (pp.part[i].grid > 0) launch_fwd<DT>(pp.part[i], s);

@@ -64,6 +64,9 @@ struct FwdArgs {
     // blc: tiles
     uint32_t nct, ntt;  // channel tiles per row, time tiles per sequence
     FastDiv div_nct, div_ntt;   // div_ntt divides by the groups per sequence
+    // two equal dense parts in one launch (canon_fwd_blc_pair_kernel): this is part 0's block, and what part 1 adds
+    int64_t pair_out_shift;     // bytes from part 0's out to part 1's
+    uint32_t pair_c;            // channels of a part: part 1's first channel in taps, bias, initial and final state
 };
 
 struct UpdArgs {
@@ -234,6 +237,7 @@ struct UpdPlan {
 struct FwdPartsPlan {
     int n;
     bool single;            // one launch over a PartTable
+    bool pair;              // ... or, two equal dense parts, one launch of the pair kernel on part[0]'s block
     uint32_t grid;          // of that launch
     FwdPlan part[kMaxParts];
 };

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define CANON_CONV1D_ABI_VERSION 8
+#define CANON_CONV1D_ABI_VERSION 9
 #define CANON_CONV1D_MIN_WIDTH 2
 #define CANON_CONV1D_MAX_WIDTH 4
 
@@ -242,7 +242,7 @@ typedef struct canon_conv1d_bwd_params {
 } canon_conv1d_bwd_params;
 
 /*
- * Backward of canon_conv1d_update (shift-register mode).  Same role as the
+ * Backward of canon_conv1d_update.  Same role as the
  * reference's short_conv_update_bwd (causal_conv1d_mps/autograd.py:465-498,
  * causal_conv1d.metal:1738-1850): dx, dconv_state, dweight, dbias from the
  * token, the state AS IT WAS BEFORE the forward call (the caller keeps a
@@ -294,6 +294,19 @@ typedef struct canon_conv1d_update_bwd_params {
     float *dbias;                   /* [channels] fp32, or NULL; needs dweight */
     void *workspace;                /* canon_conv1d_update_bwd_workspace_bytes() bytes, 16-byte aligned (unused when dweight == NULL) */
     int64_t workspace_bytes;
+    /* The decode modes of canon_conv1d_update other than the shift register (both NULL: shift register).
+     * cache_seqlens: the forward wrote the token to slot p = cache_seqlens[b] mod state_len and read the width-1
+     *   slots before it cyclically (the reference's update kernel, causal_conv1d.metal:755-775, and its backward,
+     *   :1738-1850); the formulas above hold with entry j of the state before the step in slot (p + j) mod state_len
+     *   and entry j of the updated state in slot (p + 1 + j) mod state_len.
+     * conv_state_indices: batch entry b used row conv_state_indices[b] of conv_state, so conv_state, dstate_out and
+     *   dstate have state_rows rows.  An entry whose index lies outside the pool was skipped by the forward: its dx
+     *   row is zero and it contributes nothing.  Only the rows that entries name are written: fill dstate with
+     *   dstate_out (or zeros) before the call, so that rows no entry used pass their gradient on unchanged.  Two
+     *   entries naming one row are as undefined here as in the forward. */
+    const int32_t *cache_seqlens;        /* [batch] int32, or NULL */
+    const int32_t *conv_state_indices;   /* [batch] int32, or NULL */
+    int64_t state_rows;                  /* rows of the pool; 0: not stated (indices are only checked for a negative value) */
 } canon_conv1d_update_bwd_params;
 
 /*

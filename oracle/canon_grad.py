@@ -117,3 +117,65 @@ def update_grads(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor
     loss.backward()
     return (x64.grad, s64.grad if s64.grad is not None else torch.zeros_like(s64), w64.grad,
             b64.grad if b64 is not None else None, y.detach(), new_state.detach())
+
+
+def update_grads_ext(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                     dout: torch.Tensor, dstate_out: Optional[torch.Tensor] = None, token_mask: Optional[torch.Tensor] = None,
+                     activation=None, residual=0, cache_seqlens: Optional[torch.Tensor] = None,
+                     conv_state_indices: Optional[torch.Tensor] = None):
+    """Gradients of the decode step in upstream's other two state modes, by torch autograd (float64) through the
+    step written with gather / scatter:
+
+    cache_seqlens [B]       ring buffer (the reference's update kernel, causal_conv1d.metal:755-775): the token goes
+                            to slot p = cache_seqlens % S, tap k < W-1 reads slot (p - (W-1) + k) mod S, the other
+                            slots stay.
+    conv_state_indices [B]  state pool: entry b uses row conv_state_indices[b] of conv_state [R, C, S]; an index
+                            outside [0, R) skips the entry (its output row is zero, no state row changes).
+
+    x, dout [B, C]; conv_state, dstate_out [R, C, S] (R = B without a pool).  Returns
+    (dx, dstate, dweight, dbias, out, new_state) in float64, dstate and new_state with conv_state's shape."""
+    C, W = weight.shape
+    B = x.shape[0]
+    R, _, S = conv_state.shape
+    x64 = x.detach().cpu().double().requires_grad_(True)
+    s64 = conv_state.detach().cpu().double().requires_grad_(True)
+    w64 = weight.detach().cpu().to(x.dtype).double().requires_grad_(True)
+    b64 = bias.detach().cpu().to(x.dtype).double().requires_grad_(True) if bias is not None else None
+    xt = x64 if token_mask is None else x64 * token_mask.detach().cpu().double().unsqueeze(1)
+    if conv_state_indices is not None:
+        idx = conv_state_indices.detach().cpu().long()
+        live = (idx >= 0) & (idx < R)
+    else:
+        idx = torch.arange(B)
+        live = torch.ones(B, dtype=torch.bool)
+    rows = s64[idx.clamp(0, R - 1)]                                    # [B, C, S]
+    if cache_seqlens is not None:
+        p = torch.remainder(cache_seqlens.detach().cpu().long(), S)    # non-negative
+        hist_slots = torch.remainder(p[:, None] - (W - 1) + torch.arange(W - 1)[None, :], S)      # [B, W-1]
+        write_slot = p
+    else:
+        hist_slots = (S - (W - 1) + torch.arange(W - 1))[None, :].expand(B, W - 1)
+        write_slot = None
+    hist = rows.gather(2, hist_slots[:, None, :].expand(B, C, W - 1))
+    window = torch.cat([hist, xt.unsqueeze(-1)], dim=-1)               # [B, C, W]
+    z = (window * w64.unsqueeze(0)).sum(-1)
+    if b64 is not None:
+        z = z + b64
+    y = F.silu(z) if activation in ("silu", "swish", True, 1) else z
+    if residual in (True, 1, "masked"):
+        y = y + xt
+    elif residual in (2, "unmasked"):
+        y = y + x64
+    y = y * live[:, None].double()                                      # a skipped entry's output is a constant zero
+    if write_slot is not None:
+        new_rows = rows.scatter(2, write_slot[:, None, None].expand(B, C, 1), xt.unsqueeze(-1))
+    else:
+        new_rows = torch.cat([rows[:, :, 1:], xt.unsqueeze(-1)], dim=-1)
+    new_state = s64.clone()
+    new_state[idx[live]] = new_rows[live]
+    loss = (y * dout.detach().cpu().double()).sum()
+    if dstate_out is not None:
+        loss = loss + (new_state * dstate_out.detach().cpu().double()).sum()
+    loss.backward()
+    return (x64.grad, s64.grad if s64.grad is not None else torch.zeros_like(s64), w64.grad,
+            b64.grad if b64 is not None else None, y.detach(), new_state.detach())

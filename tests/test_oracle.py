@@ -522,6 +522,61 @@ def test_update_gradient_oracle_chained_equals_the_prefill_gradient_oracle():
             assert torch.allclose(got, want, atol=1e-11), (S, W, act, res, masked)
 
 
+def test_update_gradient_oracle_of_ring_and_pool_modes_equals_the_shift_register_form():
+    """oracle/canon_grad.update_grads_ext (the step written with gather / scatter) is pinned by what defines its
+    two modes.  Ring: with the state rotated so that slot (p + j) mod S holds entry j of a shift register, and the
+    gradient of the updated state rotated by p + 1, its gradients are those of update_grads, rotated back.  Pool:
+    entries that name rows of a pool give update_grads of those rows; rows nobody names hand their gradient on;
+    an index outside the pool contributes nothing.  Both together; and neither equals update_grads itself."""
+    from oracle.canon_grad import update_grads, update_grads_ext
+    torch.manual_seed(3)
+    for (S, W), act, res, masked, through in itertools.product([(4, 4), (3, 4), (8, 4), (5, 3), (1, 2)], [None, "silu"],
+                                                               [0, 1, 2], [False, True], [False, True]):
+        B, C = 4, 5
+        x, st = torch.randn(B, C).double(), torch.randn(B, C, S).double()
+        w, b, dout = torch.randn(C, W).double(), torch.randn(C).double(), torch.randn(B, C).double()
+        dso = torch.randn(B, C, S).double() if through else None
+        mask = torch.tensor([1.0, 0.0, 1.0, 1.0]).double() if masked else None
+        plain = update_grads(x, st, w, b, dout, dso, mask, act, res)
+        same = update_grads_ext(x, st, w, b, dout, dso, mask, act, res)
+        for u, v in zip(plain, same):
+            assert torch.allclose(u, v, atol=1e-13)
+        # ring buffer
+        seqlens = torch.tensor([0, 1, S + 2, 7 * S + (S - 1)], dtype=torch.int32)
+        p = seqlens.long() % S
+        j = torch.arange(S)
+        to_slot = (p[:, None] + j[None, :]) % S                  # slot of entry j before the step
+        to_slot_after = (p[:, None] + 1 + j[None, :]) % S        # slot of entry j after it
+        def rotate(t, slots):                                   # ring[slot] = register[entry]
+            r = torch.empty_like(t)
+            r.scatter_(2, slots[:, None, :].expand_as(t), t)
+            return r
+        ring = update_grads_ext(x, rotate(st, to_slot), w, b, dout, None if dso is None else rotate(dso, to_slot_after),
+                                mask, act, res, cache_seqlens=seqlens)
+        assert torch.allclose(ring[0], plain[0], atol=1e-13) and torch.allclose(ring[2], plain[2], atol=1e-13)
+        assert torch.allclose(ring[3], plain[3], atol=1e-13) and torch.allclose(ring[4], plain[4], atol=1e-13)
+        assert torch.allclose(ring[1], rotate(plain[1], to_slot), atol=1e-13), (S, W)
+        assert torch.allclose(ring[5], rotate(plain[5], to_slot_after), atol=1e-13), (S, W)
+        # state pool of 7 rows: entries 0, 1, 3 name rows 5, 0, 2; entry 2 is skipped
+        idx = torch.tensor([5, 0, -3, 2], dtype=torch.int32)
+        live = torch.tensor([0, 1, 3])
+        pool = torch.randn(7, C, S).double()
+        pool[idx[live].long()] = st[live]
+        dpool = torch.randn(7, C, S).double() if through else None
+        if through:
+            dpool[idx[live].long()] = dso[live]
+        got = update_grads_ext(x, pool, w, b, dout, dpool, mask, act, res, conv_state_indices=idx)
+        sub = update_grads(x[live], st[live], w, b, dout[live], None if dso is None else dso[live],
+                           None if mask is None else mask[live], act, res)
+        assert torch.allclose(got[0][live], sub[0], atol=1e-13) and not got[0][2].any() and not got[4][2].any()
+        assert torch.allclose(got[2], sub[2], atol=1e-13) and torch.allclose(got[3], sub[3], atol=1e-13)
+        assert torch.allclose(got[1][idx[live].long()], sub[1], atol=1e-13)
+        for r in (1, 3, 4, 6):
+            assert torch.equal(got[1][r], dpool[r] if through else torch.zeros(C, S).double())
+            assert torch.equal(got[5][r], pool[r])
+        assert torch.allclose(got[5][idx[live].long()], sub[5], atol=1e-13)
+
+
 def test_gradient_oracle_with_initial_states_equals_the_block_in_one_go():
     """conv1d_grads(initial_states=...) on the second half of a block, continued from the (masked) last inputs
     of the first half, plus conv1d_grads on the first half, must add up to conv1d_grads on the whole block."""

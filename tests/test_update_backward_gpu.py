@@ -6,7 +6,7 @@ import itertools
 import pytest
 import torch
 
-from oracle.canon_grad import conv1d_grads, update_grads
+from oracle.canon_grad import conv1d_grads, update_grads, update_grads_ext
 from test_backward_gpu import check
 
 pytestmark = pytest.mark.gpu
@@ -64,6 +64,97 @@ def test_update_backward_matches_autograd_of_the_eager_step(cc, dtype, S, W):
             check(got[3], want[3], dtype, "dbias " + tag, sum_terms=B)
         # the state handed on is bit-exactly the shifted state with the (masked) token appended
         assert torch.equal(got[5].cpu().double(), want[5]), "state " + tag
+
+
+def run_step_ext(cc, x, state, w, b, dout, dstate_out, mask, act, residual, seqlens, indices):
+    """run_step in the ring-buffer / state-pool modes (state: the whole pool when indices are given)."""
+    xg = x.to(DEV).requires_grad_(True)
+    s0 = state.to(DEV).requires_grad_(True)
+    wg = w.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True) if b is not None else None
+    s = s0.clone()
+    out = cc.causal_conv1d_update(xg, s, wg, bg, activation=act, residual=residual,
+                                  token_mask=None if mask is None else mask.to(DEV),
+                                  cache_seqlens=None if seqlens is None else seqlens.to(DEV),
+                                  conv_state_indices=None if indices is None else indices.to(DEV))
+    loss = (out.float() * dout.to(DEV).float()).sum()
+    if dstate_out is not None:
+        loss = loss + (s.float() * dstate_out.to(DEV).float()).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    return xg.grad, s0.grad, wg.grad, (bg.grad if bg is not None else None), out.detach(), s.detach()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("S,W", [(3, 4), (4, 4), (8, 4), (2, 3), (5, 2)])
+def test_update_backward_in_ring_buffer_and_state_pool_modes(cc, dtype, S, W):
+    """The decode modes of upstream's signature: cache_seqlens (the mode the reference's own update autograd
+    differentiates, causal_conv1d_mps/autograd.py:341-498) and conv_state_indices, alone and together, against
+    torch autograd through the step written with gather / scatter."""
+    torch.manual_seed(S * 10 + W + 100)
+    B, C, R = 6, 72, 9
+    seqlens = torch.tensor([0, 1, 5, 7, 2 * S + 1, 123], dtype=torch.int32)
+    # a pool of nine rows: entries use rows 4, 0, 8, 2, a negative index and one past the pool skip their entries,
+    # rows 1, 3, 5, 6, 7 are nobody's
+    indices = torch.tensor([4, 0, -1, 8, 9, 2], dtype=torch.int32)
+    for (ring, pool), act, residual, use_mask, through_state in itertools.product(
+            [(True, False), (False, True), (True, True)], [None, "silu"], [False, True, "unmasked"], [False, True],
+            [False, True]):
+        if act is None and use_mask != (residual is not False):
+            continue
+        rows = R if pool else B
+        x, st = quantised((B, C), dtype), quantised((rows, C, S), dtype)
+        w, b = quantised((C, W), dtype, 0.5), quantised((C,), dtype, 0.1)
+        dout = quantised((B, C), dtype)
+        dso = quantised((rows, C, S), dtype) if through_state else None
+        mask = torch.tensor([1, 0, 1, 1, 0, 1], dtype=torch.int64) if use_mask else None
+        sl, ix = (seqlens if ring else None), (indices if pool else None)
+        got = run_step_ext(cc, x, st, w, b, dout, dso, mask, act, residual, sl, ix)
+        want = update_grads_ext(x, st, w, b, dout, dso, mask, act, residual, sl, ix)
+        tag = f"{dtype} S{S} W{W} ring={ring} pool={pool} act={act} res={residual} mask={use_mask} state={through_state}"
+        check(got[0], want[0], dtype, "dx " + tag)
+        check(got[1], want[1], dtype, "dstate " + tag)
+        live = B - 2 if pool else B
+        check(got[2], want[2], dtype, "dweight " + tag, sum_terms=live)
+        check(got[3], want[3], dtype, "dbias " + tag, sum_terms=live)
+        assert torch.equal(got[5].cpu().double(), want[5]), "state " + tag
+        if pool:
+            # a skipped entry has a zero output row and a zero dx row; rows of the pool that no entry names hand
+            # the gradient of the updated pool through untouched (zero when the loss does not read the pool)
+            for e in (2, 4):
+                assert not got[4][e].any() and not got[0][e].any(), tag
+            for r in (1, 3, 5, 6, 7):
+                passed = dso[r].to(DEV) if through_state else torch.zeros(C, S, dtype=dtype, device=DEV)
+                assert torch.equal(got[1][r], passed), tag
+
+
+def test_chain_of_ring_buffer_steps_has_the_gradients_of_the_shift_register_chain(cc):
+    """T tokens through an 8-slot ring (cache_seqlens = 0, 1, 2, ...) and through the shift register, same start
+    (the ring's slot j is the register's entry j at step 0): equal outputs, and bit-equal gradients of the tokens
+    and parameters (the same products in the same order; only the slot arithmetic differs)."""
+    torch.manual_seed(7)
+    B, C, S, T = 3, 40, 8, 11
+    w0, b0 = quantised((C, 4), torch.bfloat16, 0.5), quantised((C,), torch.bfloat16, 0.1)
+    xs0 = quantised((T, B, C), torch.bfloat16)
+    st0 = quantised((B, C, S), torch.bfloat16)
+    results = []
+    for ring in (False, True):
+        w = w0.to(DEV).requires_grad_(True)
+        b = b0.to(DEV).requires_grad_(True)
+        xs = xs0.to(DEV).requires_grad_(True)
+        s_leaf = st0.to(DEV).requires_grad_(True)
+        s = s_leaf.clone()
+        outs = []
+        for t in range(T):
+            sl = torch.full((B,), t, dtype=torch.int32, device=DEV) if ring else None
+            outs.append(cc.causal_conv1d_update(xs[t], s, w, b, activation="silu", residual=True, cache_seqlens=sl))
+        loss = sum((o.float() * (i + 1)).sum() for i, o in enumerate(outs)) + (s.float() ** 2).sum()
+        loss.backward()
+        results.append((torch.stack(outs).detach(), xs.grad, w.grad, b.grad, s_leaf.grad))
+    (o0, dx0, dw0, db0, ds0), (o1, dx1, dw1, db1, ds1) = results
+    assert torch.equal(o0, o1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1) and torch.equal(db0, db1)
+    # the ring starts at slot 0 = the register's oldest entry, so the initial states coincide slot by slot
+    assert torch.equal(ds0, ds1)
 
 
 def test_update_backward_finite_differences_like_the_reference_test(cc):
@@ -175,10 +266,7 @@ def test_update_backward_at_decode_shape_is_deterministic(cc):
 def test_update_backward_argument_handling(cc):
     x = torch.randn(2, 8, device=DEV, requires_grad=True)
     w = torch.randn(8, 4, device=DEV)
-    with pytest.raises(NotImplementedError, match="shift-register mode"):
-        cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV), w,
-                                cache_seqlens=torch.zeros(2, dtype=torch.int32, device=DEV))
-    with pytest.raises(NotImplementedError, match="shift-register mode"):
+    with pytest.raises(NotImplementedError, match="rounding='fused'"):
         cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV), w, rounding="eager")
     # a state that is a leaf requiring grad cannot be updated in place: torch says so itself
     with pytest.raises(RuntimeError, match="leaf"):

@@ -564,12 +564,10 @@ def causal_conv1d_update(
     if conv_state.shape[2] < weight.shape[1] - 1:
         raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
     wants_grad = _wants_grad(x, weight, bias, conv_state)
-    if wants_grad and (cache_seqlens is not None or conv_state_indices is not None or rnd != 0
-                       or torch.compiler.is_compiling()):
+    if wants_grad and (rnd != 0 or torch.compiler.is_compiling()):
         raise NotImplementedError(
-            "causal_conv1d_update (gfx950): the backward of the decode step covers the shift-register mode with "
-            "rounding='fused' outside torch.compile (no cache_seqlens / conv_state_indices); call under "
-            "torch.no_grad() or detach the inputs")
+            "causal_conv1d_update (gfx950): the backward of the decode step covers rounding='fused' outside "
+            "torch.compile; call under torch.no_grad() or detach the inputs")
     bias = _prep_bias(weight, bias)
     if token_mask is not None:
         if token_mask.dim() != 1 or token_mask.shape[0] != batch:
@@ -578,7 +576,7 @@ def causal_conv1d_update(
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
 
     if wants_grad:
-        out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res)
+        out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens, conv_state_indices)
     elif torch.compiler.is_compiling():
         out = torch.ops.canon_conv1d.update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices,
                                             act, res, rnd)
@@ -675,36 +673,40 @@ class _CanonUpdateFn(torch.autograd.Function):
     state as it was is kept for the backward (as ShortConvUpdateMPSFunction does,
     causal_conv1d_mps/autograd.py:452-453); ``conv_state`` is declared modified in place and
     returned, so a gradient that arrives through the updated state (the next decode step reading
-    it) flows back into this step's token and into the state before it."""
+    it) flows back into this step's token and into the state before it.  The ring-buffer mode
+    (``cache_seqlens``, the mode of the reference's own update autograd, causal_conv1d_mps/autograd.py:341-498) and
+    the state-pool mode (``conv_state_indices``) differentiate the same way; in pool mode ``conv_state`` is the
+    whole pool, and rows that no batch entry names pass their gradient through unchanged."""
 
     @staticmethod
-    def forward(ctx, x2, conv_state, weight, bias, token_mask, act, res):
+    def forward(ctx, x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens=None, conv_state_indices=None):
         before = conv_state.detach().clone()
-        out = _launch_update(x2, conv_state, weight, bias, token_mask, None, None, act, res, 0)
+        out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, 0)
         ctx.mark_dirty(conv_state)
         ctx.set_materialize_grads(False)
-        ctx.save_for_backward(x2, before, weight, bias, token_mask)
+        ctx.save_for_backward(x2, before, weight, bias, token_mask, cache_seqlens, conv_state_indices)
         ctx.flags = (act, res)
         return out, conv_state
 
     @staticmethod
     def backward(ctx, dout, dstate_out):
-        x2, before, weight, bias, token_mask = ctx.saved_tensors
+        x2, before, weight, bias, token_mask, cache_seqlens, conv_state_indices = ctx.saved_tensors
         act, res = ctx.flags
         if dout is None:
             dout = torch.zeros_like(x2)
         want_state = ctx.needs_input_grad[1]
         want_params = ctx.needs_input_grad[2] or (bias is not None and ctx.needs_input_grad[3])
         dx, dstate, dweight, dbias = _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res,
-                                                        want_state, want_params)
+                                                        want_state, want_params, cache_seqlens, conv_state_indices)
         return (dx, dstate, dweight.to(weight.dtype) if dweight is not None else None,
-                dbias.to(bias.dtype) if dbias is not None else None, None, None, None)
+                dbias.to(bias.dtype) if dbias is not None else None, None, None, None, None, None)
 
 
 def _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res, want_state=True,
-                       want_params=True):
+                       want_params=True, cache_seqlens=None, conv_state_indices=None):
     """One launch (+ the fixed-order reduction over the batch): (dx, dstate | None, dweight | None, dbias | None),
-    the parameter gradients in fp32."""
+    the parameter gradients in fp32.  With ``conv_state_indices`` the state tensors are pools: the kernel writes the
+    rows the batch entries name, the others carry ``dstate_out`` through."""
     if dout.dtype != x2.dtype:
         dout = dout.to(x2.dtype)
     if dstate_out is not None and dstate_out.dtype != x2.dtype:
@@ -713,7 +715,14 @@ def _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, a
     width = weight.shape[1]
     dev = x2.device
     dx = torch.empty(batch, channels, dtype=x2.dtype, device=dev)
-    dstate = torch.empty(tuple(before.shape), dtype=x2.dtype, device=dev) if want_state else None
+    if not want_state:
+        dstate = None
+    elif conv_state_indices is None:
+        dstate = torch.empty(tuple(before.shape), dtype=x2.dtype, device=dev)
+    elif dstate_out is not None:
+        dstate = dstate_out.clone(memory_format=torch.contiguous_format)
+    else:
+        dstate = torch.zeros(tuple(before.shape), dtype=x2.dtype, device=dev)
     dweight = torch.empty(channels, width, dtype=torch.float32, device=dev) if want_params else None
     dbias = torch.empty(channels, dtype=torch.float32, device=dev) if want_params and bias is not None else None
     p = _lib.UpdateBwdParams()
@@ -747,6 +756,11 @@ def _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, a
         p.dstate_stride_b, p.dstate_stride_c, p.dstate_stride_s = dstate.stride()
     p.dweight = dweight.data_ptr() if dweight is not None else None
     p.dbias = dbias.data_ptr() if dbias is not None else None
+    if cache_seqlens is not None:
+        p.cache_seqlens = cache_seqlens.data_ptr()
+    if conv_state_indices is not None:
+        p.conv_state_indices = conv_state_indices.data_ptr()
+        p.state_rows = before.shape[0]
     L = _lib.lib()
     nbytes = L.canon_conv1d_update_bwd_workspace_bytes(ctypes.byref(p))
     if nbytes < 0:

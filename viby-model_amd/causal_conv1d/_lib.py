@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcanon_conv1d.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MASK_CODE = {
@@ -102,6 +102,7 @@ class UpdateBwdParams(ctypes.Structure):
         ("dstate", _vp), ("dstate_stride_b", _i64), ("dstate_stride_c", _i64), ("dstate_stride_s", _i64),
         ("dweight", _vp), ("dbias", _vp),
         ("workspace", _vp), ("workspace_bytes", _i64),
+        ("cache_seqlens", _vp), ("conv_state_indices", _vp), ("state_rows", _i64),
     ]
 
 

@@ -732,6 +732,10 @@ int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, b
     if (p->token_mask && !valid_mask_dtype(p->mask_dtype))
         return fail(CANON_ERR_INVALID_ARGUMENT, "unknown mask_dtype %d", p->mask_dtype);
     if (p->dbias && !p->dweight) return fail(CANON_ERR_INVALID_ARGUMENT, "dbias needs dweight");
+    if (p->state_rows < 0 || p->state_rows >= (1ll << 31))
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_rows %lld must lie in [0, 2^31)", (long long)p->state_rows);
+    if (p->state_rows > 0 && !p->conv_state_indices)
+        return fail(CANON_ERR_INVALID_ARGUMENT, "state_rows is the size of the pool conv_state_indices selects from; without them it must be 0");
     const bool empty = p->batch == 0 || p->channels == 0;
     if (check_pointers && !empty) {
         if (!p->x || !p->conv_state || !p->weight || !p->dout || !p->dx)
@@ -755,6 +759,7 @@ int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, b
     a.B = (uint32_t)p->batch; a.C = (uint32_t)p->channels;
     a.W = p->width; a.S = p->state_len; a.w_dtype = p->w_dtype; a.mask_dtype = p->mask_dtype;
     a.act = p->activation; a.res_mode = p->residual_mode;
+    a.seqlens = p->cache_seqlens; a.indices = p->conv_state_indices; a.state_rows = (uint32_t)p->state_rows;
     plan->grid_c = 0;
     plan->workspace_bytes = 0;
     plan->vec = false;
@@ -769,7 +774,8 @@ int plan_update_bwd(const canon_conv1d_update_bwd_params *p, UpdBwdPlan *plan, b
     auto dense_token = [&](const void *ptr, int64_t sb, int64_t sc) {
         return (uintptr_t)ptr % 4 == 0 && sc == 1 && sb * BY % 4 == 0;
     };
-    plan->vec = (S == 3 || S == 4) && a.C % E == 0 && (!check_pointers || (
+    // (ring buffer and state pool: the strided kernel)
+    plan->vec = !p->cache_seqlens && !p->conv_state_indices && (S == 3 || S == 4) && a.C % E == 0 && (!check_pointers || (
                     dense_token(p->x, a.x_sb, a.x_sc) && dense_token(p->dout, a.g_sb, a.g_sc) &&
                     dense_token(p->dx, a.d_sb, a.d_sc) && dense_state(p->conv_state, a.s_sb, a.s_sc, a.s_ss) &&
                     dense_state(p->dstate_out, a.q_sb, a.q_sc, a.q_ss) && dense_state(p->dstate, a.r_sb, a.r_sc, a.r_ss)));

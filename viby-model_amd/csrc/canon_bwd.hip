@@ -1079,6 +1079,14 @@ __device__ __forceinline__ void store_partial_right(const UpdBwdArgs &a, float *
     pp[4] = db;
 }
 
+// Ring-buffer mode (seqlens): the forward wrote the token to slot p = seqlens[b] mod S and read the W-1 slots before
+// it cyclically, every other slot stayed where it was.  That is the shift register seen through a rotation: entry j
+// of the state before the step lives in slot (p + j) mod S, entry i of the state after it in slot (p + 1 + i) mod S,
+// so the code below is written in shift-register entries and maps them to slots where it touches memory.
+// State-pool mode (indices): batch entry b uses row indices[b] of conv_state / dstate_out / dstate; an entry whose
+// index lies outside the pool was skipped by the forward (its output is a constant zero row): dx = 0, nothing else.
+// Only the rows the entries name are written: the caller fills dstate with dstate_out (or zeros) beforehand, so that
+// the rows no entry used pass their gradient through.
 template <int DT>
 __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs a)
 {
@@ -1096,38 +1104,60 @@ __global__ __launch_bounds__(256) void canon_update_bwd_kernel(const UpdBwdArgs 
     for (uint32_t b0 = b_begin; b0 < b_stop; b0 += NB) {
         // every load of the NB entries first (nothing is stored in between, so they are in flight together)
         float xr[NB], go[NB], m[NB], wn[NB][3], qr[NB][4];
+        int64_t row[NB];                    // row of the state tensors, -1: entry skipped
+        int pos[NB];                        // ring: slot of the token, else -1
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
             const uint32_t b = b0 + n < b_stop ? b0 + n : b_stop - 1u;
+            row[n] = b;
+            if (a.indices) {
+                const int32_t i = a.indices[b];
+                row[n] = (i < 0 || (a.state_rows > 0 && (uint32_t)i >= a.state_rows)) ? -1 : i;
+            }
+            pos[n] = -1;
+            if (a.seqlens) {
+                pos[n] = a.seqlens[b] % S;
+                if (pos[n] < 0) pos[n] += S;
+            }
+            const bool live = row[n] >= 0;
+            // slots of entry j of the state before the step and of entry e of the state after it
+            auto slot = [&](int j) { return pos[n] < 0 ? j : (pos[n] + j) % S; };
+            auto slot_after = [&](int e) { return pos[n] < 0 ? e : (pos[n] + 1 + e) % S; };
             xr[n] = load1<DT>(a.x, (int64_t)b * a.x_sb + (int64_t)c * a.x_sc);
-            go[n] = load1<DT>(a.dy, (int64_t)b * a.g_sb + (int64_t)c * a.g_sc);
+            go[n] = live ? load1<DT>(a.dy, (int64_t)b * a.g_sb + (int64_t)c * a.g_sc) : 0.0f;
             m[n] = a.tmask ? load_mask(a.tmask, (int64_t)b * a.m_sb, a.mask_dtype) : 1.0f;
-            const int64_t so = (int64_t)b * a.s_sb + (int64_t)c * a.s_sc;
-            const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
+            const int64_t so = row[n] * a.s_sb + (int64_t)c * a.s_sc;
+            const int64_t qo = row[n] * a.q_sb + (int64_t)c * a.q_sc;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                if (i < 3) wn[n][i] = i >= lead ? load1<DT>(a.state, so + (int64_t)(S - 3 + i) * a.s_ss) : 0.0f;
-                qr[n][i] = (a.dso && i >= lead && S - 4 + i >= 0) ? load1<DT>(a.dso, qo + (int64_t)(S - 4 + i) * a.q_ss) : 0.0f;
+                if (i < 3) wn[n][i] = (live && i >= lead) ? load1<DT>(a.state, so + (int64_t)slot(S - 3 + i) * a.s_ss) : 0.0f;
+                qr[n][i] = (live && a.dso && i >= lead && S - 4 + i >= 0) ? load1<DT>(a.dso, qo + (int64_t)slot_after(S - 4 + i) * a.q_ss) : 0.0f;
             }
         }
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
             const uint32_t b = b0 + n;
             if (b >= b_stop) break;
+            if (row[n] < 0) {
+                store1<DT>(a.dx, (int64_t)b * a.d_sb + (int64_t)c * a.d_sc, 0.0f);
+                continue;
+            }
+            auto slot = [&](int j) { return pos[n] < 0 ? j : (pos[n] + j) % S; };
+            auto slot_after = [&](int e) { return pos[n] < 0 ? e : (pos[n] + 1 + e) % S; };
             const float xt = a.tmask ? mul_round<DT>(xr[n], m[n]) : xr[n];
             float dxv;
             const float dz = update_bwd_point(a, wr, bv, wn[n], qr[n], xr[n], xt, go[n], m[n], dwr, db, dxv);
             store1<DT>(a.dx, (int64_t)b * a.d_sb + (int64_t)c * a.d_sc, dxv);
             if (a.ds) {
-                const int64_t ro = (int64_t)b * a.r_sb + (int64_t)c * a.r_sc;
-                const int64_t qo = (int64_t)b * a.q_sb + (int64_t)c * a.q_sc;
-                // slots no tap reads: the gradient of the updated state shifted by one
+                const int64_t ro = row[n] * a.r_sb + (int64_t)c * a.r_sc;
+                const int64_t qo = row[n] * a.q_sb + (int64_t)c * a.q_sc;
+                // entries no tap reads: the gradient of the updated state one entry earlier (the same slot of a ring)
                 for (int j = 0; j < S - 3 + lead; ++j)
-                    store1<DT>(a.ds, ro + (int64_t)j * a.r_ss,
-                               (a.dso && j >= 1) ? load1<DT>(a.dso, qo + (int64_t)(j - 1) * a.q_ss) : 0.0f);
+                    store1<DT>(a.ds, ro + (int64_t)slot(j) * a.r_ss,
+                               (a.dso && j >= 1) ? load1<DT>(a.dso, qo + (int64_t)slot_after(j - 1) * a.q_ss) : 0.0f);
 #pragma unroll
                 for (int i = 0; i < 3; ++i)
-                    if (i >= lead) store1<DT>(a.ds, ro + (int64_t)(S - 3 + i) * a.r_ss, fmaf(wr[i], dz, qr[n][i]));
+                    if (i >= lead) store1<DT>(a.ds, ro + (int64_t)slot(S - 3 + i) * a.r_ss, fmaf(wr[i], dz, qr[n][i]));
             }
         }
     }

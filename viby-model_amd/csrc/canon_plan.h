@@ -158,6 +158,10 @@ struct UpdBwdArgs {
     uint32_t group;        // batch entries per group
     uint32_t ngroups;
     int32_t W, S, w_dtype, mask_dtype, act, res_mode;
+    // the modes the strided kernel alone covers
+    const int32_t *seqlens;   // ring buffer: the forward wrote the token to slot seqlens[b] % S
+    const int32_t *indices;   // state pool: batch entry b used row indices[b] of the state tensors
+    uint32_t state_rows;      // rows of the pool (0: not stated)
 };
 
 // Several channel ranges of one logical [B, C, L] problem that live in separate

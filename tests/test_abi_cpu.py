@@ -566,6 +566,13 @@ def test_torch_operators_for_traced_graphs_have_shape_only_twins():
     assert [tuple(t.shape) for t in outs] == [(2, 12, 40), (2, 4, 40), (2, 16, 3)]
     outs = ops.update_parts([x[:, :12, 0], x[:, 12:, 0]], st, w, None, None, 0, 0, 0)
     assert [tuple(t.shape) for t in outs] == [(2, 12), (2, 4)]
+    # the decode step as a function (traced graphs with gradients): output and new state, nothing written to
+    out, new = ops.update_step(x[:, :, 0], st, w, b, None, None, None, 1, 1)
+    assert tuple(out.shape) == (2, 16) and new.shape == st.shape and new.dtype == st.dtype
+    assert "!" not in str(ops.update_step.default._schema)
+    g = ops.update_bwd(x[:, :, 0], st, w, b, None, x[:, :, 0], st, None, None, 1, 1)
+    assert [tuple(t.shape) for t in g] == [(2, 16), (2, 16, 4), (16, 4), (16,)] and g[2].dtype == w.dtype
+    assert tuple(ops.update_bwd(x[:, :, 0], st, w, None, None, x[:, :, 0], st, None, None, 0, 0)[3].shape) == (0,)
     # the state arguments of the decode operators are declared as written to
     assert "Tensor(a1!) conv_state" in str(ops.update.default._schema)
     assert "Tensor(a1!) conv_state" in str(ops.update_parts.default._schema)

@@ -339,3 +339,68 @@ def test_compiled_training_through_the_captured_state(cc):
         got = step(fn)
         for name, a, e, tol in zip(("y", "dx", "dweight", "dbias"), got, want, (1e-6, 2e-5, 1e-4, 1e-4)):
             assert (a - e).abs().max().item() <= tol * (e.abs().max().item() + 1e-30), name
+
+
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+@pytest.mark.parametrize("mode", ["shift", "ring"])
+def test_compiled_decode_steps_have_the_eager_gradients(cc, backend, mode):
+    """A chain of single-token steps traced with gradients (the step as a function with its backward registered,
+    the state overwritten by a copy the tracer understands): outputs, final state and every gradient, the one
+    that flows from step to step through the state included, equal those of the same chain run eagerly."""
+    torch.manual_seed(11)
+    B, C, S, T = 4, 128, 4, 3
+    xs0 = torch.randn(T, B, C, device=DEV).bfloat16()
+    st0 = torch.randn(B, C, S, device=DEV).bfloat16()
+    w0 = (torch.randn(C, 4, device=DEV) * 0.3).bfloat16()
+    b0 = (torch.randn(C, device=DEV) * 0.1).bfloat16()
+    tm = torch.tensor([1, 1, 0, 1], device=DEV)
+    seqlens = [torch.full((B,), 5 + t, dtype=torch.int32, device=DEV) if mode == "ring" else None for t in range(T)]
+
+    def chain(xs, state0, w, b):
+        s = state0.clone()
+        outs = []
+        for t in range(T):
+            outs.append(cc.causal_conv1d_update(xs[t], s, w, b, activation="silu", token_mask=tm, residual=True,
+                                                cache_seqlens=seqlens[t]))
+        return torch.stack(outs), s
+
+    def run(fn):
+        xs, st, w, b = (t.clone().requires_grad_() for t in (xs0, st0, w0, b0))
+        outs, s = fn(xs, st, w, b)
+        loss = (outs.float() * torch.arange(1, T + 1, device=DEV).view(T, 1, 1)).sum() + (s.float() ** 2).sum()
+        loss.backward()
+        return outs.detach(), s.detach(), xs.grad, st.grad, w.grad, b.grad
+
+    want = run(chain)
+    got = run(torch.compile(chain, backend=backend, fullgraph=True))
+    for name, a, e in zip(("out", "state", "dx", "dstate", "dweight", "dbias"), got, want):
+        if backend == "inductor" and name in ("dweight", "dbias"):
+            # the three steps' bf16 contributions are added up by the compiler in one fused kernel (one rounding)
+            # and by eager autograd one after the other (two)
+            torch.testing.assert_close(a.float(), e.float(), rtol=2e-2, atol=2e-2, msg=name)
+        else:
+            assert torch.equal(bits(a), bits(e)), name
+
+
+def test_compiled_decode_step_with_gradients_on_a_cache_tensor(cc):
+    """The state as an argument of the traced function (a cache tensor that lives outside it, as CanonLayer keeps
+    it): each compiled call overwrites it, and the gradient flows back through it from call to call."""
+    torch.manual_seed(12)
+    B, C, S, T = 2, 64, 4, 3
+    xs0 = torch.randn(T, B, C, device=DEV).bfloat16()
+    w0 = (torch.randn(C, 4, device=DEV) * 0.3).bfloat16()
+
+    def step(x, state, w):
+        return cc.causal_conv1d_update(x, state, w, residual=True) * 2.0
+
+    def run(fn):
+        xs, w = xs0.clone().requires_grad_(), w0.clone().requires_grad_()
+        state = torch.zeros(B, C, S, device=DEV, dtype=torch.bfloat16)
+        outs = [fn(xs[t], state, w) for t in range(T)]
+        (torch.stack(outs).float().sum() + (state.float() ** 2).sum()).backward()
+        return torch.stack(outs).detach(), state.detach(), xs.grad, w.grad
+
+    want = run(step)
+    got = run(torch.compile(step, backend="aot_eager", fullgraph=True))
+    for name, a, e in zip(("out", "state", "dx", "dweight"), got, want):
+        assert torch.equal(bits(a), bits(e)), name

@@ -564,10 +564,10 @@ def causal_conv1d_update(
     if conv_state.shape[2] < weight.shape[1] - 1:
         raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
     wants_grad = _wants_grad(x, weight, bias, conv_state)
-    if wants_grad and (rnd != 0 or torch.compiler.is_compiling()):
+    if wants_grad and rnd != 0:
         raise NotImplementedError(
-            "causal_conv1d_update (gfx950): the backward of the decode step covers rounding='fused' outside "
-            "torch.compile; call under torch.no_grad() or detach the inputs")
+            "causal_conv1d_update (gfx950): the backward of the decode step covers rounding='fused'; call under "
+            "torch.no_grad() or detach the inputs")
     bias = _prep_bias(weight, bias)
     if token_mask is not None:
         if token_mask.dim() != 1 or token_mask.shape[0] != batch:
@@ -575,7 +575,15 @@ def causal_conv1d_update(
         if token_mask.dtype not in _lib.MASK_CODE or token_mask.device != x.device:
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
 
-    if wants_grad:
+    if wants_grad and torch.compiler.is_compiling():
+        # a traced graph with gradients: the step as a function (token, state) -> (output, new state) with its
+        # backward registered, and the caller's state tensor overwritten by an ordinary copy the tracer understands
+        # (the operator keeps its state argument for the backward, so it is handed a copy that the write below does
+        # not touch)
+        out, new_state = torch.ops.canon_conv1d.update_step(x2, conv_state.clone(), weight, bias, token_mask,
+                                                            cache_seqlens, conv_state_indices, act, res)
+        conv_state.copy_(new_state)
+    elif wants_grad:
         out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens, conv_state_indices)
     elif torch.compiler.is_compiling():
         out = torch.ops.canon_conv1d.update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices,
@@ -1047,6 +1055,57 @@ def _op_update(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, 
 @_op_update.register_fake
 def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
     return x.new_empty(tuple(x.shape))
+
+
+# The decode step as a function, for traced graphs that need its gradient: the state is not overwritten but returned
+# (an operator that mutates an argument cannot carry a gradient through that argument).
+@torch.library.custom_op("canon_conv1d::update_step", mutates_args=(), device_types="cuda")
+def _op_update_step(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                    token_mask: Optional[torch.Tensor], cache_seqlens: Optional[torch.Tensor],
+                    conv_state_indices: Optional[torch.Tensor], act: int, res: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    new_state = conv_state.clone(memory_format=torch.contiguous_format)
+    out = _launch_update(x, new_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, 0)
+    return out, new_state
+
+
+@_op_update_step.register_fake
+def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res):
+    return x.new_empty(tuple(x.shape)), torch.empty_like(conv_state, memory_format=torch.contiguous_format)
+
+
+@torch.library.custom_op("canon_conv1d::update_bwd", mutates_args=(), device_types="cuda")
+def _op_update_bwd(x: torch.Tensor, before: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                   token_mask: Optional[torch.Tensor], dout: torch.Tensor, dstate_out: torch.Tensor,
+                   cache_seqlens: Optional[torch.Tensor], conv_state_indices: Optional[torch.Tensor], act: int, res: int
+                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    dx, dstate, dweight, dbias = _launch_update_bwd(x, before, weight, bias, token_mask, dout, dstate_out, act, res,
+                                                    True, True, cache_seqlens, conv_state_indices)
+    return (dx, dstate, dweight.to(weight.dtype),
+            dbias.to(bias.dtype) if dbias is not None else weight.new_empty((0,)))
+
+
+@_op_update_bwd.register_fake
+def _(x, before, weight, bias, token_mask, dout, dstate_out, cache_seqlens, conv_state_indices, act, res):
+    return (x.new_empty(tuple(x.shape)), torch.empty_like(before, memory_format=torch.contiguous_format),
+            torch.empty_like(weight, memory_format=torch.contiguous_format),
+            weight.new_empty((weight.shape[0],), dtype=bias.dtype) if bias is not None else weight.new_empty((0,)))
+
+
+def _op_update_step_setup(ctx, inputs, output):
+    x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res = inputs
+    ctx.save_for_backward(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices)
+    ctx.flags = (act, res, bias is not None)
+
+
+def _op_update_step_backward(ctx, dout, dnew_state):
+    x, before, weight, bias, token_mask, cache_seqlens, conv_state_indices = ctx.saved_tensors
+    act, res, has_bias = ctx.flags
+    dx, dstate, dweight, dbias = torch.ops.canon_conv1d.update_bwd(
+        x, before, weight, bias, token_mask, dout.contiguous(), dnew_state, cache_seqlens, conv_state_indices, act, res)
+    return dx, dstate, dweight, (dbias if has_bias else None), None, None, None, None, None
+
+
+_op_update_step.register_autograd(_op_update_step_backward, setup_context=_op_update_step_setup)
 
 
 @torch.library.custom_op("canon_conv1d::fwd_parts", mutates_args=(), device_types="cuda")

@@ -71,6 +71,47 @@ def test_config2_bf16_prefill(cc, C, act):
         assert_parity(got, want, exact=act is None, what=f"config2/C{C}/{act}/{name}")
 
 
+# ---- unmasked channel-contiguous launches of 40 MB and more run slabs of four time steps per wave -----------------------
+@pytest.mark.parametrize("dtype,B,C,L", [(torch.bfloat16, 4, 2048, 1723), (torch.float16, 3, 3456, 1030),
+                                         (torch.float32, 2, 2600, 1029)])
+def test_short_slab_launches_with_everything_on(cc, dtype, B, C, L):
+    """The large unmasked launches (slabs of 4 steps, taps fetched first through the leading arguments): lengths that
+    end inside a tile and inside a slab, a channel count that ends inside a 64-lane tile, initial and final states,
+    SiLU, both residual settings, fp32 taps on 16-bit inputs, both rounding modes; the same call with an all-ones
+    mask (slabs of 8 steps) gives the same bits."""
+    g = torch.Generator().manual_seed(L)
+    assert 2 * B * C * L * torch.empty(0, dtype=dtype).element_size() >= 40 << 20
+    x = torch.randn(B, C, L, generator=g).to(dtype)
+    w = (torch.randn(C, 4, generator=g) * 0.3).to(dtype)
+    b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+    init = torch.randn(B, C, 5, generator=g).to(dtype)
+    xg = x.transpose(1, 2).contiguous().to(DEV).transpose(1, 2)
+    ones = torch.ones(B, L, dtype=torch.bool)
+    for act, residual, use_state, wt in [(None, True, True, dtype), ("silu", False, False, dtype),
+                                         ("silu", True, True, torch.float32), (None, False, False, torch.float32)]:
+        if wt != dtype and dtype == torch.float32:
+            continue
+        ww, bb = w.to(wt), b.to(wt)
+        want = co.conv1d_fwd(x, ww, bb, activation=act, residual=1 if residual else 0,
+                             initial_state=init if use_state else None, final_state_len=6 if use_state else None)
+        want_out, want_fs = want if use_state else (want, None)
+        r = run_fwd(cc, xg, ww, bb, act=act, residual=residual, init=init if use_state else None,
+                    S_out=6 if use_state else None)
+        got, fs = r if use_state else (r, None)
+        what = f"short slabs/{dtype}/{act}/res{residual}/state{use_state}/taps {wt}"
+        assert_parity(got, want_out, exact=act is None, what=what, res=x if residual else None)
+        if use_state:
+            assert torch.equal(bits(fs), bits(want_fs)), what
+        r8 = run_fwd(cc, xg, ww, bb, act=act, residual=residual, mask=ones, init=init if use_state else None,
+                     S_out=6 if use_state else None)
+        got8 = r8[0] if use_state else r8
+        assert torch.equal(bits(got), bits(got8)), what + ": slabs of 4 and of 8 steps differ"
+    # the eager module's rounding points, against the C oracle's round_mode = 1
+    want = co.conv1d_fwd(x, w, b, residual=1, round_mode=1)
+    got = run_fwd(cc, xg, w, b, residual=True, rounding="eager")
+    assert torch.equal(bits(got), bits(want)), f"short slabs/{dtype}/eager rounding"
+
+
 # ---- benchmark configuration 3: ragged right-padded batch of 32 ------------------------------------------------------
 @pytest.mark.parametrize("residual", ["masked", "unmasked"])
 def test_config3_ragged_padded_prefill(cc, residual):

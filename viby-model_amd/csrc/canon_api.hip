@@ -88,7 +88,14 @@ Extent extent_of(const void *base, int64_t B, int64_t C, int64_t L, int64_t sb, 
     return e;
 }
 
-int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
+// Time steps per wave of the channel-contiguous prefill for a problem that moves `bytes` (see kBlcRowsShort).
+static int blc_rows_for(const canon_conv1d_fwd_params *p, uint64_t bytes)
+{
+    return (!p->mask && !p->seq_idx && p->width == 4 && bytes >= kBlcShortSlabBytes) ? kBlcRowsShort : kBlcRows;
+}
+
+// blc_rows: time steps per wave of the channel-contiguous kernel; 0 = chosen here from the call's own size
+int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan, int blc_rows = 0)
 {
     if (!p) return fail(CANON_ERR_INVALID_ARGUMENT, "params is NULL");
     if (p->struct_size != sizeof(canon_conv1d_fwd_params))
@@ -247,7 +254,9 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan)
     if (blc_ok) {
         const uint32_t nvec = a.C / EB;
         const uint32_t nct = (nvec + 64 * kBlcWC - 1) / (64 * kBlcWC);          // channel tiles per row
-        const uint32_t ntt = (a.L + kBlcWaves * kBlcRows - 1) / (kBlcWaves * kBlcRows);   // time tiles per sequence
+        if (blc_rows == 0) blc_rows = blc_rows_for(p, 2ull * rows * a.L * elem_bytes(p->x_dtype));
+        plan->rows = blc_rows;
+        const uint32_t ntt = (a.L + kBlcWaves * blc_rows - 1) / (kBlcWaves * blc_rows);   // time tiles per sequence
         // `group` consecutive time tiles of a channel tile run back to back on one XCD (see blc_block_body): the
         // largest power of two up to kBlcGroup (the kernel divides by it with a shift) that leaves at most an
         // eighth of the block slots of a sequence without a tile (such blocks return at once)
@@ -410,6 +419,7 @@ int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *pa
     int64_t c0 = 0;
     uint64_t blocks = 0;
     bool all_blc = true;
+    canon_conv1d_fwd_params qs[kMaxParts];
     for (int i = 0; i < nparts; ++i) {
         canon_conv1d_fwd_params q = *p;
         q.channels = parts[i].channels;
@@ -420,8 +430,9 @@ int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *pa
         q.bias = advance(p->bias, c0, wb);
         q.initial_state = advance(p->initial_state, c0 * p->init_stride_c, xb);
         q.final_state = (void *)advance(p->final_state, c0 * p->final_stride_c, xb);
-        rc = plan_fwd(&q, &pp->part[i]);
+        rc = plan_fwd(&q, &pp->part[i], kBlcRows);   // (the table-of-parts kernel has the long slabs only)
         if (rc != CANON_OK) return rc;
+        qs[i] = q;
         if (pp->part[i].grid > 0) {
             all_blc = all_blc && pp->part[i].kind == FWD_BLC;
             blocks += pp->part[i].grid;
@@ -447,9 +458,29 @@ int plan_fwd_parts(const canon_conv1d_fwd_params *p, const canon_conv1d_part *pa
             (uint64_t)u.nvec * kBlcVecBytes < (1ull << 31) && nblocks < (1ull << 31) - 8) {
             pp->pair = true;
             pp->grid = (uint32_t)nblocks;
+            // the slab length is chosen on the whole problem, like the store policy
+            const int r = blc_rows_for(p, 2ull * (uint64_t)p->batch * (uint64_t)p->channels * (uint64_t)p->seqlen * xb);
+            if (r != kBlcRows) {
+                for (int i = 0; i < 2; ++i) {
+                    rc = plan_fwd(&qs[i], &pp->part[i], r);
+                    if (rc != CANON_OK) return rc;
+                    pp->part[i].args.nt = nt;
+                }
+                const uint64_t nb = (2ull * pp->part[0].args.ntasks + 7) / 8 * 8 * pp->part[0].args.chunk;
+                if (pp->part[0].kind != FWD_BLC || pp->part[1].kind != FWD_BLC || nb >= (1ull << 31) - 8)
+                    return fail(CANON_ERR_UNSUPPORTED, "internal: the pair launch could not be planned with short slabs");
+                pp->grid = (uint32_t)nb;
+            }
         }
     }
 #endif
+    // parts that go out as launches of their own are planned as single tensors are
+    if (!pp->single && !pp->pair)
+        for (int i = 0; i < nparts; ++i) {
+            rc = plan_fwd(&qs[i], &pp->part[i]);
+            if (rc != CANON_OK) return rc;
+            pp->part[i].args.nt = nt;
+        }
     return CANON_OK;
 }
 

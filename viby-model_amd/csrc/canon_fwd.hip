@@ -1083,10 +1083,20 @@ template <int DT, int W, bool MASK, bool BIG> void launch_fwd_vec(const FwdPlan 
         const uint32_t packed = lg | (uint32_t)a.tap_mode << 2 | a.div_nct.s1 << 4 | a.div_nct.s2 << 5 | a.div_ntt.s1 << 10 |
                                 a.div_ntt.s2 << 11 | a.nct << 16;
         const uint64_t wp = (uint64_t)(uintptr_t)a.weight, bp = (uint64_t)(uintptr_t)a.bias;
-        hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, kBlcRows, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, a.x,
-                           (uint32_t)(a.x_sb / (kBlcVecBytes / Elem<DT>::bytes)), (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec,
-                           a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp, (uint32_t)bp,
-                           (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a);
+#define CANON_BLC_LAUNCH(RR)                                                                                             \
+    hipLaunchKernelGGL((canon_fwd_blc_kernel<DT, W, RR, MASK, BIG>), dim3(pl.grid), dim3(kBlcThreads), 0, s, a.x,        \
+                       (uint32_t)(a.x_sb / (kBlcVecBytes / Elem<DT>::bytes)), (uint32_t)(a.x_sl * Elem<DT>::bytes), a.L, a.nvec, \
+                       a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp, (uint32_t)bp,                 \
+                       (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a)
+        // (short slabs are planned for unmasked width-4 launches only)
+        if constexpr (W == 4 && !MASK) {
+            if (pl.rows == kBlcRowsShort) {
+                CANON_BLC_LAUNCH(kBlcRowsShort);
+                return;
+            }
+        }
+        CANON_BLC_LAUNCH(kBlcRows);
+#undef CANON_BLC_LAUNCH
     }
 }
 
@@ -1142,9 +1152,18 @@ template <int DT, bool MASK, bool BIG> void launch_blc_pair(const FwdPartsPlan &
     const uint32_t packed = lg | (uint32_t)a.tap_mode << 2 | a.div_nct.s1 << 4 | a.div_nct.s2 << 5 | a.div_ntt.s1 << 10 |
                             a.div_ntt.s2 << 11 | a.nct << 16;
     const uint64_t wp = (uint64_t)(uintptr_t)a.weight, bp = (uint64_t)(uintptr_t)a.bias;
-    hipLaunchKernelGGL((canon_fwd_blc_pair_kernel<DT, 4, kBlcRows, MASK, BIG>), dim3(pp.grid), dim3(kBlcThreads), 0, s, a.x,
-                       pp.part[1].args.x, a.L, a.nvec, a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp,
-                       (uint32_t)bp, (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a);
+#define CANON_PAIR_LAUNCH(RR)                                                                                            \
+    hipLaunchKernelGGL((canon_fwd_blc_pair_kernel<DT, 4, RR, MASK, BIG>), dim3(pp.grid), dim3(kBlcThreads), 0, s, a.x,   \
+                       pp.part[1].args.x, a.L, a.nvec, a.ntasks, a.div_nct.m, a.nseg, a.div_ntt.m, packed, (uint32_t)wp, \
+                       (uint32_t)bp, (uint32_t)(wp >> 32) | (uint32_t)(bp >> 32) << 16, a)
+    if constexpr (!MASK) {
+        if (pp.part[0].rows == kBlcRowsShort) {
+            CANON_PAIR_LAUNCH(kBlcRowsShort);
+            return;
+        }
+    }
+    CANON_PAIR_LAUNCH(kBlcRows);
+#undef CANON_PAIR_LAUNCH
 }
 #endif
 

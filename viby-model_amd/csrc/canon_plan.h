@@ -203,6 +203,11 @@ enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel
 constexpr int kBlcRows = CANON_BLC_ROWS;   // time steps per wave in the channel-contiguous kernel
+// ... and in its unmasked width-4 launches that move at least kBlcShortSlabBytes (single tensor or pair): measured
+// 2-8 % faster there (B 8, C 3456, bf16: 19.9 -> 19.45 us, with SiLU 20.85 -> 19.86 us; B 16, C 640: 10.2 -> 9.4 us),
+// 5-16 % slower below that size (B 8, C 640 / 960: 5.3 -> 6.2 / 6.7 -> 7.8 us) and 0-4 % slower with a padding mask
+constexpr int kBlcRowsShort = 4;
+constexpr uint64_t kBlcShortSlabBytes = 40ull << 20;
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work
 // channels a lane of the vectorised update owns: as many as make its piece of the [B, C, S] state one run
@@ -228,6 +233,7 @@ struct FwdPlan {
     int U;
     bool edge;   // bcl: rows do not start on 16-byte boundaries
     uint32_t wpb; // bcl: waves per block
+    int rows;    // blc: time steps per wave (kBlcRows or kBlcRowsShort)
     FwdArgs args;
     uint32_t grid;
 };

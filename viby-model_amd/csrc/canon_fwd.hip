@@ -552,7 +552,7 @@ __device__ __forceinline__ const void *shifted(const void *p, int64_t bytes) { r
 template <int DT, int W, int R, bool MASK, bool BIG, bool SEQ, int VB, int MODE, typename ARGS>
 __device__ __forceinline__ void blc_block_body(const ARGS &args, const BlcLead &h, const uint32_t tb, const uint32_t ct, const uint32_t tt,
                                                typename VecIO<VB>::type (*tail)[3][64],   // LDS: raw last three rows of each wave's slab
-                                               uint32_t (*taps_lds)[64 * (VB / 2) * 5])   // LDS: taps and bias of each channel tile
+                                               uint32_t (*taps_lds)[64 * (VB / 2) * 4 + 64 * kBlcWaves * ((VB / 2 + kBlcWaves - 1) / kBlcWaves)])   // LDS: taps and bias of each channel tile
 {
     constexpr int E = VB / Elem<DT>::bytes;
     constexpr int BY = Elem<DT>::bytes;
@@ -749,7 +749,7 @@ __device__ __forceinline__ void blc_block(const ARGS &a, const BlcLead &h, const
     __shared__ typename VecIO<VB>::type tail[kBlcWaves * kBlcWC][3][64];
     // taps and bias of the block's channel tiles as fetched by its waves together: fp32 weights of 16-bit x are the
     // largest case, 64 lanes x 4 channels x (4 taps + bias) x 4 bytes
-    constexpr int kTapWordsLds = 64 * (VB / 2) * 5;
+    constexpr int kTapWordsLds = 64 * (VB / 2) * 4 + 64 * kBlcWaves * ((VB / 2 + kBlcWaves - 1) / kBlcWaves);
     __shared__ uint32_t taps_lds[kBlcWC][kTapWordsLds];
     if constexpr (W == 4) {
         if (tap_mode == TAPS_SAME) {

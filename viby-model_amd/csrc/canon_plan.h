@@ -206,7 +206,10 @@ constexpr int kBlcRows = CANON_BLC_ROWS;   // time steps per wave in the channel
 // ... and in its unmasked width-4 launches that move at least kBlcShortSlabBytes (single tensor or pair): measured
 // 2-8 % faster there (B 8, C 3456, bf16: 19.9 -> 19.45 us, with SiLU 20.85 -> 19.86 us; B 16, C 640: 10.2 -> 9.4 us),
 // 5-16 % slower below that size (B 8, C 640 / 960: 5.3 -> 6.2 / 6.7 -> 7.8 us) and 0-4 % slower with a padding mask
-constexpr int kBlcRowsShort = 4;
+#ifndef CANON_BLC_ROWS_SHORT
+#define CANON_BLC_ROWS_SHORT 4
+#endif
+constexpr int kBlcRowsShort = CANON_BLC_ROWS_SHORT;
 constexpr uint64_t kBlcShortSlabBytes = 40ull << 20;
 constexpr uint64_t kStreamBytes = 64ull << 20;  // above this much traffic, x / out are accessed non-temporally
 constexpr int kUpdNB = 2;               // batch rows per lane in the vectorised update when there is plenty of work

@@ -227,7 +227,7 @@ int plan_fwd(const canon_conv1d_fwd_params *p, FwdPlan *plan, int blc_rows = 0)
         // 5+ TB/s.  Idle lane slots cost next to nothing here.
         int U = 1;
         uint64_t best = (nvec + 63u) / 64u;
-        for (int cand = 2; cand <= 4; cand *= 2) {
+        for (int cand = 2; cand <= kBclMaxVectorsPerLane; cand *= 2) {
             const uint64_t nseg = (nvec + 64u * cand - 1) / (64u * cand);
             if (nseg < best && rows * nseg >= 2048) {
                 U = cand;

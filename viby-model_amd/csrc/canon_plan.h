@@ -199,6 +199,10 @@ constexpr int kBwdVecBytes = CANON_BWD_VEC_BYTES;   // bytes per lane and row in
 constexpr int kBwdWaves = 4;
 constexpr int kBwdMaxChunk = 32 * kBwdSlab * kBwdWaves;   // most time steps one block of the channel-contiguous backward walks
 enum FwdKind { FWD_BCL, FWD_BCL_SHORT, FWD_BLC, FWD_GENERIC };
+#ifndef CANON_BCL_MAX_U
+#define CANON_BCL_MAX_U 4
+#endif
+constexpr int kBclMaxVectorsPerLane = CANON_BCL_MAX_U;   // most 16-byte vectors a lane of the time-contiguous kernel takes (1, 2 or 4)
 enum UpdKind { UPD_VEC, UPD_GENERIC };
 
 constexpr uint32_t kGenericChunk = 8;   // time steps per thread in the scalar kernel

@@ -450,8 +450,9 @@ COPY_LIB = os.path.join(ROOT, "tests", "copy_ceiling", "libcopy_ceiling.so")
 
 def bench_copy_ceiling(steps, warmup):
     """Plain copies with the prefill kernels' access patterns (tests/copy_ceiling/copy_ceiling.hip): whole rows
-    (every lane 16 bytes, 2 KB per wave: the time-contiguous kernel without its arithmetic) and 32-row x 512-byte
-    tiles through buffer accesses (the channel-contiguous kernel without history, taps and LDS), at the metric
+    (every lane 16 bytes, 2 KB per wave: the time-contiguous kernel without its arithmetic) and 512-byte wide tiles
+    of 16 rows (4 per wave, as the kernel's unmasked launches of 40 MB and more; 32 rows below that) through buffer
+    accesses (the channel-contiguous kernel without history, taps and LDS), at the metric
     shape and at four times it, same buffer rotation as the kernels; and an empty launch.  The line through the
     two sizes separates what a launch costs from the rate the data moves at."""
     import torch

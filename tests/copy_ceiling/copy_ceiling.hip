@@ -4,7 +4,8 @@
 //
 //   copy_rows   every lane 16 bytes, a wave two vectors per lane = 2 KB of one row, streamed accesses:
 //               the time-contiguous kernel without its arithmetic
-//   copy_tiles  [B, L, rowbytes] memory in tiles of 32 rows x 512 bytes: 8 bytes per lane, 8 rows per wave,
+//   copy_tiles  [B, L, rowbytes] memory in tiles of 32 rows x 512 bytes: 8 bytes per lane, 8 rows per wave (from 40 MB
+//               of traffic: 16 rows x 512 bytes, 4 rows per wave, as the kernel's unmasked launches of that size),
 //               4 waves per block, buffer accesses, consecutive time tiles of a column on one XCD, stores written
 //               through from 64 MB of traffic: the channel-contiguous kernel without history, taps, LDS and arithmetic
 //   copy_tile_shape  the same memory in other tile shapes (16 x 512 B, 16 x 1 KB and 32 x 1 KB with 16-byte lanes,
@@ -34,10 +35,11 @@ struct Tiles {
     uint32_t ncols, nct, ntt, L, rowbytes;
 };
 constexpr uint64_t kThroughBytes = 64ull << 20;   // traffic from which the channel-contiguous prefill writes its stores through
+constexpr uint64_t kShortSlabBytes = 40ull << 20; // ... and from which its unmasked launches run slabs of four rows
 
-template <int AUXS> __global__ __launch_bounds__(256) void copy_tiles_kernel(const Tiles g)
+template <int AUXS, uint32_t R> __global__ __launch_bounds__(256) void copy_tiles_kernel(const Tiles g)
 {
-    constexpr uint32_t R = 8, WT = 4, VB = 8;
+    constexpr uint32_t WT = 4, VB = 8;
     // block = (column group * ntt + time tile) * 8 + XCD; column = (batch entry, channel tile)
     const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
     const uint32_t jg = j / g.ntt, tt = j - jg * g.ntt;
@@ -138,15 +140,18 @@ __attribute__((visibility("default"))) int copy_tiles(const void *in, void *out,
     g.in = (const char *)in;
     g.out = (char *)out;
     g.nct = (rowbytes + 511u) / 512u;
-    g.ntt = (rows + 31u) / 32u;
+    const uint64_t traffic = 2ull * batch * rows * rowbytes;
+    const uint32_t slab = traffic >= kShortSlabBytes ? 4u : 8u;
+    g.ntt = (rows + 4u * slab - 1u) / (4u * slab);
     g.L = rows;
     g.rowbytes = rowbytes;
     const uint64_t ncols = (uint64_t)batch * g.nct;
     const uint64_t grid = (ncols + 7) / 8 * 8 * g.ntt;
     if (grid >= (1ull << 31)) return 1;
     g.ncols = (uint32_t)ncols;
-    if (2ull * batch * rows * rowbytes >= kThroughBytes) hipLaunchKernelGGL(copy_tiles_kernel<2 | 16>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
-    else hipLaunchKernelGGL(copy_tiles_kernel<2>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
+    if (traffic >= kThroughBytes) hipLaunchKernelGGL((copy_tiles_kernel<2 | 16, 4>), dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
+    else if (slab == 4u) hipLaunchKernelGGL((copy_tiles_kernel<2, 4>), dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
+    else hipLaunchKernelGGL((copy_tiles_kernel<2, 8>), dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, g);
     return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

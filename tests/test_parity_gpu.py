@@ -668,6 +668,35 @@ def test_large_time_contiguous_launches_in_blocks_of_eight_waves(cc):
             assert torch.equal(bits(state), bits(want_state)), what
 
 
+@pytest.mark.parametrize("dtype,shape", [(torch.bfloat16, (2, 40, 4096)), (torch.bfloat16, (1, 24, 8192 + 64)),
+                                         (torch.float32, (1, 16, 4096)), (torch.float16, (3, 8, 2048 + 512))])
+def test_long_unmasked_time_contiguous_rows_of_several_segments(cc, dtype, shape):
+    """Aligned rows longer than one wave covers, without a mask: every segment after a row's first takes its three
+    inputs of history from the vector before it, which its first lane requests together with the segment.  Widths
+    2-4, SiLU, both residual settings, initial and final states, both rounding modes."""
+    g = torch.Generator().manual_seed(shape[2])
+    B, C, L = shape
+    x = torch.randn(B, C, L, generator=g).to(dtype)
+    init = torch.randn(B, C, 4, generator=g).to(dtype)
+    xg = x.to(DEV)
+    for W in (2, 3, 4):
+        w = (torch.randn(C, W, generator=g) * 0.3).to(dtype)
+        b = (torch.randn(C, generator=g) * 0.1).to(dtype)
+        assert cc.kernel_plan_fwd(xg, w.to(DEV)) == "bcl_vec"
+        for act, res, st in [(None, True, True), ("silu", False, False), ("silu", True, True)]:
+            want = co.conv1d_fwd(x, w, b, activation=act, residual=1 if res else 0,
+                                 initial_state=init if st else None, final_state_len=5 if st else None)
+            want_out, want_fs = want if st else (want, None)
+            r = run_fwd(cc, xg, w, b, act=act, residual=res, init=init if st else None, S_out=5 if st else None)
+            got, fs = r if st else (r, None)
+            what = f"long rows/{dtype}/{shape}/W{W}/{act}/res{res}/state{st}"
+            assert_parity(got, want_out, exact=act is None, what=what, res=x if res else None)
+            if st:
+                assert torch.equal(bits(fs), bits(want_fs)), what
+        want = co.conv1d_fwd(x, w, b, residual=1, round_mode=1)
+        assert torch.equal(bits(run_fwd(cc, xg, w, b, residual=True, rounding="eager")), bits(want)), f"{shape}/W{W}/eager"
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_short_time_contiguous_rows_share_a_wave(cc, dtype):
     """Rows of 1..32 whole vectors: 2..64 rows per wave (every power-of-two group size, vector counts on and

@@ -130,7 +130,10 @@ __global__ __launch_bounds__(64 * kBclMaxWaves) void canon_fwd_bcl_kernel(const 
     const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * wpb + (threadIdx.x >> 6));
     if (task >= ntasks) return;
     uint32_t row = task, seg = 0;
-    if (nseg > 1) {
+    if (nseg == 2) {          // (from the leading scalars alone: no read of the argument block before the row loads)
+        row = task >> 1;
+        seg = task & 1u;
+    } else if (nseg > 1) {
         row = fdiv(task, a.div_nseg);
         seg = task - row * nseg;
     }
@@ -159,6 +162,13 @@ __global__ __launch_bounds__(64 * kBclMaxWaves) void canon_fwd_bcl_kernel(const 
         const uint32_t v = v0 + u * 64u;
         X[u] = make_uint4(0, 0, 0, 0);
         if (v < nvec) X[u] = load_vec<true>(xvec + (int64_t)v * 16);
+    }
+    // a later segment's history: the vector before the segment, requested by lane 0 together with the segment itself
+    // (the wave of the segment before requests the same vector at about the same time)
+    uint4 P = make_uint4(0, 0, 0, 0);
+    constexpr bool kPrevVector = !MASK && !EDGE;
+    if constexpr (kPrevVector) {
+        if (seg > 0 && lane == 0) P = load_vec<false>(xvec + ((int64_t)v0 - 1) * 16);
     }
 
     // EDGE: lanes 0 .. head-1 of the first segment take the elements before the first vector,
@@ -209,7 +219,13 @@ __global__ __launch_bounds__(64 * kBclMaxWaves) void canon_fwd_bcl_kernel(const 
 
     // history of the segment's first vector (only lane 0's copy is consumed)
     float carry[3] = {0.0f, 0.0f, 0.0f};
-    if (lane == 0) {
+    if (kPrevVector && seg > 0) {
+        float pv[E];
+        unpack_vec<DT>(P, pv);
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+            if (j >= 3 - (W - 1)) carry[j] = pv[E - 3 + j];
+    } else if (lane == 0) {
         if (seg > 0 || (EDGE && head > 0)) {
             const int64_t t0 = (int64_t)head + (int64_t)v0 * E;
 #pragma unroll

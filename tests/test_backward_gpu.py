@@ -222,8 +222,6 @@ def test_canon_layer_trains(cc):
 def test_unsupported_gradients_raise(cc):
     x = torch.randn(2, 8, 16, device=DEV, requires_grad=True)
     w = torch.randn(8, 4, device=DEV)
-    with pytest.raises(NotImplementedError, match="initial_states"):
-        cc.causal_conv1d_fn_parts([x[:, :4], x[:, 4:]], w, initial_states=torch.zeros(2, 8, 3, device=DEV))
     with pytest.raises(NotImplementedError, match="backward of the decode step"):
         cc.causal_conv1d_update_parts([x[:, :4, 0], x[:, 4:, 0]], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
@@ -469,6 +467,52 @@ def test_backward_through_final_states(cc, dtype, layout):
             check(ig.grad, want[4], dtype, "dinit " + tag)
         check(wg.grad, want[1], dtype, "dweight " + tag, sum_terms=B * L)
         check(bg.grad, want[2], dtype, "dbias " + tag, sum_terms=B * L)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_multi_part_call_differentiates_through_both_states(cc, dtype):
+    """causal_conv1d_fn_parts with initial_states and a captured final state that the loss reads: the gradients of
+    every part, of weight / bias and of the initial state against float64 autograd on the concatenation, and
+    against the single-tensor call on the concatenation (same kernels on the same rows: same bits)."""
+    torch.manual_seed(31)
+    for dims, L, S_in, S_out, act, residual, masked in [((24, 8, 8), 40, 3, 4, "silu", True, True),
+                                                       ((64, 64), 70, 4, 8, None, False, False),
+                                                       ((16, 40), 2, 8, 3, "silu", "unmasked", True),
+                                                       ((520, 8, 1032, 64), 33, 3, 8, None, True, False)]:
+        B, C, W = 2, sum(dims), 4
+        x = torch.randn(B, C, L).to(dtype)
+        w, b = (torch.randn(C, W) * 0.5).to(dtype), (torch.randn(C) * 0.1).to(dtype)
+        init = torch.randn(B, C, S_in).to(dtype)
+        dout, dfin = torch.randn(B, C, L).to(dtype), torch.randn(B, C, S_out).to(dtype)
+        mask = (torch.rand(B, L) > 0.3).to(torch.int64) if masked else None
+        mg = None if mask is None else mask.to(DEV)
+
+        def leaves():
+            parts = [t.transpose(1, 2).contiguous().to(DEV).transpose(1, 2).requires_grad_(True) for t in x.split(list(dims), dim=1)]
+            return parts, w.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True), init.to(DEV).requires_grad_(True)
+
+        parts, wg, bg, ig = leaves()
+        outs, fs = cc.causal_conv1d_fn_parts(parts, wg, bg, activation=act, initial_states=ig, residual=residual,
+                                             attention_mask=mg, final_states_out=torch.empty(B, C, S_out, dtype=dtype, device=DEV))
+        loss = sum((o.float() * d.to(DEV).float()).sum() for o, d in zip(outs, dout.split(list(dims), dim=1)))
+        (loss + (fs.float() * dfin.to(DEV).float()).sum()).backward()
+        torch.cuda.synchronize()
+        want = conv1d_grads(x, w, b, dout, mask=mask, activation=act, residual=residual, initial_states=init, dfinal=dfin)
+        tag = f"{dtype} dims{dims} L{L} S_in{S_in} S_out{S_out} act={act} res={residual} mask={masked}"
+        dx = torch.cat([p.grad.contiguous() for p in parts], dim=1)
+        check(dx, want[0], dtype, "dx " + tag)
+        check(ig.grad, want[4], dtype, "dinit " + tag)
+        check(wg.grad, want[1], dtype, "dweight " + tag, sum_terms=B * L)
+        check(bg.grad, want[2], dtype, "dbias " + tag, sum_terms=B * L)
+        # the single-tensor call on the concatenation
+        parts1, w1, b1, i1 = leaves()
+        xcat = torch.cat([p.detach() for p in parts1], dim=1).transpose(1, 2).contiguous().transpose(1, 2).requires_grad_(True)
+        out1, fs1 = cc.causal_conv1d_fn(xcat, w1, b1, activation=act, initial_states=i1, residual=residual, attention_mask=mg,
+                                        final_states_out=torch.empty(B, C, S_out, dtype=dtype, device=DEV))
+        ((out1.float() * dout.to(DEV).float()).sum() + (fs1.float() * dfin.to(DEV).float()).sum()).backward()
+        assert torch.equal(bits(dx), bits(xcat.grad.contiguous())), "dx vs concatenation " + tag
+        assert torch.equal(bits(ig.grad), bits(i1.grad)), "dinit vs concatenation " + tag
+        assert torch.equal(bits(fs), bits(fs1)), tag
 
 
 def test_block_in_two_chunks_trains_like_the_block_in_one_go(cc):

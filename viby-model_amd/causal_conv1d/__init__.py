@@ -850,8 +850,10 @@ def causal_conv1d_fn_parts(
     if batch * dim * seqlen == 0 and final_states is not None and final_states.numel():
         raise ValueError("cannot produce final states from an empty input")
 
-    if _wants_grad(*xs, weight, bias) and initial_states is not None:
-        raise NotImplementedError("gradients through a call with initial_states are not implemented")
+    wants_grad = _wants_grad(*xs, weight, bias, initial_states)
+    if wants_grad and initial_states is not None and torch.compiler.is_compiling():
+        raise NotImplementedError("causal_conv1d_fn_parts (gfx950): gradients through a call with initial_states are "
+                                  "implemented outside torch.compile")
     if torch.compiler.is_compiling():
         *outs, fin = torch.ops.canon_conv1d.fwd_parts(xs, weight, bias, attention_mask, initial_states,
                                                       final_states.shape[2] if final_states is not None else 0,
@@ -859,8 +861,8 @@ def causal_conv1d_fn_parts(
         outs = tuple(outs)
         if final_states is not None:
             final_states.copy_(fin)
-    elif _wants_grad(*xs, weight, bias):
-        result = _CanonConvPartsFn.apply(weight, bias, attention_mask, final_states, act, res, rnd, *xs)
+    elif wants_grad:
+        result = _CanonConvPartsFn.apply(weight, bias, attention_mask, final_states, act, res, rnd, initial_states, *xs)
         outs = tuple(result[:len(xs)])
     else:
         outs = _launch_fwd_parts(xs, weight, bias, attention_mask, initial_states, final_states, act, res, rnd)
@@ -882,35 +884,49 @@ def _launch_fwd_parts(xs, weight, bias, mask, initial_states, final_states, act,
 
 class _CanonConvPartsFn(torch.autograd.Function):
     """Autograd node of the multi-part prefill: one forward launch over all parts; the backward
-    runs the fused backward once per part, on that part's rows of weight / bias, so neither
-    direction concatenates anything."""
+    runs the fused backward once per part, on that part's rows of weight / bias and that part's channels of the
+    states, so neither direction concatenates anything.  As in the single-tensor node the captured final state is
+    differentiable (a gradient arriving through it flows back into the inputs) and so is the initial state."""
 
     @staticmethod
-    def forward(ctx, weight, bias, mask, final_states, act, res, rnd, *xs):
-        outs = _launch_fwd_parts(xs, weight, bias, mask, None, final_states, act, res, rnd)
-        ctx.save_for_backward(weight, bias, mask, *xs)
-        ctx.flags = (act, res)
+    def forward(ctx, weight, bias, mask, final_states, act, res, rnd, initial_states, *xs):
+        outs = _launch_fwd_parts(xs, weight, bias, mask, initial_states, final_states, act, res, rnd)
+        # (a copy of the small initial state: callers keep it in a cache tensor they overwrite right after the call)
+        ctx.save_for_backward(weight, bias, mask, initial_states.detach().clone() if initial_states is not None else None,
+                              *xs)
+        ctx.flags = (act, res, final_states is not None)
+        ctx.set_materialize_grads(False)
         if final_states is not None:
-            ctx.mark_non_differentiable(final_states)
+            ctx.mark_dirty(final_states)
             return (*outs, final_states)
         return outs
 
     @staticmethod
-    def backward(ctx, *douts):
-        weight, bias, mask, *xs = ctx.saved_tensors
-        act, res = ctx.flags
+    def backward(ctx, *grads):
+        weight, bias, mask, initial_states, *xs = ctx.saved_tensors
+        act, res, has_final = ctx.flags
+        douts = grads[:len(xs)]
+        dfinal = grads[len(xs)] if has_final else None
         channels, width = weight.shape
         dev = xs[0].device
         dweight = torch.empty(channels, width, dtype=torch.float32, device=dev)
         dbias = torch.empty(channels, dtype=torch.float32, device=dev) if bias is not None else None
+        dinit = None
+        if initial_states is not None and ctx.needs_input_grad[7]:
+            dinit = torch.empty_like(initial_states)
         dxs, c0 = [], 0
         for x, dout in zip(xs, douts):
             c1 = c0 + x.shape[1]
+            if dout is None:
+                dout = torch.zeros_like(x)
             dxs.append(_launch_bwd(x, dout, weight[c0:c1], bias[c0:c1] if bias is not None else None, mask,
-                                   dweight[c0:c1], dbias[c0:c1] if dbias is not None else None, act, res))
+                                   dweight[c0:c1], dbias[c0:c1] if dbias is not None else None, act, res, None,
+                                   initial_states[:, c0:c1] if initial_states is not None else None,
+                                   dinit[:, c0:c1] if dinit is not None else None,
+                                   dfinal[:, c0:c1] if dfinal is not None else None))
             c0 = c1
         return (dweight.to(weight.dtype), dbias.to(bias.dtype) if bias is not None else None,
-                None, None, None, None, None, *dxs)
+                None, None, None, None, None, dinit, *dxs)
 
 
 def causal_conv1d_update_parts(

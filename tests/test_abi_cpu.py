@@ -567,7 +567,7 @@ def test_torch_operators_for_traced_graphs_have_shape_only_twins():
     outs = ops.update_parts([x[:, :12, 0], x[:, 12:, 0]], st, w, None, None, 0, 0, 0)
     assert [tuple(t.shape) for t in outs] == [(2, 12), (2, 4)]
     # the decode step as a function (traced graphs with gradients): output and new state, nothing written to
-    out, new = ops.update_step(x[:, :, 0], st, w, b, None, None, None, 1, 1)
+    out, new = ops.update_step(x[:, :, 0], st, w, b, None, None, None, 1, 1, 0)
     assert tuple(out.shape) == (2, 16) and new.shape == st.shape and new.dtype == st.dtype
     assert "!" not in str(ops.update_step.default._schema)
     g = ops.update_bwd(x[:, :, 0], st, w, b, None, x[:, :, 0], st, None, None, 1, 1)

@@ -503,8 +503,6 @@ def test_errors_surface(cc):
         cc.causal_conv1d_fn(x, w, seq_idx=torch.zeros(2, 16, dtype=torch.int64, device=DEV))
     with pytest.raises(ValueError, match="shorter than width-1"):
         cc.causal_conv1d_update(x[:, :, 0], torch.zeros(2, 8, 2, device=DEV), w)
-    with pytest.raises(NotImplementedError, match="backward"):
-        cc.causal_conv1d_update(x[:, :, 0].requires_grad_(), torch.zeros(2, 8, 4, device=DEV), w, rounding="eager")
 
 
 def test_integer_mask_narrowing_is_never_stale(cc):

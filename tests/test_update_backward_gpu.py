@@ -266,8 +266,16 @@ def test_update_backward_at_decode_shape_is_deterministic(cc):
 def test_update_backward_argument_handling(cc):
     x = torch.randn(2, 8, device=DEV, requires_grad=True)
     w = torch.randn(8, 4, device=DEV)
-    with pytest.raises(NotImplementedError, match="rounding='fused'"):
-        cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV), w, rounding="eager")
+    # the eager module's rounding points in the forward, the gradient of the unrounded step in the backward
+    xe = x.detach().clone().requires_grad_(True)
+    se, sf = torch.randn(2, 8, 4, device=DEV), None
+    sf = se.clone()
+    oe = cc.causal_conv1d_update(xe, se, w, activation="silu", rounding="eager")
+    xf = x.detach().clone().requires_grad_(True)
+    of = cc.causal_conv1d_update(xf, sf, w, activation="silu")
+    oe.sum().backward()
+    of.sum().backward()
+    assert torch.allclose(oe, of, rtol=1e-5, atol=1e-6) and torch.equal(xe.grad, xf.grad)
     # a state that is a leaf requiring grad cannot be updated in place: torch says so itself
     with pytest.raises(RuntimeError, match="leaf"):
         cc.causal_conv1d_update(x, torch.zeros(2, 8, 4, device=DEV, requires_grad=True), w)

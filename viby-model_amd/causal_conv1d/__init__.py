@@ -564,10 +564,6 @@ def causal_conv1d_update(
     if conv_state.shape[2] < weight.shape[1] - 1:
         raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
     wants_grad = _wants_grad(x, weight, bias, conv_state)
-    if wants_grad and rnd != 0:
-        raise NotImplementedError(
-            "causal_conv1d_update (gfx950): the backward of the decode step covers rounding='fused'; call under "
-            "torch.no_grad() or detach the inputs")
     bias = _prep_bias(weight, bias)
     if token_mask is not None:
         if token_mask.dim() != 1 or token_mask.shape[0] != batch:
@@ -581,10 +577,11 @@ def causal_conv1d_update(
         # (the operator keeps its state argument for the backward, so it is handed a copy that the write below does
         # not touch)
         out, new_state = torch.ops.canon_conv1d.update_step(x2, conv_state.clone(), weight, bias, token_mask,
-                                                            cache_seqlens, conv_state_indices, act, res)
+                                                            cache_seqlens, conv_state_indices, act, res, rnd)
         conv_state.copy_(new_state)
     elif wants_grad:
-        out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens, conv_state_indices)
+        out, _ = _CanonUpdateFn.apply(x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens, conv_state_indices,
+                                      rnd)
     elif torch.compiler.is_compiling():
         out = torch.ops.canon_conv1d.update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices,
                                             act, res, rnd)
@@ -684,12 +681,15 @@ class _CanonUpdateFn(torch.autograd.Function):
     it) flows back into this step's token and into the state before it.  The ring-buffer mode
     (``cache_seqlens``, the mode of the reference's own update autograd, causal_conv1d_mps/autograd.py:341-498) and
     the state-pool mode (``conv_state_indices``) differentiate the same way; in pool mode ``conv_state`` is the
-    whole pool, and rows that no batch entry names pass their gradient through unchanged."""
+    whole pool, and rows that no batch entry names pass their gradient through unchanged.  With
+    ``rounding='eager'`` the forward rounds where the eager module does and the backward is that of the unrounded
+    step, as for the prefill."""
 
     @staticmethod
-    def forward(ctx, x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens=None, conv_state_indices=None):
+    def forward(ctx, x2, conv_state, weight, bias, token_mask, act, res, cache_seqlens=None, conv_state_indices=None,
+                rnd=0):
         before = conv_state.detach().clone()
-        out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, 0)
+        out = _launch_update(x2, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
         ctx.mark_dirty(conv_state)
         ctx.set_materialize_grads(False)
         ctx.save_for_backward(x2, before, weight, bias, token_mask, cache_seqlens, conv_state_indices)
@@ -707,7 +707,7 @@ class _CanonUpdateFn(torch.autograd.Function):
         dx, dstate, dweight, dbias = _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res,
                                                         want_state, want_params, cache_seqlens, conv_state_indices)
         return (dx, dstate, dweight.to(weight.dtype) if dweight is not None else None,
-                dbias.to(bias.dtype) if dbias is not None else None, None, None, None, None, None)
+                dbias.to(bias.dtype) if dbias is not None else None, None, None, None, None, None, None)
 
 
 def _launch_update_bwd(x2, before, weight, bias, token_mask, dout, dstate_out, act, res, want_state=True,
@@ -1078,14 +1078,15 @@ def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices
 @torch.library.custom_op("canon_conv1d::update_step", mutates_args=(), device_types="cuda")
 def _op_update_step(x: torch.Tensor, conv_state: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                     token_mask: Optional[torch.Tensor], cache_seqlens: Optional[torch.Tensor],
-                    conv_state_indices: Optional[torch.Tensor], act: int, res: int) -> Tuple[torch.Tensor, torch.Tensor]:
+                    conv_state_indices: Optional[torch.Tensor], act: int, res: int, rnd: int
+                    ) -> Tuple[torch.Tensor, torch.Tensor]:
     new_state = conv_state.clone(memory_format=torch.contiguous_format)
-    out = _launch_update(x, new_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, 0)
+    out = _launch_update(x, new_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd)
     return out, new_state
 
 
 @_op_update_step.register_fake
-def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res):
+def _(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, rnd):
     return x.new_empty(tuple(x.shape)), torch.empty_like(conv_state, memory_format=torch.contiguous_format)
 
 
@@ -1108,7 +1109,7 @@ def _(x, before, weight, bias, token_mask, dout, dstate_out, cache_seqlens, conv
 
 
 def _op_update_step_setup(ctx, inputs, output):
-    x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res = inputs
+    x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices, act, res, _rnd = inputs
     ctx.save_for_backward(x, conv_state, weight, bias, token_mask, cache_seqlens, conv_state_indices)
     ctx.flags = (act, res, bias is not None)
 
@@ -1118,7 +1119,7 @@ def _op_update_step_backward(ctx, dout, dnew_state):
     act, res, has_bias = ctx.flags
     dx, dstate, dweight, dbias = torch.ops.canon_conv1d.update_bwd(
         x, before, weight, bias, token_mask, dout.contiguous(), dnew_state, cache_seqlens, conv_state_indices, act, res)
-    return dx, dstate, dweight, (dbias if has_bias else None), None, None, None, None, None
+    return dx, dstate, dweight, (dbias if has_bias else None), None, None, None, None, None, None
 
 
 _op_update_step.register_autograd(_op_update_step_backward, setup_context=_op_update_step_setup)

@@ -222,8 +222,6 @@ def test_canon_layer_trains(cc):
 def test_unsupported_gradients_raise(cc):
     x = torch.randn(2, 8, 16, device=DEV, requires_grad=True)
     w = torch.randn(8, 4, device=DEV)
-    with pytest.raises(NotImplementedError, match="backward of the decode step"):
-        cc.causal_conv1d_update_parts([x[:, :4, 0], x[:, 4:, 0]], torch.zeros(2, 8, 4, device=DEV), w)
     out, fs = cc.causal_conv1d_fn(x, w, return_final_states=True)
     assert out.requires_grad and fs.requires_grad          # the captured state is differentiable
 

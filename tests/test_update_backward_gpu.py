@@ -157,6 +157,36 @@ def test_chain_of_ring_buffer_steps_has_the_gradients_of_the_shift_register_chai
     assert torch.equal(ds0, ds1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_multi_part_decode_step_has_the_gradients_of_the_single_tensor_step(cc, dtype):
+    """causal_conv1d_update_parts under autograd (q / k / v or gate / up tokens as separate tensors, one state):
+    outputs, updated state and every gradient, the one through the updated state included, equal those of
+    causal_conv1d_update on the concatenation (float64 autograd as the common yardstick)."""
+    torch.manual_seed(41)
+    for dims, S, act, residual, use_mask in [((24, 8, 8), 4, "silu", True, True), ((64, 64), 3, None, False, False),
+                                             ((16, 40), 8, "silu", "unmasked", True)]:
+        B, C = 5, sum(dims)
+        x, st = quantised((B, C), dtype), quantised((B, C, S), dtype)
+        w, b = quantised((C, 4), dtype, 0.5), quantised((C,), dtype, 0.1)
+        dout, dso = quantised((B, C), dtype), quantised((B, C, S), dtype)
+        mask = torch.tensor([1, 0, 1, 1, 0], dtype=torch.int64) if use_mask else None
+        parts = [t.contiguous().to(DEV).requires_grad_(True) for t in x.split(list(dims), dim=1)]
+        s0 = st.to(DEV).requires_grad_(True)
+        wg, bg = w.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+        s = s0.clone()
+        outs = cc.causal_conv1d_update_parts(parts, s, wg, bg, activation=act, residual=residual,
+                                             token_mask=None if mask is None else mask.to(DEV))
+        loss = sum((o.float() * d.to(DEV).float()).sum() for o, d in zip(outs, dout.split(list(dims), dim=1)))
+        (loss + (s.float() * dso.to(DEV).float()).sum()).backward()
+        want = update_grads(x, st, w, b, dout, dso, mask, act, residual)
+        tag = f"{dtype} dims{dims} S{S} act={act} res={residual} mask={use_mask}"
+        check(torch.cat([p.grad for p in parts], dim=1), want[0], dtype, "dx " + tag)
+        check(s0.grad, want[1], dtype, "dstate " + tag)
+        check(wg.grad, want[2], dtype, "dweight " + tag, sum_terms=B)
+        check(bg.grad, want[3], dtype, "dbias " + tag, sum_terms=B)
+        assert torch.equal(s.detach().cpu().double(), want[5]), "state " + tag
+
+
 def test_update_backward_finite_differences_like_the_reference_test(cc):
     """causal-conv1d-mps/test.py:294-321: batch 2, dim 8, width 4, state_len 8, SiLU, residual; eps 1e-3,
     atol 1e-3, rtol 1e-2, loss = out.sum() (test.py:8-80).  The state gradient is checked as well."""

@@ -77,13 +77,6 @@ def _require_gpu(t: torch.Tensor, what: str) -> None:
         raise ValueError(f"{what} must be on a ROCm GPU device (device type 'cuda'), got {t.device}")
 
 
-def _no_grad_needed(*tensors) -> None:
-    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
-        raise NotImplementedError(
-            "causal_conv1d_update_parts (gfx950): backward of the decode step is implemented for the single-tensor "
-            "call only; call under torch.no_grad() or detach the inputs")
-
-
 def _check_shapes(x_dim: int, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> None:
     """Shape / dtype errors first (they do not depend on where the tensors live)."""
     if weight.dim() != 2:
@@ -965,7 +958,11 @@ def causal_conv1d_update_parts(
     _check_devices(weight, bias, x0.device)
     if conv_state.shape[2] < weight.shape[1] - 1:
         raise ValueError(f"conv_state length {conv_state.shape[2]} is shorter than width-1 = {weight.shape[1] - 1}")
-    _no_grad_needed(*xs, weight, bias, conv_state)
+    wants_grad = _wants_grad(*xs, weight, bias, conv_state)
+    if wants_grad and torch.compiler.is_compiling():
+        raise NotImplementedError(
+            "causal_conv1d_update_parts (gfx950): the backward of the multi-part decode step is implemented outside "
+            "torch.compile; call under torch.no_grad() or detach the inputs")
     bias = _prep_bias(weight, bias)
     if token_mask is not None:
         if token_mask.dim() != 1 or token_mask.shape[0] != batch:
@@ -974,7 +971,51 @@ def causal_conv1d_update_parts(
             raise ValueError("token_mask must be a bool/int/float tensor on the device of x")
     if torch.compiler.is_compiling():
         return tuple(torch.ops.canon_conv1d.update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd))
+    if wants_grad:
+        return tuple(_CanonUpdatePartsFn.apply(conv_state, weight, bias, token_mask, act, res, rnd, *xs)[:len(xs)])
     return _launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd)
+
+
+class _CanonUpdatePartsFn(torch.autograd.Function):
+    """Autograd node of the multi-part decode step: one forward launch over all parts; the backward runs the decode
+    step's backward once per part, on that part's channels of the saved state and of the state gradients and on its
+    rows of weight / bias.  The state is modified in place and differentiable, as in ``_CanonUpdateFn``."""
+
+    @staticmethod
+    def forward(ctx, conv_state, weight, bias, token_mask, act, res, rnd, *xs):
+        before = conv_state.detach().clone()
+        outs = _launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd)
+        ctx.mark_dirty(conv_state)
+        ctx.set_materialize_grads(False)
+        ctx.save_for_backward(before, weight, bias, token_mask, *xs)
+        ctx.flags = (act, res)
+        return (*outs, conv_state)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        before, weight, bias, token_mask, *xs = ctx.saved_tensors
+        act, res = ctx.flags
+        douts, dstate_out = grads[:len(xs)], grads[len(xs)]
+        want_state = ctx.needs_input_grad[0]
+        want_params = ctx.needs_input_grad[1] or (bias is not None and ctx.needs_input_grad[2])
+        dstate = torch.empty_like(before) if want_state else None
+        dws, dbs, dxs, c0 = [], [], [], 0
+        for x, dout in zip(xs, douts):
+            c1 = c0 + x.shape[1]
+            if dout is None:
+                dout = torch.zeros_like(x)
+            dx, ds, dw, db = _launch_update_bwd(x, before[:, c0:c1], weight[c0:c1], bias[c0:c1] if bias is not None else None,
+                                                token_mask, dout, dstate_out[:, c0:c1] if dstate_out is not None else None,
+                                                act, res, want_state, want_params)
+            if want_state:
+                dstate[:, c0:c1] = ds
+            dxs.append(dx)
+            dws.append(dw)
+            dbs.append(db)
+            c0 = c1
+        dweight = torch.cat(dws, dim=0).to(weight.dtype) if want_params else None
+        dbias = torch.cat(dbs, dim=0).to(bias.dtype) if want_params and bias is not None else None
+        return (dstate, dweight, dbias, None, None, None, None, *dxs)
 
 
 def _launch_update_parts(xs, conv_state, weight, bias, token_mask, act, res, rnd):

@@ -96,6 +96,13 @@ def test_prefill_parts_metric_shape(cc):
                                              attention_mask=mask.to(DEV), return_final_states=True)
         assert_parity(torch.cat([o.contiguous() for o in outs], dim=1), want, exact=True, what=f"parts/metric/full/{wt.dtype}")
         assert torch.equal(bits(fs), bits(want_state)), wt.dtype
+    # unmasked with both states and SiLU: the slabs of four steps of the large unmasked launches
+    init = torch.randn(B, C, 3, generator=g).bfloat16()
+    want, want_state = co.conv1d_fwd(x, w, b, activation="silu", residual=1, initial_state=init, final_state_len=5)
+    outs, fs = cc.causal_conv1d_fn_parts(xs, w.to(DEV), b.to(DEV), activation="silu", residual=True,
+                                         initial_states=init.to(DEV), final_states_out=torch.empty(B, C, 5, dtype=torch.bfloat16, device=DEV))
+    assert_parity(torch.cat([o.contiguous() for o in outs], dim=1), want, exact=False, what="parts/metric/states", res=x)
+    assert torch.equal(bits(fs), bits(want_state))
     # views into one projection output are not dense: the launch over a table of parts
     assert cc.kernel_plan_fwd_parts(blc_parts(x, dims, "sliced"), w.to(DEV)) == "blc_vec_parts"
 

@@ -840,6 +840,64 @@ def test_randomised_shapes_layouts_and_options(cc):
     assert set(plans) >= {"bcl_vec", "bcl_vec_short", "blc_vec", "blc_vec_seq", "generic"}, plans
 
 
+def test_randomised_large_channel_contiguous_launches(cc):
+    """Twelve seeded random channel-contiguous calls that move 40-90 MB (the launches with their own slab length,
+    store policy and request order): one tensor or two equal dense parts, channel counts that end inside a tile,
+    lengths that end inside a slab, with and without mask / SiLU / states, each against the oracle."""
+    g = torch.Generator().manual_seed(4040)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    def pick(seq):
+        return seq[ri(0, len(seq) - 1)]
+
+    plans = {}
+    for case in range(12):
+        dtype = pick([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        es = torch.empty(0, dtype=dtype).element_size()
+        pair = case % 2 == 1
+        C = 8 * ri(60, 500)                                   # a multiple of 8, so that two equal parts stay whole lanes
+        B = ri(1, 4)
+        target = ri(42, 90) << 20
+        L = max(40, target // (2 * B * C * es))
+        act = pick([None, "silu"])
+        res = pick([False, "masked", "unmasked"])
+        use_mask, use_state = ri(0, 1), ri(0, 1)
+        wdt = pick([dtype, torch.float32])
+        x = torch.randn(B, C, L, generator=g).to(dtype)
+        w = (torch.randn(C, 4, generator=g) * 0.4).to(wdt)
+        b = (torch.randn(C, generator=g) * 0.2).to(wdt)
+        mask = right_padded_mask([ri(1, L) for _ in range(B)], L, dtype=pick([torch.int64, torch.bool])) if use_mask else None
+        init = torch.randn(B, C, 4, generator=g).to(dtype) if use_state else None
+        want = co.conv1d_fwd(x, w, b, mask=mask, activation=act, residual=res, initial_state=init,
+                             final_state_len=7 if use_state else None)
+        want_out, want_state = want if use_state else (want, None)
+        kw = dict(activation=act, residual=res, attention_mask=None if mask is None else mask.to(DEV),
+                  initial_states=None if init is None else init.to(DEV),
+                  final_states_out=torch.full((B, C, 7), float("nan"), dtype=dtype, device=DEV) if use_state else None)
+        what = f"case {case}: {dtype} w{wdt} {'pair' if pair else 'one'} {B}x{C}x{L} {act} {res} mask{use_mask} state{use_state}"
+        if pair:
+            xs = [t.transpose(1, 2).contiguous().to(DEV).transpose(1, 2) for t in x.split([C // 2, C // 2], dim=1)]
+            plan = cc.kernel_plan_fwd_parts(xs, w.to(DEV), attention_mask=kw["attention_mask"])
+            r = cc.causal_conv1d_fn_parts(xs, w.to(DEV), b.to(DEV), **kw)
+            outs, fs = r if use_state else (r, None)
+            got = torch.cat([o.contiguous() for o in outs], dim=1)
+        else:
+            xg = x.transpose(1, 2).contiguous().to(DEV).transpose(1, 2)
+            plan = cc.kernel_plan_fwd(xg, w.to(DEV))
+            r = cc.causal_conv1d_fn(xg, w.to(DEV), b.to(DEV), **kw)
+            got, fs = r if use_state else (r, None)
+        plans[plan] = plans.get(plan, 0) + 1
+        xm = x if mask is None else (x.float() * mask[:, None, :].float()).to(dtype)
+        added = None if not res else (x if res == "unmasked" else xm)
+        assert_parity(got, want_out, exact=act is None, what=what, res=added)
+        if use_state:
+            assert torch.equal(bits(fs), bits(want_state)), what
+        del x, got, want, want_out
+    assert set(plans) == {"blc_vec", "blc_vec_pair"}, plans
+
+
 def test_randomised_decode_steps(cc):
     """200 seeded random decode calls: dtypes, widths, state lengths, strided states, token masks, residual
     modes, ring-buffer and state-pool addressing, each carried for three steps against the oracle."""

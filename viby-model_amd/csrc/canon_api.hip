@@ -625,7 +625,11 @@ int plan_bwd(const canon_conv1d_bwd_params *p, BwdPlan *plan, bool check_pointer
     const bool states = p->initial_state != nullptr || p->dfinal_state != nullptr;
     const bool rows = !packed && !states && ptrs16 && a.x_sl == 1 && a.g_sl == 1 && a.d_sl == 1 && a.L % E == 0 && a.L / E >= 16 &&
                       a.x_sb % E == 0 && a.x_sc % E == 0 && a.g_sb % E == 0 && a.g_sc % E == 0 &&
-                      a.d_sb % E == 0 && a.d_sc % E == 0;
+                      a.d_sb % E == 0 && a.d_sc % E == 0 &&
+                      // the kernel receives the batch and channel strides of x and dout in vectors, as 32-bit leading scalars
+                      a.x_sb >= 0 && a.x_sc >= 0 && a.g_sb >= 0 && a.g_sc >= 0 &&
+                      (uint64_t)(a.x_sb / E) < (1ull << 32) && (uint64_t)(a.x_sc / E) < (1ull << 32) &&
+                      (uint64_t)(a.g_sb / E) < (1ull << 32) && (uint64_t)(a.g_sc / E) < (1ull << 32);
     if (rows) {
         const uint32_t nvec = a.L / E;
         const uint64_t nrows = (uint64_t)a.B * a.C;

@@ -788,26 +788,33 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
+// The scalars in front of the argument block are what a wave needs to request its rows of x and dout; they arrive in
+// registers with the wave (kernel-argument preload), so the loads are issued without a read of the argument block in
+// front of them, as in the forward kernel.  g_sb / g_sc: the strides of dout when they differ from x's, else a copy
+// of x's; `divC_s`: s1 | s2 << 1 of the division by C.
 template <int DT, int W, int U, bool MASK>
-__global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const BwdArgs a)
+__global__ __launch_bounds__(256) void canon_bwd_bcl_kernel(const char *x_base, const char *g_base, uint32_t x_sb32,
+                                                            uint32_t x_sc32, uint32_t g_sb32, uint32_t g_sc32,
+                                                            uint32_t nthreads, uint32_t nchunk, uint32_t C, uint32_t divC_m,
+                                                            uint32_t divC_s, uint32_t nvec, const BwdArgs a)
 {
     constexpr int E = Elem<DT>::per_vec;
     constexpr int BY = Elem<DT>::bytes;
     const int lane = threadIdx.x & 63;
     const uint32_t task = __builtin_amdgcn_readfirstlane(blockIdx.x * 4u + (threadIdx.x >> 6));
-    if (task >= a.nthreads) return;          // nthreads = wave tasks in this kernel
+    if (task >= nthreads) return;            // nthreads = wave tasks in this kernel
     uint32_t row = task, seg = 0;
-    if (a.nchunk > 1) {                      // nchunk = segments per row
+    if (nchunk > 1) {                        // nchunk = segments per row
         row = fdiv(task, a.div_nchunk);
-        seg = task - row * a.nchunk;
+        seg = task - row * nchunk;
     }
-    const uint32_t b = fdiv(row, a.div_nvec);   // div_nvec divides by C here
-    const uint32_t c = row - b * a.C;
+    const uint32_t b = fdiv(row, FastDiv{C, divC_m, divC_s & 1u, divC_s >> 1});
+    const uint32_t c = row - b * C;
 
-    const char *xrow = a.x + ((int64_t)b * a.x_sb + (int64_t)c * a.x_sc) * BY;
-    const char *grow = a.dy + ((int64_t)b * a.g_sb + (int64_t)c * a.g_sc) * BY;
+    // (strides in vectors of E elements: the planner takes this kernel only for rows that start on 16-byte boundaries)
+    const char *xrow = x_base + ((int64_t)b * x_sb32 + (int64_t)c * x_sc32) * 16;
+    const char *grow = g_base + ((int64_t)b * g_sb32 + (int64_t)c * g_sc32) * 16;
     char *drow = a.dx + ((int64_t)b * a.d_sb + (int64_t)c * a.d_sc) * BY;
-    const uint32_t nvec = a.L / E;
     const uint32_t v0 = seg * (64u * U) + lane;
 
     uint4 X[U], G[U];
@@ -1282,10 +1289,17 @@ template <int DT, int W, bool MASK> void launch_bwd_m(const BwdPlan &pl, hipStre
 {
     const dim3 g(pl.grid), b(256);
     if (pl.kind == BWD_BCL_VEC) {
+        const BwdArgs &A = pl.args;
+        constexpr int64_t EV = Elem<DT>::per_vec;
         switch (pl.U) {
-        case 4: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 4, MASK>), g, b, 0, s, pl.args); break;
-        case 2: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 2, MASK>), g, b, 0, s, pl.args); break;
-        default: hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, 1, MASK>), g, b, 0, s, pl.args); break;
+#define CANON_BWD_BCL_LAUNCH(UU)                                                                                         \
+    hipLaunchKernelGGL((canon_bwd_bcl_kernel<DT, W, UU, MASK>), g, b, 0, s, A.x, A.dy, (uint32_t)(A.x_sb / EV),         \
+                       (uint32_t)(A.x_sc / EV), (uint32_t)(A.g_sb / EV), (uint32_t)(A.g_sc / EV), A.nthreads, A.nchunk,  \
+                       A.C, A.div_nvec.m, A.div_nvec.s1 | A.div_nvec.s2 << 1, A.L / (uint32_t)EV, A)
+        case 4: CANON_BWD_BCL_LAUNCH(4); break;
+        case 2: CANON_BWD_BCL_LAUNCH(2); break;
+        default: CANON_BWD_BCL_LAUNCH(1); break;
+#undef CANON_BWD_BCL_LAUNCH
         }
     } else if (pl.kind == BWD_BLC_VEC)
     {
